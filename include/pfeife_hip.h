@@ -1,0 +1,257 @@
+/*
+ * pfeife_hip.h -- C ABI of libpfeife_hip.so: the gfx950 (MI355X) kernels behind
+ * the pipeline-stage hot path of Pfeife.
+ *
+ * The reference (MerHS/pfeife) is pure Python and has no FFI of its own: every
+ * device operation on its hot path is an ATen eager kernel reached through
+ * `self.mods[node.idx](*inputs)` (pfeife/mp/worker.py:1494), through
+ * `torch.autograd.backward` (pfeife/mp/worker.py:1585-1587), through the
+ * same-rank handoff copies (pfeife/mp/worker.py:1096-1151) and through the
+ * loss modules (pfeife/loss.py:53-70).  Each entry point below names the ATen
+ * call site(s) of the reference that it replaces.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; all pointers are DEVICE pointers owned by
+ *     the caller (PyTorch owns every buffer; nothing here allocates or frees);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *   - every call only enqueues work (no host synchronisation) and returns
+ *     PF_OK (0) or a negative pf_status; pf_last_error() gives the text of the
+ *     last failure on the calling thread;
+ *   - sizes are in ELEMENTS unless a name says bytes; leading dimensions (ld*)
+ *     are row strides in elements;
+ *   - 16-bit operands of the vectorised kernels must be 16-byte aligned and have
+ *     leading dimensions that are multiples of 8 elements (checked, PF_ERR_INVALID).
+ */
+#ifndef PFEIFE_HIP_H_
+#define PFEIFE_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum pf_dtype { PF_F32 = 0, PF_F16 = 1, PF_BF16 = 2, PF_I64 = 3, PF_I32 = 4, PF_U8 = 5 };
+enum pf_status { PF_OK = 0, PF_ERR_INVALID = -1, PF_ERR_UNSUPPORTED = -2, PF_ERR_HIP = -3 };
+enum pf_act { PF_ACT_NONE = 0, PF_ACT_GELU = 1, PF_ACT_GELU_TANH = 2, PF_ACT_SILU = 3, PF_ACT_RELU = 4 };
+
+/* ---- library state ------------------------------------------------------- */
+
+/* ABI version of this header (bumped when a signature changes). */
+int pf_version(void);
+/* Text of the last error raised on the calling host thread ("" if none). */
+const char* pf_last_error(void);
+/* Checks that `device` is a gfx950 part and makes it current for the calling
+ * thread.  Counterpart of torch.cuda.set_device in PfeifeState.__init__
+ * (pfeife/mp/net_states.py:131-132). */
+int pf_init(int device);
+
+/* ---- dense contractions (MFMA) -------------------------------------------
+ * One descriptor covers every matrix product a stage executes:
+ *   C[z] = epilogue( alpha * op(A[z]) . op(B[z]) )        for z in [0, batch1*batch2)
+ * with the reduction over K, op(A) an M x K matrix and op(B) a K x N matrix.
+ *   a_trans = 0 : A is stored M x K (element (m,k) at A[m*lda + k])
+ *   a_trans = 1 : A is stored K x M (element (m,k) at A[k*lda + m])
+ *   b_trans = 0 : B is stored N x K (element (k,n) at B[n*ldb + k])  -- an nn.Linear weight
+ *   b_trans = 1 : B is stored K x N (element (k,n) at B[k*ldb + n])
+ * so that  y = x W^T        is (a_trans 0, b_trans 0)   [F.linear forward]
+ *          dx = dy W        is (a_trans 0, b_trans 1)   [grad wrt input]
+ *          dW = dy^T x      is (a_trans 1, b_trans 1)   [grad wrt weight, beta = 1
+ *                                                        accumulates into param.grad]
+ * Batch z decomposes as z1 = z / batch2, z2 = z % batch2 and each operand moves
+ * by  z1*stride1 + z2*stride2  elements (attention heads inside a packed qkv).
+ *
+ * Epilogue, applied per element v = alpha*acc in this order:
+ *   v += bias[n]                       if bias
+ *   v  = round_to(in_dtype, v)         if round_mid (mirrors autocast's 16-bit result)
+ *   aux_out[m*ld_aux_out+n] = v        if aux_out   (kept for the backward pass; dtype = in_dtype)
+ *   v  = act(v)                        if act != PF_ACT_NONE
+ *   v *= act'(aux_in[m*ld_aux_in+n])   if dact != PF_ACT_NONE (dtype of aux_in = in_dtype)
+ *   v += residual[m*ld_res+n]          if residual
+ *   v += C[m*ldc+n]                    if beta == 1
+ *   C[m*ldc+n] = v  (stored as c_dtype)
+ * bias/aux/residual require batch1*batch2 == 1.
+ *
+ * in_dtype PF_F16/PF_BF16 run on v_mfma_f32_32x32x16 with fp32 accumulation;
+ * in_dtype PF_F32 runs a full-precision fp32 FMA kernel (the fp32 parity path).
+ *
+ * Replaces: aten::linear / aten::addmm / aten::mm / aten::bmm forward and
+ * backward, the autocast casts around them, aten::gelu(+backward), the
+ * residual aten::add and autograd's AccumulateGrad add_ for weight gradients,
+ * as executed by pfeife/mp/worker.py:1494 (forward) and :1585-1587 (backward).
+ */
+typedef struct pf_gemm_desc {
+  int32_t in_dtype;
+  int32_t c_dtype;
+  int32_t a_trans;
+  int32_t b_trans;
+  int64_t M, N, K;
+  const void* A;
+  int64_t lda;
+  const void* B;
+  int64_t ldb;
+  void* C;
+  int64_t ldc;
+  int64_t batch1, batch2;
+  int64_t a_stride1, a_stride2;
+  int64_t b_stride1, b_stride2;
+  int64_t c_stride1, c_stride2;
+  float alpha;
+  int32_t beta;
+  const void* bias;
+  int32_t bias_dtype;
+  int32_t round_mid;
+  void* aux_out;
+  int64_t ld_aux_out;
+  int32_t act;
+  int32_t dact;
+  const void* aux_in;
+  int64_t ld_aux_in;
+  const void* residual;
+  int64_t ld_res;
+  int32_t res_dtype;
+  int32_t reserved;
+} pf_gemm_desc;
+
+int pf_gemm(const pf_gemm_desc* desc, void* stream);
+
+/* ---- normalisation (HBM-bound, one wavefront per row) ---------------------
+ * LayerNorm over the last dimension d of a [rows, d] matrix; gamma/beta are
+ * fp32 [d] (beta may be NULL); mean/rstd are fp32 [rows] saved for backward.
+ * Replaces aten::native_layer_norm / native_layer_norm_backward (stage
+ * forward/backward, pfeife/mp/worker.py:1494, :1585-1587). */
+int pf_layernorm_fwd(const void* x, int x_dtype, const float* gamma, const float* beta, void* y, int y_dtype,
+                     float* mean, float* rstd, int64_t rows, int64_t d, float eps, void* stream);
+/* dx = LN'(dy) (+ dx_add if given: the gradient already accumulated on x from
+ * its other consumer, i.e. the residual branch); dgamma_acc/dbeta_acc (fp32
+ * [d], may be NULL) are ACCUMULATED (+=), which is AccumulateGrad for the
+ * norm's parameters.  workspace: >= pf_colreduce_workspace(rows, d) floats. */
+int pf_layernorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
+                     const float* mean, const float* rstd, const void* dx_add, int add_dtype, void* dx,
+                     int dx_dtype, float* dgamma_acc, float* dbeta_acc, float* workspace, int64_t rows,
+                     int64_t d, void* stream);
+/* RMSNorm: y = x * rsqrt(mean(x^2) + eps) * gamma.  rstd fp32 [rows].
+ * Replaces the pow/mean/rsqrt/mul chain (or aten::rms_norm) of Llama-style blocks. */
+int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, void* y, int y_dtype, float* rstd,
+                   int64_t rows, int64_t d, float eps, void* stream);
+int pf_rmsnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
+                   const float* rstd, const void* dx_add, int add_dtype, void* dx, int dx_dtype,
+                   float* dgamma_acc, float* workspace, int64_t rows, int64_t d, void* stream);
+/* Number of fp32 workspace elements the column reductions below need. */
+int64_t pf_colreduce_workspace(int64_t rows, int64_t cols);
+/* acc[c] += sum_r x[r*ld + c]  (bias gradient; deterministic two-stage reduce).
+ * Replaces the sum-to-size of aten::addmm's bias gradient + AccumulateGrad. */
+int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
+                         float* workspace, void* stream);
+
+/* ---- softmax / attention probabilities ------------------------------------
+ * Row softmax over [rows, cols] fp32 scores (row stride ld_s) producing
+ * probabilities of dtype p_dtype (row stride ld_p; pad columns cols..ld_p-1 are
+ * written as zero so that P can feed pf_gemm with K = cols).  If causal != 0,
+ * row r only sees columns c <= (r % q_len) + (cols - q_len).
+ * Replaces aten::_softmax inside scaled_dot_product_attention / eager attention. */
+int pf_softmax_fwd(const float* s, int64_t ld_s, void* p, int p_dtype, int64_t ld_p, int64_t rows,
+                   int64_t cols, int64_t q_len, int causal, void* stream);
+/* ds = scale * p * (dp - sum_c(dp*p)); dp fp32 (ld_dp), ds dtype ds_dtype (ld_ds, pad zeroed). */
+int pf_softmax_bwd(const float* dp, int64_t ld_dp, const void* p, int p_dtype, int64_t ld_p, void* ds,
+                   int ds_dtype, int64_t ld_ds, int64_t rows, int64_t cols, float scale, void* stream);
+
+/* ---- losses (pfeife/loss.py:53-70 CrossEntropyLoss / HFCrossEntropyLoss; the
+ * mean-reduced nn.CrossEntropyLoss they wrap) -------------------------------
+ * logits [rows, classes] (dtype l_dtype, contiguous), targets int64 [rows];
+ * rows whose target == ignore_index contribute nothing and are left out of the
+ * mean.  row_loss/row_lse: fp32 [rows] scratch kept for backward; loss: fp32 [2]
+ * = { mean loss, number of rows that were not ignored }. */
+int pf_cross_entropy_fwd(const void* logits, int l_dtype, const int64_t* targets, float* row_loss,
+                         float* row_lse, float* loss, int64_t rows, int64_t classes, int64_t ignore_index,
+                         void* stream);
+/* dlogits = (softmax(logits) - onehot(target)) * (*dloss) / (*n_valid), written
+ * as dl_dtype; dloss is a device fp32 scalar (NULL means 1), n_valid is loss+1
+ * of the forward call. */
+int pf_cross_entropy_bwd(const void* logits, int l_dtype, const int64_t* targets, const float* row_lse,
+                         const float* dloss, const float* n_valid, void* dlogits, int dl_dtype, int64_t rows,
+                         int64_t classes, int64_t ignore_index, void* stream);
+/* Mean squared error (F.mse_loss, bench_models/models/train_sdxl.py:1422-1424):
+ * loss[0] = mean((a-b)^2) computed in fp32; partial: fp32 [pf_reduce_workspace(n)]. */
+int64_t pf_reduce_workspace(int64_t n);
+int pf_mse_fwd(const void* a, int a_dtype, const void* b, int b_dtype, float* partial, float* loss, int64_t n,
+               void* stream);
+/* da = 2 (a-b) * (*dloss) / n */
+int pf_mse_bwd(const void* a, int a_dtype, const void* b, int b_dtype, const float* dloss, void* da,
+               int da_dtype, int64_t n, void* stream);
+/* loss[0] = sum(x) in fp32 (SumLoss, pfeife/loss.py:9-13). */
+int pf_sum_fwd(const void* x, int x_dtype, float* partial, float* loss, int64_t n, void* stream);
+
+/* ---- elementwise (HBM-bound, 16-byte vector accesses) ----------------------
+ * Unary activation y = act(x) and its backward dx = dy * act'(x).
+ * Replaces aten::gelu / aten::silu / aten::relu and their backward kernels. */
+int pf_act_fwd(const void* x, void* y, int dtype, int act, int64_t n, void* stream);
+int pf_act_bwd(const void* dy, const void* x, void* dx, int dtype, int act, int64_t n, void* stream);
+/* Gated MLP: y = act(gate) * up ; (dgate, dup) from dy.  SwiGLU is act = SILU,
+ * GEGLU is act = GELU.  Rows of `cols` elements with independent row strides so
+ * that gate/up may be the two halves of one fused projection. */
+int pf_glu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* y, int64_t ld_y,
+               int dtype, int act, int64_t rows, int64_t cols, void* stream);
+int pf_glu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate, const void* up, int64_t ld_up,
+               void* dgate, int64_t ld_dgate, void* dup, int64_t ld_dup, int dtype, int act, int64_t rows,
+               int64_t cols, void* stream);
+/* out = alpha*a + beta*b, each operand with its own dtype (residual add,
+ * fan-out gradient sum `g.add_(lg)` of pfeife/mp/worker.py:1543). n elements. */
+int pf_axpby(const void* a, int a_dtype, float alpha, const void* b, int b_dtype, float beta, void* out,
+             int out_dtype, int64_t n, void* stream);
+/* y[r, c] = x[r, c] + bias[c % bias_len] (broadcast add of a bias / positional
+ * embedding over the leading dimension). */
+int pf_bias_add(const void* x, int x_dtype, const void* bias, int bias_dtype, void* y, int y_dtype, int64_t n,
+                int64_t bias_len, void* stream);
+/* dtype conversion / copy of n contiguous elements (autocast's weight casts,
+ * done once per optimiser step instead of once per micro-batch). */
+int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream);
+/* dst[i] = value for n elements of a 4-byte or 2-byte float dtype
+ * (optimizer.zero_grad(set_to_none=False), pfeife/mp/worker.py:583-597). */
+int pf_fill(void* dst, int dtype, float value, int64_t n, void* stream);
+/* Generic strided copy with dtype conversion of a tensor of up to 6 dims:
+ * dst[idx . dst_strides] = src[idx . src_strides]  (strides in elements). Used
+ * for layout changes that are not views: patch extraction, head merges, cat. */
+int pf_copy_strided(const void* src, int src_dtype, const int64_t* src_strides, void* dst, int dst_dtype,
+                    const int64_t* dst_strides, const int64_t* sizes, int ndim, int accumulate, void* stream);
+/* Rotary position embedding (rotate-half convention of HF Llama: element i
+ * pairs with i + D/2): x and y are [B, T, H, D] tensors addressed with element
+ * strides (sb, st, sh, 1); cos_t/sin_t are fp32 [T, D/2].
+ *   y[i]       = x[i] cos[t,i] - x[i+D/2] sin[t,i]
+ *   y[i+D/2]   = x[i+D/2] cos[t,i] + x[i] sin[t,i]
+ * inverse != 0 applies the transposed rotation (the backward pass). y may alias x. */
+int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t B, int64_t T,
+            int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh, int64_t y_sb, int64_t y_st,
+            int64_t y_sh, int inverse, void* stream);
+
+/* ---- gradient accumulation --------------------------------------------------
+ * acc[i] += g[i] for i < n, acc fp32, g of dtype g_dtype: autograd's
+ * AccumulateGrad `param.grad.add_(new_grad)` executed once per parameter per
+ * micro-batch by torch.autograd.backward (pfeife/mp/worker.py:1585-1587).
+ * Algorithmic traffic: 12 bytes per element for fp32 g. */
+int pf_grad_accumulate_f32(float* acc, const void* g, int g_dtype, int64_t n, void* stream);
+
+/* ---- micro-batch split / merge ----------------------------------------------
+ * Row gather:  dst[i, :] = src[index ? index[i] : row_start + i, :]  for i < n_rows,
+ * rows of row_bytes bytes (any dtype; 16-byte fast path when aligned).
+ * With index == NULL this materialises chunk `row_start .. row_start+n_rows` of
+ * torch.tensor_split(v, batch_cnt, 0) (pfeife/batch.py:45) as a contiguous slab. */
+int pf_split_gather(const void* src, void* dst, int64_t row_bytes, int64_t row_start, int64_t n_rows,
+                    const int64_t* index, void* stream);
+/* Row scatter: dst[index ? index[i] : row_start + i, :] = src[i, :]; stacks the
+ * per-micro-batch results back into one batch-major tensor (the inverse of the
+ * split; the reference returns a Python list, pfeife/mp/partial/module.py:99-102). */
+int pf_merge_scatter(const void* src, void* dst, int64_t row_bytes, int64_t row_start, int64_t n_rows,
+                     const int64_t* index, void* stream);
+/* Embedding lookup out[i, :] = table[ids[i], :] with dtype conversion, and its
+ * backward dtable[ids[i], :] += dout[i, :] (fp32 accumulate, atomics-free:
+ * one wavefront owns a table row).  Replaces aten::embedding(+dense backward). */
+int pf_embedding_fwd(const void* table, int t_dtype, const int64_t* ids, void* out, int o_dtype, int64_t n_ids,
+                     int64_t dim, int64_t vocab, void* stream);
+int pf_embedding_bwd(const void* dout, int d_dtype, const int64_t* ids, float* dtable_acc, int64_t n_ids,
+                     int64_t dim, int64_t vocab, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PFEIFE_HIP_H_ */

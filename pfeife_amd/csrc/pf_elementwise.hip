@@ -1,0 +1,353 @@
+// HBM-bound streaming kernels: activations, gated MLP, axpby, bias add, casts,
+// fills, strided copies, rotary embedding and the fp32 gradient accumulation.
+// All of them move 16 bytes (8 x 16-bit) or 32 bytes (8 x fp32) per lane per
+// step in a grid-stride loop sized to keep every CU busy.
+#include "pf_common.h"
+
+namespace {
+
+constexpr int EW_BLOCK = 256;
+constexpr int EW_MAX_BLOCKS = 256 * 16;  // 16 workgroups per CU is plenty of bytes in flight
+
+inline dim3 ew_grid(int64_t work_items) {
+  int64_t b = (work_items + EW_BLOCK - 1) / EW_BLOCK;
+  if (b < 1) b = 1;
+  if (b > EW_MAX_BLOCKS) b = EW_MAX_BLOCKS;
+  return dim3((unsigned)b);
+}
+
+// F provides:  void run<W>(int64_t i)  processing W elements starting at i
+template <class F>
+__global__ __launch_bounds__(EW_BLOCK) void ew_kernel(F f, int64_t n, int vec) {
+  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  const int64_t nv = vec ? n / 8 : 0;
+  for (int64_t i = gtid; i < nv; i += gsz) f.template run<8>(i * 8);
+  for (int64_t i = nv * 8 + gtid; i < n; i += gsz) f.template run<1>(i);
+}
+
+template <class F>
+int ew_launch(const F& f, int64_t n, bool vec, hipStream_t st, const char* name) {
+  if (n <= 0) return PF_OK;
+  hipLaunchKernelGGL(ew_kernel<F>, ew_grid(vec ? (n + 7) / 8 : n), dim3(EW_BLOCK), 0, st, f, n, vec ? 1 : 0);
+  PF_CHECK_LAUNCH(name);
+  return PF_OK;
+}
+
+inline bool al16(const void* p) { return pf_aligned(p, 16); }
+
+struct ActFwd {
+  const void* x; void* y; int dt, act;
+  template <int W> __device__ void run(int64_t i) const {
+    float v[W];
+    ld_vec<W>(x, i, dt, v);
+#pragma unroll
+    for (int k = 0; k < W; ++k) v[k] = pf_act(act, v[k]);
+    st_vec<W>(y, i, dt, v);
+  }
+};
+struct ActBwd {
+  const void* dy; const void* x; void* dx; int dt, act;
+  template <int W> __device__ void run(int64_t i) const {
+    float g[W], v[W];
+    ld_vec<W>(dy, i, dt, g);
+    ld_vec<W>(x, i, dt, v);
+#pragma unroll
+    for (int k = 0; k < W; ++k) g[k] *= pf_act_grad(act, v[k]);
+    st_vec<W>(dx, i, dt, g);
+  }
+};
+struct Axpby {
+  const void* a; const void* b; void* o; int adt, bdt, odt; float alpha, beta;
+  template <int W> __device__ void run(int64_t i) const {
+    float x[W], y[W];
+    ld_vec<W>(a, i, adt, x);
+    ld_vec<W>(b, i, bdt, y);
+#pragma unroll
+    for (int k = 0; k < W; ++k) x[k] = alpha * x[k] + beta * y[k];
+    st_vec<W>(o, i, odt, x);
+  }
+};
+struct Scale {  // out = alpha * a (b absent)
+  const void* a; void* o; int adt, odt; float alpha;
+  template <int W> __device__ void run(int64_t i) const {
+    float x[W];
+    ld_vec<W>(a, i, adt, x);
+#pragma unroll
+    for (int k = 0; k < W; ++k) x[k] *= alpha;
+    st_vec<W>(o, i, odt, x);
+  }
+};
+struct Cast {
+  const void* s; void* d; int sdt, ddt;
+  template <int W> __device__ void run(int64_t i) const {
+    float x[W];
+    ld_vec<W>(s, i, sdt, x);
+    st_vec<W>(d, i, ddt, x);
+  }
+};
+struct Fill {
+  void* d; int dt; float value;
+  template <int W> __device__ void run(int64_t i) const {
+    float x[W];
+#pragma unroll
+    for (int k = 0; k < W; ++k) x[k] = value;
+    st_vec<W>(d, i, dt, x);
+  }
+};
+struct GradAcc {
+  float* acc; const void* g; int gdt;
+  template <int W> __device__ void run(int64_t i) const {
+    float a[W], x[W];
+    ld_vec<W>(acc, i, PF_F32, a);
+    ld_vec<W>(g, i, gdt, x);
+#pragma unroll
+    for (int k = 0; k < W; ++k) a[k] += x[k];
+    st_vec<W>(acc, i, PF_F32, a);
+  }
+};
+struct BiasAdd {  // bias_len is a multiple of 8 on the vector path
+  const void* x; const void* bias; void* y; int xdt, bdt, ydt; int64_t bias_len;
+  template <int W> __device__ void run(int64_t i) const {
+    float v[W], b[W];
+    ld_vec<W>(x, i, xdt, v);
+    ld_vec<W>(bias, i % bias_len, bdt, b);
+#pragma unroll
+    for (int k = 0; k < W; ++k) v[k] += b[k];
+    st_vec<W>(y, i, ydt, v);
+  }
+};
+
+// gated MLP: rows x cols with independent row strides; index space is rows*cols
+struct GluFwd {
+  const void* gate; const void* up; void* y; int64_t ldg, ldu, ldy, cols; int dt, act;
+  template <int W> __device__ void run(int64_t i) const {
+    const int64_t r = i / cols, c = i % cols;
+    float g[W], u[W];
+    ld_vec<W>(gate, r * ldg + c, dt, g);
+    ld_vec<W>(up, r * ldu + c, dt, u);
+#pragma unroll
+    for (int k = 0; k < W; ++k) g[k] = pf_round_to(dt, pf_act(act, g[k])) * u[k];
+    st_vec<W>(y, r * ldy + c, dt, g);
+  }
+};
+struct GluBwd {
+  const void* dy; const void* gate; const void* up; void* dgate; void* dup;
+  int64_t lddy, ldg, ldu, lddg, lddu, cols; int dt, act;
+  template <int W> __device__ void run(int64_t i) const {
+    const int64_t r = i / cols, c = i % cols;
+    float d[W], g[W], u[W], dg[W], du[W];
+    ld_vec<W>(dy, r * lddy + c, dt, d);
+    ld_vec<W>(gate, r * ldg + c, dt, g);
+    ld_vec<W>(up, r * ldu + c, dt, u);
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      du[k] = d[k] * pf_round_to(dt, pf_act(act, g[k]));
+      dg[k] = d[k] * u[k] * pf_act_grad(act, g[k]);
+    }
+    st_vec<W>(dgate, r * lddg + c, dt, dg);
+    st_vec<W>(dup, r * lddu + c, dt, du);
+  }
+};
+
+// ---- strided copy (<= 6 dims) ----------------------------------------------
+struct CopyDesc {
+  int64_t size[6], ss[6], ds[6];  // innermost dimension last; size of the innermost already divided by W
+  int ndim;
+};
+template <int W>
+__global__ __launch_bounds__(EW_BLOCK) void copy_strided_kernel(const void* src, int sdt, void* dst, int ddt,
+                                                                CopyDesc cd, int64_t total, int accumulate) {
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gsz) {
+    int64_t rem = i, so = 0, dof = 0;
+#pragma unroll
+    for (int k = 5; k >= 0; --k) {
+      if (k < cd.ndim) {
+        const int64_t idx = rem % cd.size[k];
+        rem /= cd.size[k];
+        const int64_t mul = (k == cd.ndim - 1) ? W : 1;
+        so += idx * cd.ss[k] * mul;
+        dof += idx * cd.ds[k] * mul;
+      }
+    }
+    float v[W];
+    ld_vec<W>(src, so, sdt, v);
+    if (accumulate) {
+      float o[W];
+      ld_vec<W>(dst, dof, ddt, o);
+#pragma unroll
+      for (int k = 0; k < W; ++k) v[k] += o[k];
+    }
+    st_vec<W>(dst, dof, ddt, v);
+  }
+}
+
+// ---- rotary embedding --------------------------------------------------------
+// one thread per (b, t, h, i) pair index i < D/2
+__global__ __launch_bounds__(EW_BLOCK) void rope_kernel(const void* x, void* y, int dt, const float* cos_t,
+                                                        const float* sin_t, int64_t B, int64_t T, int64_t H,
+                                                        int64_t D, int64_t xsb, int64_t xst, int64_t xsh, int64_t ysb,
+                                                        int64_t yst, int64_t ysh, int inverse) {
+  const int64_t half = D / 2;
+  const int64_t total = B * T * H * half;
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gsz) {
+    const int64_t i = idx % half;
+    int64_t r = idx / half;
+    const int64_t h = r % H;
+    r /= H;
+    const int64_t t = r % T, b = r / T;
+    const int64_t xo = b * xsb + t * xst + h * xsh, yo = b * ysb + t * yst + h * ysh;
+    const float x1 = pf_load_as_f32(x, xo + i, dt), x2 = pf_load_as_f32(x, xo + i + half, dt);
+    const float c = cos_t[t * half + i];
+    const float s = inverse ? -sin_t[t * half + i] : sin_t[t * half + i];
+    pf_store_from_f32(y, yo + i, dt, x1 * c - x2 * s);
+    pf_store_from_f32(y, yo + i + half, dt, x2 * c + x1 * s);
+  }
+}
+
+}  // namespace
+
+extern "C" int pf_act_fwd(const void* x, void* y, int dtype, int act, int64_t n, void* stream) {
+  PF_REQUIRE(n >= 0 && pf_is_float_dtype(dtype), "pf_act_fwd: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(x && y, "pf_act_fwd: null pointer");
+  ActFwd f{x, y, dtype, act};
+  return ew_launch(f, n, al16(x) && al16(y), (hipStream_t)stream, "pf_act_fwd");
+}
+
+extern "C" int pf_act_bwd(const void* dy, const void* x, void* dx, int dtype, int act, int64_t n, void* stream) {
+  PF_REQUIRE(n >= 0 && pf_is_float_dtype(dtype), "pf_act_bwd: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(dy && x && dx, "pf_act_bwd: null pointer");
+  ActBwd f{dy, x, dx, dtype, act};
+  return ew_launch(f, n, al16(dy) && al16(x) && al16(dx), (hipStream_t)stream, "pf_act_bwd");
+}
+
+extern "C" int pf_glu_fwd(const void* gate, int64_t ld_gate, const void* up, int64_t ld_up, void* y, int64_t ld_y,
+                          int dtype, int act, int64_t rows, int64_t cols, void* stream) {
+  PF_REQUIRE(rows >= 0 && cols >= 0 && pf_is_float_dtype(dtype), "pf_glu_fwd: bad arguments");
+  if (rows == 0 || cols == 0) return PF_OK;
+  PF_REQUIRE(gate && up && y, "pf_glu_fwd: null pointer");
+  PF_REQUIRE(ld_gate >= cols && ld_up >= cols && ld_y >= cols, "pf_glu_fwd: leading dimension too small");
+  const bool vec = al16(gate) && al16(up) && al16(y) && cols % 8 == 0 && ld_gate % 8 == 0 && ld_up % 8 == 0 &&
+                   ld_y % 8 == 0;
+  GluFwd f{gate, up, y, ld_gate, ld_up, ld_y, cols, dtype, act};
+  return ew_launch(f, rows * cols, vec, (hipStream_t)stream, "pf_glu_fwd");
+}
+
+extern "C" int pf_glu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate, const void* up,
+                          int64_t ld_up, void* dgate, int64_t ld_dgate, void* dup, int64_t ld_dup, int dtype, int act,
+                          int64_t rows, int64_t cols, void* stream) {
+  PF_REQUIRE(rows >= 0 && cols >= 0 && pf_is_float_dtype(dtype), "pf_glu_bwd: bad arguments");
+  if (rows == 0 || cols == 0) return PF_OK;
+  PF_REQUIRE(dy && gate && up && dgate && dup, "pf_glu_bwd: null pointer");
+  PF_REQUIRE(ld_dy >= cols && ld_gate >= cols && ld_up >= cols && ld_dgate >= cols && ld_dup >= cols,
+             "pf_glu_bwd: leading dimension too small");
+  const bool vec = al16(dy) && al16(gate) && al16(up) && al16(dgate) && al16(dup) && cols % 8 == 0 &&
+                   ld_dy % 8 == 0 && ld_gate % 8 == 0 && ld_up % 8 == 0 && ld_dgate % 8 == 0 && ld_dup % 8 == 0;
+  GluBwd f{dy, gate, up, dgate, dup, ld_dy, ld_gate, ld_up, ld_dgate, ld_dup, cols, dtype, act};
+  return ew_launch(f, rows * cols, vec, (hipStream_t)stream, "pf_glu_bwd");
+}
+
+extern "C" int pf_axpby(const void* a, int a_dtype, float alpha, const void* b, int b_dtype, float beta, void* out,
+                        int out_dtype, int64_t n, void* stream) {
+  PF_REQUIRE(n >= 0 && pf_is_float_dtype(a_dtype) && pf_is_float_dtype(out_dtype), "pf_axpby: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(a && out, "pf_axpby: null pointer");
+  if (!b) {
+    Scale f{a, out, a_dtype, out_dtype, alpha};
+    return ew_launch(f, n, al16(a) && al16(out), (hipStream_t)stream, "pf_axpby");
+  }
+  PF_REQUIRE(pf_is_float_dtype(b_dtype), "pf_axpby: bad b dtype");
+  Axpby f{a, b, out, a_dtype, b_dtype, out_dtype, alpha, beta};
+  return ew_launch(f, n, al16(a) && al16(b) && al16(out), (hipStream_t)stream, "pf_axpby");
+}
+
+extern "C" int pf_bias_add(const void* x, int x_dtype, const void* bias, int bias_dtype, void* y, int y_dtype,
+                           int64_t n, int64_t bias_len, void* stream) {
+  PF_REQUIRE(n >= 0 && bias_len > 0 && pf_is_float_dtype(x_dtype) && pf_is_float_dtype(bias_dtype) &&
+                 pf_is_float_dtype(y_dtype),
+             "pf_bias_add: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(x && bias && y, "pf_bias_add: null pointer");
+  PF_REQUIRE(n % bias_len == 0, "pf_bias_add: n must be a multiple of bias_len");
+  BiasAdd f{x, bias, y, x_dtype, bias_dtype, y_dtype, bias_len};
+  return ew_launch(f, n, al16(x) && al16(bias) && al16(y) && bias_len % 8 == 0, (hipStream_t)stream, "pf_bias_add");
+}
+
+extern "C" int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream) {
+  PF_REQUIRE(n >= 0 && pf_is_float_dtype(src_dtype) && pf_is_float_dtype(dst_dtype), "pf_cast: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(src && dst, "pf_cast: null pointer");
+  Cast f{src, dst, src_dtype, dst_dtype};
+  return ew_launch(f, n, al16(src) && al16(dst), (hipStream_t)stream, "pf_cast");
+}
+
+extern "C" int pf_fill(void* dst, int dtype, float value, int64_t n, void* stream) {
+  PF_REQUIRE(n >= 0 && pf_is_float_dtype(dtype), "pf_fill: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(dst, "pf_fill: null pointer");
+  Fill f{dst, dtype, value};
+  return ew_launch(f, n, al16(dst), (hipStream_t)stream, "pf_fill");
+}
+
+extern "C" int pf_grad_accumulate_f32(float* acc, const void* g, int g_dtype, int64_t n, void* stream) {
+  PF_REQUIRE(n >= 0 && pf_is_float_dtype(g_dtype), "pf_grad_accumulate_f32: bad arguments");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(acc && g, "pf_grad_accumulate_f32: null pointer");
+  GradAcc f{acc, g, g_dtype};
+  return ew_launch(f, n, al16(acc) && al16(g), (hipStream_t)stream, "pf_grad_accumulate_f32");
+}
+
+extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* src_strides, void* dst, int dst_dtype,
+                               const int64_t* dst_strides, const int64_t* sizes, int ndim, int accumulate,
+                               void* stream) {
+  PF_REQUIRE(ndim >= 1 && ndim <= 6, "pf_copy_strided: ndim %d outside 1..6", ndim);
+  PF_REQUIRE(src_strides && dst_strides && sizes, "pf_copy_strided: null shape");
+  PF_REQUIRE(pf_is_float_dtype(src_dtype) && pf_is_float_dtype(dst_dtype), "pf_copy_strided: bad dtype");
+  CopyDesc cd;
+  cd.ndim = ndim;
+  int64_t total = 1;
+  bool vec = pf_aligned(src, 16) && pf_aligned(dst, 16);
+  for (int k = 0; k < 6; ++k) {
+    cd.size[k] = k < ndim ? sizes[k] : 1;
+    cd.ss[k] = k < ndim ? src_strides[k] : 0;
+    cd.ds[k] = k < ndim ? dst_strides[k] : 0;
+    if (k < ndim) {
+      PF_REQUIRE(sizes[k] >= 0, "pf_copy_strided: negative size");
+      PF_REQUIRE(dst_strides[k] >= 0 && src_strides[k] >= 0, "pf_copy_strided: negative stride");
+      total *= sizes[k];
+      if (k < ndim - 1) vec = vec && src_strides[k] % 8 == 0 && dst_strides[k] % 8 == 0;
+    }
+  }
+  if (total == 0) return PF_OK;
+  PF_REQUIRE(src && dst, "pf_copy_strided: null pointer");
+  vec = vec && src_strides[ndim - 1] == 1 && dst_strides[ndim - 1] == 1 && sizes[ndim - 1] % 8 == 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (vec) {
+    cd.size[ndim - 1] /= 8;
+    total /= 8;
+    hipLaunchKernelGGL(copy_strided_kernel<8>, ew_grid(total), dim3(EW_BLOCK), 0, st, src, src_dtype, dst, dst_dtype,
+                       cd, total, accumulate);
+  } else {
+    hipLaunchKernelGGL(copy_strided_kernel<1>, ew_grid(total), dim3(EW_BLOCK), 0, st, src, src_dtype, dst, dst_dtype,
+                       cd, total, accumulate);
+  }
+  PF_CHECK_LAUNCH("pf_copy_strided");
+  return PF_OK;
+}
+
+extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t B,
+                       int64_t T, int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh, int64_t y_sb,
+                       int64_t y_st, int64_t y_sh, int inverse, void* stream) {
+  PF_REQUIRE(B >= 0 && T >= 0 && H >= 0 && D >= 0 && D % 2 == 0 && pf_is_float_dtype(dtype), "pf_rope: bad arguments");
+  const int64_t total = B * T * H * (D / 2);
+  if (total == 0) return PF_OK;
+  PF_REQUIRE(x && y && cos_t && sin_t, "pf_rope: null pointer");
+  hipLaunchKernelGGL(rope_kernel, ew_grid(total), dim3(EW_BLOCK), 0, (hipStream_t)stream, x, y, dtype, cos_t, sin_t, B,
+                     T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
+  PF_CHECK_LAUNCH("pf_rope");
+  return PF_OK;
+}

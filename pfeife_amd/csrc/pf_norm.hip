@@ -1,0 +1,325 @@
+// LayerNorm / RMSNorm forward+backward and column reductions (HBM-bound).
+//
+// One 64-lane wavefront owns one row; row statistics are butterfly reductions
+// inside the wavefront (no LDS, no atomics).  A row is re-read from L2 for the
+// second/third pass, so HBM sees it once.  Parameter gradients (dgamma, dbeta,
+// bias gradients) are reduced deterministically in two stages: per-workgroup
+// column partials in a caller-supplied workspace, then one thread per column.
+#include "pf_common.h"
+
+namespace {
+
+constexpr int COLRED_MAX_BLOCKS = 512;
+
+// ---- forward ---------------------------------------------------------------
+template <int W>
+__global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, const float* gamma, const float* beta,
+                                                       void* y, int y_dt, float* mean, float* rstd, int64_t rows,
+                                                       int64_t d, float eps, int rms) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  const int64_t base = row * d;
+  float mu = 0.f;
+  if (!rms) {
+    float s = 0.f;
+    for (int64_t c = (int64_t)lane * W; c < d; c += 64 * W) {
+      float v[W];
+      ld_vec<W>(x, base + c, x_dt, v);
+#pragma unroll
+      for (int k = 0; k < W; ++k) s += v[k];
+    }
+    mu = pf_wave_sum(s) / (float)d;
+  }
+  float q = 0.f;
+  for (int64_t c = (int64_t)lane * W; c < d; c += 64 * W) {
+    float v[W];
+    ld_vec<W>(x, base + c, x_dt, v);
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      const float t = v[k] - mu;
+      q += t * t;
+    }
+  }
+  const float var = pf_wave_sum(q) / (float)d;
+  const float rs = 1.0f / sqrtf(var + eps);
+  for (int64_t c = (int64_t)lane * W; c < d; c += 64 * W) {
+    float v[W], g[W], o[W];
+    ld_vec<W>(x, base + c, x_dt, v);
+    ld_vec<W>(gamma, c, PF_F32, g);
+    if (beta) {
+      float b[W];
+      ld_vec<W>(beta, c, PF_F32, b);
+#pragma unroll
+      for (int k = 0; k < W; ++k) o[k] = (v[k] - mu) * rs * g[k] + b[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < W; ++k) o[k] = (v[k] - mu) * rs * g[k];
+    }
+    st_vec<W>(y, base + c, y_dt, o);
+  }
+  if (lane == 0) {
+    if (mean) mean[row] = mu;
+    rstd[row] = rs;
+  }
+}
+
+// ---- backward ----------------------------------------------------------------
+// NV = column groups a lane owns (d <= 64 * W * NV).  Column partials for
+// dgamma/dbeta stay in registers across the rows a wavefront processes.
+template <int W, int NV>
+__global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt, const void* x, int x_dt,
+                                                       const float* gamma, const float* mean, const float* rstd,
+                                                       const void* dx_add, int add_dt, void* dx, int dx_dt,
+                                                       float* ws, int64_t rows, int64_t d, int rms, int want_wgrad) {
+  __shared__ float red[4][64 * W];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float pg[NV][W], pb[NV][W];
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+#pragma unroll
+    for (int k = 0; k < W; ++k) pg[i][k] = pb[i][k] = 0.f;
+
+  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < rows; row += (int64_t)gridDim.x * 4) {
+    const int64_t base = row * d;
+    const float mu = rms ? 0.f : mean[row];
+    const float rs = rstd[row];
+    float c1 = 0.f, c2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int64_t c = ((int64_t)lane + i * 64) * W;
+      if (c < d) {
+        float vdy[W], vx[W], g[W];
+        ld_vec<W>(dy, base + c, dy_dt, vdy);
+        ld_vec<W>(x, base + c, x_dt, vx);
+        ld_vec<W>(gamma, c, PF_F32, g);
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          const float gg = vdy[k] * g[k];
+          const float xh = (vx[k] - mu) * rs;
+          c1 += gg;
+          c2 += gg * xh;
+        }
+      }
+    }
+    c1 = rms ? 0.f : pf_wave_sum(c1) / (float)d;
+    c2 = pf_wave_sum(c2) / (float)d;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int64_t c = ((int64_t)lane + i * 64) * W;
+      if (c < d) {
+        float vdy[W], vx[W], g[W], o[W];
+        ld_vec<W>(dy, base + c, dy_dt, vdy);
+        ld_vec<W>(x, base + c, x_dt, vx);
+        ld_vec<W>(gamma, c, PF_F32, g);
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          const float gg = vdy[k] * g[k];
+          const float xh = (vx[k] - mu) * rs;
+          o[k] = rs * (gg - c1 - xh * c2);
+          pg[i][k] += vdy[k] * xh;
+          pb[i][k] += vdy[k];
+        }
+        if (dx_add) {
+          float a[W];
+          ld_vec<W>(dx_add, base + c, add_dt, a);
+#pragma unroll
+          for (int k = 0; k < W; ++k) o[k] += a[k];
+        }
+        st_vec<W>(dx, base + c, dx_dt, o);
+      }
+    }
+  }
+  if (!want_wgrad) return;  // uniform over the block
+  // reduce the 4 wavefronts through LDS, then one partial row per block:
+  // ws layout [gridDim.x][2][d]
+  float* wrow = ws + (int64_t)blockIdx.x * 2 * d;
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      __syncthreads();
+#pragma unroll
+      for (int k = 0; k < W; ++k) red[wave][lane * W + k] = which ? pb[i][k] : pg[i][k];
+      __syncthreads();
+      if (wave == 0) {
+        const int64_t c = ((int64_t)lane + i * 64) * W;
+        if (c < d) {
+#pragma unroll
+          for (int k = 0; k < W; ++k) {
+            const float s = red[0][lane * W + k] + red[1][lane * W + k] + red[2][lane * W + k] + red[3][lane * W + k];
+            wrow[which * d + c + k] = s;
+          }
+        }
+      }
+    }
+  }
+}
+
+// acc[c] += sum_p ws[p*stride + c]
+__global__ void colreduce_finalize_kernel(const float* ws, int n_partials, int64_t stride, int64_t cols, float* acc) {
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  float s = 0.f;
+  for (int p = 0; p < n_partials; ++p) s += ws[(int64_t)p * stride + c];
+  acc[c] += s;
+}
+
+// column sums of x[rows, cols]: block = 4 wavefronts sharing one 64*W column
+// strip, wavefront w takes rows w, w+4, ... of its row chunk.
+template <int W>
+__global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t ld,
+                                                     float* ws, int64_t rows_per_chunk) {
+  __shared__ float red[4][64 * W];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t c = ((int64_t)blockIdx.x * 64 + lane) * W;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
+  const int64_t r1 = r0 + rows_per_chunk < rows ? r0 + rows_per_chunk : rows;
+  float s[W];
+#pragma unroll
+  for (int k = 0; k < W; ++k) s[k] = 0.f;
+  if (c < cols) {
+    for (int64_t r = r0 + wave; r < r1; r += 4) {
+      float v[W];
+      ld_vec<W>(x, r * ld + c, x_dt, v);
+#pragma unroll
+      for (int k = 0; k < W; ++k) s[k] += v[k];
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < W; ++k) red[wave][lane * W + k] = s[k];
+  __syncthreads();
+  if (wave == 0 && c < cols) {
+#pragma unroll
+    for (int k = 0; k < W; ++k)
+      ws[(int64_t)blockIdx.y * cols + c + k] =
+          red[0][lane * W + k] + red[1][lane * W + k] + red[2][lane * W + k] + red[3][lane * W + k];
+  }
+}
+
+inline int norm_bwd_blocks(int64_t rows) {
+  int64_t b = (rows + 3) / 4;
+  if (b < 1) b = 1;
+  if (b > COLRED_MAX_BLOCKS) b = COLRED_MAX_BLOCKS;
+  return (int)b;
+}
+
+bool vec_ok(const void* p, int dt, int64_t ld) {
+  if (!p) return true;
+  return pf_aligned(p, 16) && (ld % 8 == 0) && pf_is_float_dtype(dt);
+}
+
+int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, void* y, int y_dt, float* mean,
+             float* rstd, int64_t rows, int64_t d, float eps, int rms, hipStream_t st, const char* name) {
+  PF_REQUIRE(rows >= 0 && d > 0, "%s: bad shape rows=%lld d=%lld", name, (long long)rows, (long long)d);
+  if (rows == 0) return PF_OK;
+  PF_REQUIRE(x && gamma && y && rstd, "%s: null pointer", name);
+  PF_REQUIRE(pf_is_float_dtype(x_dt) && pf_is_float_dtype(y_dt), "%s: bad dtype", name);
+  PF_REQUIRE((rows + 3) / 4 < (1ll << 31), "%s: too many rows", name);
+  const dim3 grid((unsigned)((rows + 3) / 4));
+  const bool v = vec_ok(x, x_dt, d) && vec_ok(y, y_dt, d) && vec_ok(gamma, PF_F32, d) && vec_ok(beta, PF_F32, d);
+  if (v) hipLaunchKernelGGL(norm_fwd_kernel<8>, grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms);
+  else hipLaunchKernelGGL(norm_fwd_kernel<1>, grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms);
+  PF_CHECK_LAUNCH(name);
+  return PF_OK;
+}
+
+int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* gamma, const float* mean,
+             const float* rstd, const void* dx_add, int add_dt, void* dx, int dx_dt, float* dgamma, float* dbeta,
+             float* ws, int64_t rows, int64_t d, int rms, hipStream_t st, const char* name) {
+  PF_REQUIRE(rows >= 0 && d > 0, "%s: bad shape", name);
+  if (rows == 0) return PF_OK;
+  PF_REQUIRE(dy && x && gamma && rstd && dx, "%s: null pointer", name);
+  PF_REQUIRE(rms || mean, "%s: mean required", name);
+  PF_REQUIRE(pf_is_float_dtype(dy_dt) && pf_is_float_dtype(x_dt) && pf_is_float_dtype(dx_dt), "%s: bad dtype", name);
+  const int want = (dgamma || dbeta) ? 1 : 0;
+  if (want) PF_REQUIRE(ws, "%s: workspace required for parameter gradients", name);
+  const int blocks = norm_bwd_blocks(rows);
+  const bool v = vec_ok(dy, dy_dt, d) && vec_ok(x, x_dt, d) && vec_ok(dx, dx_dt, d) && vec_ok(gamma, PF_F32, d) &&
+                 vec_ok(dx_add, dx_add ? add_dt : PF_F32, d);
+#define PF_NB(W, NV)                                                                                          \
+  hipLaunchKernelGGL((norm_bwd_kernel<W, NV>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, mean, \
+                     rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want)
+  if (v) {
+    if (d <= 64 * 8 * 2) PF_NB(8, 2);
+    else if (d <= 64 * 8 * 4) PF_NB(8, 4);
+    else if (d <= 64 * 8 * 8) PF_NB(8, 8);
+    else if (d <= 64 * 8 * 16) PF_NB(8, 16);
+    else { pf_set_error("%s: d=%lld exceeds 8192", name, (long long)d); return PF_ERR_UNSUPPORTED; }
+  } else {
+    if (d <= 64 * 16) PF_NB(1, 16);
+    else if (d <= 64 * 64) PF_NB(1, 64);
+    else { pf_set_error("%s: unaligned d=%lld exceeds 4096", name, (long long)d); return PF_ERR_UNSUPPORTED; }
+  }
+#undef PF_NB
+  PF_CHECK_LAUNCH(name);
+  if (want) {
+    const dim3 fg((unsigned)((d + 255) / 256));
+    if (dgamma) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws, blocks, 2 * d, d, dgamma);
+    if (dbeta) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws + d, blocks, 2 * d, d, dbeta);
+    PF_CHECK_LAUNCH(name);
+  }
+  return PF_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t pf_colreduce_workspace(int64_t rows, int64_t cols) {
+  (void)rows;
+  return 2 * (int64_t)COLRED_MAX_BLOCKS * (cols > 0 ? cols : 1);
+}
+
+extern "C" int pf_layernorm_fwd(const void* x, int x_dtype, const float* gamma, const float* beta, void* y,
+                                int y_dtype, float* mean, float* rstd, int64_t rows, int64_t d, float eps,
+                                void* stream) {
+  PF_REQUIRE(mean != nullptr || rows == 0, "pf_layernorm_fwd: mean required");
+  return norm_fwd(x, x_dtype, gamma, beta, y, y_dtype, mean, rstd, rows, d, eps, 0, (hipStream_t)stream,
+                  "pf_layernorm_fwd");
+}
+
+extern "C" int pf_layernorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
+                                const float* mean, const float* rstd, const void* dx_add, int add_dtype, void* dx,
+                                int dx_dtype, float* dgamma_acc, float* dbeta_acc, float* workspace, int64_t rows,
+                                int64_t d, void* stream) {
+  return norm_bwd(dy, dy_dtype, x, x_dtype, gamma, mean, rstd, dx_add, add_dtype, dx, dx_dtype, dgamma_acc,
+                  dbeta_acc, workspace, rows, d, 0, (hipStream_t)stream, "pf_layernorm_bwd");
+}
+
+extern "C" int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, void* y, int y_dtype, float* rstd,
+                              int64_t rows, int64_t d, float eps, void* stream) {
+  return norm_fwd(x, x_dtype, gamma, nullptr, y, y_dtype, nullptr, rstd, rows, d, eps, 1, (hipStream_t)stream,
+                  "pf_rmsnorm_fwd");
+}
+
+extern "C" int pf_rmsnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
+                              const float* rstd, const void* dx_add, int add_dtype, void* dx, int dx_dtype,
+                              float* dgamma_acc, float* workspace, int64_t rows, int64_t d, void* stream) {
+  return norm_bwd(dy, dy_dtype, x, x_dtype, gamma, nullptr, rstd, dx_add, add_dtype, dx, dx_dtype, dgamma_acc,
+                  nullptr, workspace, rows, d, 1, (hipStream_t)stream, "pf_rmsnorm_bwd");
+}
+
+extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
+                                    float* workspace, void* stream) {
+  hipStream_t st = (hipStream_t)stream;
+  PF_REQUIRE(rows >= 0 && cols >= 0 && ld >= cols, "pf_colsum_accumulate: bad shape");
+  if (rows == 0 || cols == 0) return PF_OK;
+  PF_REQUIRE(x && acc && workspace, "pf_colsum_accumulate: null pointer");
+  PF_REQUIRE(pf_is_float_dtype(x_dtype), "pf_colsum_accumulate: bad dtype");
+  int64_t chunks = (rows + 31) / 32;
+  if (chunks > 256) chunks = 256;
+  const int64_t rpc = (rows + chunks - 1) / chunks;
+  chunks = (rows + rpc - 1) / rpc;
+  const bool v = vec_ok(x, x_dtype, ld) && cols % 8 == 0;
+  if (v) {
+    const dim3 grid((unsigned)((cols + 511) / 512), (unsigned)chunks);
+    hipLaunchKernelGGL(colsum_kernel<8>, grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc);
+  } else {
+    const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)chunks);
+    hipLaunchKernelGGL(colsum_kernel<1>, grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc);
+  }
+  PF_CHECK_LAUNCH("pf_colsum_accumulate");
+  hipLaunchKernelGGL(colreduce_finalize_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, st, workspace,
+                     (int)chunks, cols, cols, acc);
+  PF_CHECK_LAUNCH("pf_colsum_accumulate(finalize)");
+  return PF_OK;
+}

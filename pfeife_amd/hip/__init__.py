@@ -1,0 +1,330 @@
+"""ctypes binding of libpfeife_hip.so and the tensor-level kernel table built on it.
+
+`HipKernels` is the only kernel table the product ships: every method takes
+preallocated torch tensors (device memory owned by PyTorch), resolves them to raw
+pointers once, and returns a *prepared launch*: a callable `launch(stream)` that
+re-issues exactly the same C call.  Stage programs are lists of prepared
+launches, so a steady-state step does no argument marshalling at all.
+
+There is no fallback: if the shared library is missing, `load()` raises.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, byref, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpfeife_hip.so")
+ABI_VERSION = 1
+
+PF_F32, PF_F16, PF_BF16, PF_I64, PF_I32, PF_U8 = 0, 1, 2, 3, 4, 5
+ACT_NONE, ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU = 0, 1, 2, 3, 4
+
+_DTYPE_CODE = {
+    torch.float32: PF_F32,
+    torch.float16: PF_F16,
+    torch.bfloat16: PF_BF16,
+    torch.int64: PF_I64,
+    torch.int32: PF_I32,
+    torch.uint8: PF_U8,
+}
+
+
+def dtype_code(dtype):
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise RuntimeError("pfeife_amd: dtype %s has no HIP kernel support" % (dtype,))
+
+
+class GemmDesc(Structure):
+    """Mirror of `pf_gemm_desc` in include/pfeife_hip.h (field order is ABI)."""
+
+    _fields_ = [
+        ("in_dtype", c_int32), ("c_dtype", c_int32), ("a_trans", c_int32), ("b_trans", c_int32),
+        ("M", c_int64), ("N", c_int64), ("K", c_int64),
+        ("A", c_void_p), ("lda", c_int64),
+        ("B", c_void_p), ("ldb", c_int64),
+        ("C", c_void_p), ("ldc", c_int64),
+        ("batch1", c_int64), ("batch2", c_int64),
+        ("a_stride1", c_int64), ("a_stride2", c_int64),
+        ("b_stride1", c_int64), ("b_stride2", c_int64),
+        ("c_stride1", c_int64), ("c_stride2", c_int64),
+        ("alpha", c_float), ("beta", c_int32),
+        ("bias", c_void_p), ("bias_dtype", c_int32), ("round_mid", c_int32),
+        ("aux_out", c_void_p), ("ld_aux_out", c_int64),
+        ("act", c_int32), ("dact", c_int32),
+        ("aux_in", c_void_p), ("ld_aux_in", c_int64),
+        ("residual", c_void_p), ("ld_res", c_int64),
+        ("res_dtype", c_int32), ("reserved", c_int32),
+    ]
+
+
+# name -> argtypes (every function returns int unless listed in _RET_I64)
+_P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
+_SIGNATURES = {
+    "pf_init": [_I],
+    "pf_gemm": [POINTER(GemmDesc), _P],
+    "pf_layernorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _F, _P],
+    "pf_layernorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P],
+    "pf_rmsnorm_fwd": [_P, _I, _P, _P, _I, _P, _L, _L, _F, _P],
+    "pf_rmsnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _L, _L, _P],
+    "pf_colsum_accumulate": [_P, _I, _L, _L, _L, _P, _P, _P],
+    "pf_softmax_fwd": [_P, _L, _P, _I, _L, _L, _L, _L, _I, _P],
+    "pf_softmax_bwd": [_P, _L, _P, _I, _L, _P, _I, _L, _L, _L, _F, _P],
+    "pf_cross_entropy_fwd": [_P, _I, _P, _P, _P, _P, _L, _L, _L, _P],
+    "pf_cross_entropy_bwd": [_P, _I, _P, _P, _P, _P, _P, _I, _L, _L, _L, _P],
+    "pf_mse_fwd": [_P, _I, _P, _I, _P, _P, _L, _P],
+    "pf_mse_bwd": [_P, _I, _P, _I, _P, _P, _I, _L, _P],
+    "pf_sum_fwd": [_P, _I, _P, _P, _L, _P],
+    "pf_act_fwd": [_P, _P, _I, _I, _L, _P],
+    "pf_act_bwd": [_P, _P, _P, _I, _I, _L, _P],
+    "pf_glu_fwd": [_P, _L, _P, _L, _P, _L, _I, _I, _L, _L, _P],
+    "pf_glu_bwd": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _L, _L, _P],
+    "pf_axpby": [_P, _I, _F, _P, _I, _F, _P, _I, _L, _P],
+    "pf_bias_add": [_P, _I, _P, _I, _P, _I, _L, _L, _P],
+    "pf_cast": [_P, _I, _P, _I, _L, _P],
+    "pf_fill": [_P, _I, _F, _L, _P],
+    "pf_copy_strided": [_P, _I, POINTER(c_int64), _P, _I, POINTER(c_int64), POINTER(c_int64), _I, _I, _P],
+    "pf_rope": [_P, _P, _I, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P],
+    "pf_grad_accumulate_f32": [_P, _P, _I, _L, _P],
+    "pf_split_gather": [_P, _P, _L, _L, _L, _P, _P],
+    "pf_merge_scatter": [_P, _P, _L, _L, _L, _P, _P],
+    "pf_embedding_fwd": [_P, _I, _P, _P, _I, _L, _L, _L, _P],
+    "pf_embedding_bwd": [_P, _I, _P, _P, _L, _L, _L, _P],
+}
+_RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L]}
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_RET_I64) + ["pf_version", "pf_last_error"])
+
+_lib = None
+
+
+def load(path=None):
+    """Load the shared library (once) and declare every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = path or LIB_PATH
+    if not os.path.exists(path):
+        raise RuntimeError(
+            "pfeife_amd: %s is missing. Build it with `python -m pfeife_amd.hip.build` "
+            "(hipcc, gfx950). There is no fallback path." % path
+        )
+    lib = ctypes.CDLL(path)
+    lib.pf_version.restype = c_int
+    lib.pf_version.argtypes = []
+    lib.pf_last_error.restype = c_char_p
+    lib.pf_last_error.argtypes = []
+    for name, args in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = c_int
+        fn.argtypes = args
+    for name, args in _RET_I64.items():
+        fn = getattr(lib, name)
+        fn.restype = c_int64
+        fn.argtypes = args
+    if lib.pf_version() != ABI_VERSION:
+        raise RuntimeError("pfeife_amd: library ABI %d != binding ABI %d" % (lib.pf_version(), ABI_VERSION))
+    _lib = lib
+    return lib
+
+
+def last_error():
+    return load().pf_last_error().decode("utf-8", "replace")
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _dt(t, default=PF_F32):
+    return default if t is None else dtype_code(t.dtype)
+
+
+def current_stream_ptr():
+    return torch.cuda.current_stream().cuda_stream
+
+
+class HipKernels:
+    """Tensor-level kernel table backed by libpfeife_hip.so.
+
+    Every public method returns a prepared launch `fn(stream)`; `run(name, ...)`
+    prepares and immediately issues it on torch's current stream.
+    """
+
+    name = "hip"
+
+    def __init__(self, device=None):
+        self.lib = load()
+        if not torch.cuda.is_available():
+            raise RuntimeError("pfeife_amd: no GPU visible; the HIP kernel table cannot run")
+        self.device = torch.device("cuda", torch.cuda.current_device() if device is None else device)
+        rc = self.lib.pf_init(self.device.index or 0)
+        if rc != 0:
+            raise RuntimeError("pfeife_amd: pf_init failed: %s" % last_error())
+
+    # -- helpers -------------------------------------------------------------
+    def _prep(self, fname, args, keep):
+        fn = getattr(self.lib, fname)
+        lib = self.lib
+
+        def launch(stream, _fn=fn, _args=args, _keep=keep, _name=fname):
+            rc = _fn(*_args, stream)
+            if rc != 0:
+                raise RuntimeError("%s failed (%d): %s" % (_name, rc, lib.pf_last_error().decode()))
+
+        launch.kernel = fname
+        return launch
+
+    def run(self, name, *a, **kw):
+        getattr(self, name)(*a, **kw)(current_stream_ptr())
+
+    def colreduce_workspace(self, rows, cols):
+        return int(self.lib.pf_colreduce_workspace(rows, cols))
+
+    def reduce_workspace(self, n):
+        return int(self.lib.pf_reduce_workspace(n))
+
+    # -- dense contractions ----------------------------------------------------
+    def gemm(self, a, b, c, M, N, K, lda, ldb, ldc, a_trans=0, b_trans=0, batch=(1, 1), sa=(0, 0), sb=(0, 0),
+             sc=(0, 0), alpha=1.0, beta=0, bias=None, round_mid=0, aux_out=None, ld_aux_out=0, act=0, dact=0,
+             aux_in=None, ld_aux_in=0, residual=None, ld_res=0):
+        if a.dtype != b.dtype:
+            raise RuntimeError("gemm: operand dtypes differ (%s, %s)" % (a.dtype, b.dtype))
+        d = GemmDesc()
+        d.in_dtype, d.c_dtype = dtype_code(a.dtype), dtype_code(c.dtype)
+        d.a_trans, d.b_trans = int(a_trans), int(b_trans)
+        d.M, d.N, d.K = M, N, K
+        d.A, d.lda, d.B, d.ldb, d.C, d.ldc = _ptr(a), lda, _ptr(b), ldb, _ptr(c), ldc
+        d.batch1, d.batch2 = batch
+        d.a_stride1, d.a_stride2 = sa
+        d.b_stride1, d.b_stride2 = sb
+        d.c_stride1, d.c_stride2 = sc
+        d.alpha, d.beta = alpha, int(beta)
+        d.bias, d.bias_dtype, d.round_mid = _ptr(bias), _dt(bias), int(round_mid)
+        d.aux_out, d.ld_aux_out = _ptr(aux_out), ld_aux_out
+        d.act, d.dact = int(act), int(dact)
+        d.aux_in, d.ld_aux_in = _ptr(aux_in), ld_aux_in
+        d.residual, d.ld_res, d.res_dtype = _ptr(residual), ld_res, _dt(residual)
+        for t in (aux_out, aux_in):
+            if t is not None and t.dtype != a.dtype:
+                raise RuntimeError("gemm: aux tensors must have the operand dtype")
+        return self._prep("pf_gemm", (byref(d),), (d, a, b, c, bias, aux_out, aux_in, residual))
+
+    # -- normalisation -----------------------------------------------------------
+    def layernorm_fwd(self, x, gamma, beta, y, mean, rstd, rows, d, eps):
+        args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(beta), _ptr(y), _dt(y), _ptr(mean), _ptr(rstd), rows, d, eps)
+        return self._prep("pf_layernorm_fwd", args, (x, gamma, beta, y, mean, rstd))
+
+    def layernorm_bwd(self, dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws, rows, d):
+        args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx_add), _dt(dx_add),
+                _ptr(dx), _dt(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), rows, d)
+        return self._prep("pf_layernorm_bwd", args, (dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws))
+
+    def rmsnorm_fwd(self, x, gamma, y, rstd, rows, d, eps):
+        args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(y), _dt(y), _ptr(rstd), rows, d, eps)
+        return self._prep("pf_rmsnorm_fwd", args, (x, gamma, y, rstd))
+
+    def rmsnorm_bwd(self, dy, x, gamma, rstd, dx_add, dx, dgamma, ws, rows, d):
+        args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(rstd), _ptr(dx_add), _dt(dx_add), _ptr(dx),
+                _dt(dx), _ptr(dgamma), _ptr(ws), rows, d)
+        return self._prep("pf_rmsnorm_bwd", args, (dy, x, gamma, rstd, dx_add, dx, dgamma, ws))
+
+    def colsum_accumulate(self, x, rows, cols, ld, acc, ws):
+        args = (_ptr(x), _dt(x), rows, cols, ld, _ptr(acc), _ptr(ws))
+        return self._prep("pf_colsum_accumulate", args, (x, acc, ws))
+
+    # -- softmax / losses ----------------------------------------------------------
+    def softmax_fwd(self, s, ld_s, p, ld_p, rows, cols, q_len, causal):
+        args = (_ptr(s), ld_s, _ptr(p), _dt(p), ld_p, rows, cols, q_len, int(causal))
+        return self._prep("pf_softmax_fwd", args, (s, p))
+
+    def softmax_bwd(self, dp, ld_dp, p, ld_p, ds, ld_ds, rows, cols, scale):
+        args = (_ptr(dp), ld_dp, _ptr(p), _dt(p), ld_p, _ptr(ds), _dt(ds), ld_ds, rows, cols, scale)
+        return self._prep("pf_softmax_bwd", args, (dp, p, ds))
+
+    def cross_entropy_fwd(self, logits, targets, row_loss, row_lse, loss, rows, classes, ignore_index):
+        args = (_ptr(logits), _dt(logits), _ptr(targets), _ptr(row_loss), _ptr(row_lse), _ptr(loss), rows, classes,
+                ignore_index)
+        return self._prep("pf_cross_entropy_fwd", args, (logits, targets, row_loss, row_lse, loss))
+
+    def cross_entropy_bwd(self, logits, targets, row_lse, dloss, loss, dlogits, rows, classes, ignore_index):
+        n_valid = loss.data_ptr() + 4
+        args = (_ptr(logits), _dt(logits), _ptr(targets), _ptr(row_lse), _ptr(dloss), n_valid, _ptr(dlogits),
+                _dt(dlogits), rows, classes, ignore_index)
+        return self._prep("pf_cross_entropy_bwd", args, (logits, targets, row_lse, dloss, loss, dlogits))
+
+    def mse_fwd(self, a, b, partial, loss, n):
+        args = (_ptr(a), _dt(a), _ptr(b), _dt(b), _ptr(partial), _ptr(loss), n)
+        return self._prep("pf_mse_fwd", args, (a, b, partial, loss))
+
+    def mse_bwd(self, a, b, dloss, da, n):
+        args = (_ptr(a), _dt(a), _ptr(b), _dt(b), _ptr(dloss), _ptr(da), _dt(da), n)
+        return self._prep("pf_mse_bwd", args, (a, b, dloss, da))
+
+    def sum_fwd(self, x, partial, loss, n):
+        args = (_ptr(x), _dt(x), _ptr(partial), _ptr(loss), n)
+        return self._prep("pf_sum_fwd", args, (x, partial, loss))
+
+    # -- elementwise -----------------------------------------------------------------
+    def act_fwd(self, x, y, act, n):
+        return self._prep("pf_act_fwd", (_ptr(x), _ptr(y), _dt(x), int(act), n), (x, y))
+
+    def act_bwd(self, dy, x, dx, act, n):
+        return self._prep("pf_act_bwd", (_ptr(dy), _ptr(x), _ptr(dx), _dt(x), int(act), n), (dy, x, dx))
+
+    def glu_fwd(self, gate, ld_gate, up, ld_up, y, ld_y, act, rows, cols):
+        args = (_ptr(gate), ld_gate, _ptr(up), ld_up, _ptr(y), ld_y, _dt(gate), int(act), rows, cols)
+        return self._prep("pf_glu_fwd", args, (gate, up, y))
+
+    def glu_bwd(self, dy, ld_dy, gate, ld_gate, up, ld_up, dgate, ld_dgate, dup, ld_dup, act, rows, cols):
+        args = (_ptr(dy), ld_dy, _ptr(gate), ld_gate, _ptr(up), ld_up, _ptr(dgate), ld_dgate, _ptr(dup), ld_dup,
+                _dt(gate), int(act), rows, cols)
+        return self._prep("pf_glu_bwd", args, (dy, gate, up, dgate, dup))
+
+    def axpby(self, a, alpha, b, beta, out, n):
+        args = (_ptr(a), _dt(a), alpha, _ptr(b), _dt(b), beta, _ptr(out), _dt(out), n)
+        return self._prep("pf_axpby", args, (a, b, out))
+
+    def bias_add(self, x, bias, y, n, bias_len):
+        args = (_ptr(x), _dt(x), _ptr(bias), _dt(bias), _ptr(y), _dt(y), n, bias_len)
+        return self._prep("pf_bias_add", args, (x, bias, y))
+
+    def cast(self, src, dst, n):
+        return self._prep("pf_cast", (_ptr(src), _dt(src), _ptr(dst), _dt(dst), n), (src, dst))
+
+    def fill(self, dst, value, n):
+        return self._prep("pf_fill", (_ptr(dst), _dt(dst), float(value), n), (dst,))
+
+    def copy_strided(self, src, src_strides, dst, dst_strides, sizes, accumulate=0):
+        nd = len(sizes)
+        arr = c_int64 * nd
+        ss, ds, sz = arr(*src_strides), arr(*dst_strides), arr(*sizes)
+        args = (_ptr(src), _dt(src), ss, _ptr(dst), _dt(dst), ds, sz, nd, int(accumulate))
+        return self._prep("pf_copy_strided", args, (src, dst, ss, ds, sz))
+
+    def rope(self, x, y, cos_t, sin_t, B, T, H, D, xs, ys, inverse):
+        args = (_ptr(x), _ptr(y), _dt(x), _ptr(cos_t), _ptr(sin_t), B, T, H, D, xs[0], xs[1], xs[2], ys[0], ys[1],
+                ys[2], int(inverse))
+        return self._prep("pf_rope", args, (x, y, cos_t, sin_t))
+
+    def grad_accumulate(self, acc, g, n):
+        return self._prep("pf_grad_accumulate_f32", (_ptr(acc), _ptr(g), _dt(g), n), (acc, g))
+
+    # -- micro-batch split / merge, embedding ---------------------------------------------
+    def split_gather(self, src, dst, row_bytes, row_start, n_rows, index=None):
+        args = (_ptr(src), _ptr(dst), row_bytes, row_start, n_rows, _ptr(index))
+        return self._prep("pf_split_gather", args, (src, dst, index))
+
+    def merge_scatter(self, src, dst, row_bytes, row_start, n_rows, index=None):
+        args = (_ptr(src), _ptr(dst), row_bytes, row_start, n_rows, _ptr(index))
+        return self._prep("pf_merge_scatter", args, (src, dst, index))
+
+    def embedding_fwd(self, table, ids, out, n_ids, dim, vocab):
+        args = (_ptr(table), _dt(table), _ptr(ids), _ptr(out), _dt(out), n_ids, dim, vocab)
+        return self._prep("pf_embedding_fwd", args, (table, ids, out))
+
+    def embedding_bwd(self, dout, ids, dtable, n_ids, dim, vocab):
+        args = (_ptr(dout), _dt(dout), _ptr(ids), _ptr(dtable), n_ids, dim, vocab)
+        return self._prep("pf_embedding_bwd", args, (dout, ids, dtable))

@@ -1,0 +1,385 @@
+"""Parity of every HIP kernel (through the C ABI) against the CPU oracle on the
+same seeded inputs.  Integer / byte movers must be bit-exact; floating-point
+kernels must agree within the tolerance written next to each test."""
+import itertools
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+F16, BF16, F32 = torch.float16, torch.bfloat16, torch.float32
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def both(hip, oracle, name, tensors, outs, **scalars):
+    """Run kernel `name` on the GPU (HIP) and on CPU (oracle) from identical
+    inputs; returns {out_name: (hip_result_on_cpu, oracle_result)}."""
+    print("kernel", name, {k: (tuple(v.shape), str(v.dtype)) for k, v in tensors.items() if v is not None},
+          scalars, flush=True)
+    dev = {k: (None if v is None else v.cuda()) for k, v in tensors.items()}
+    cpu = {k: (None if v is None else v.clone()) for k, v in tensors.items()}
+    hip.run(name, **dev, **scalars)
+    torch.cuda.synchronize()
+    oracle.run(name, **cpu, **scalars)
+    return {o: (dev[o].cpu(), cpu[o]) for o in outs}
+
+
+def close(pair, rtol, atol):
+    a, b = pair
+    assert a.dtype == b.dtype and a.shape == b.shape
+    torch.testing.assert_close(a.float(), b.float(), rtol=rtol, atol=atol)
+
+
+TOL = {F32: (2e-5, 2e-5), F16: (4e-3, 4e-3), BF16: (2e-2, 2e-2)}
+
+GEMM_SHAPES = [(197, 197, 64), (130, 72, 200), (257, 1000, 88), (512, 384, 1024), (64, 64, 8), (1, 8, 8)]
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+@pytest.mark.parametrize("a_trans,b_trans", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_gemm_layouts(hip, oracle, dtype, a_trans, b_trans):
+    for i, (M, N, K) in enumerate(GEMM_SHAPES):
+        pad = 8
+        lda = (M if a_trans else K) + pad
+        ldb = (N if b_trans else K) + pad
+        ldc = N + 3
+        a = rnd((K if a_trans else M, lda), dtype, 10 + i)
+        b = rnd((K if b_trans else N, ldb), dtype, 20 + i)
+        c = torch.zeros(M, ldc, dtype=F32)
+        r = both(hip, oracle, "gemm", dict(a=a, b=b, c=c), ["c"], M=M, N=N, K=K, lda=lda, ldb=ldb, ldc=ldc,
+                 a_trans=a_trans, b_trans=b_trans, alpha=0.5)
+        # fp32 accumulation of the same 16-bit products: only the summation order differs
+        close(r["c"], rtol=1e-4, atol=1e-4 * (K ** 0.5))
+        assert torch.all(r["c"][0][:, N:] == 0), "columns beyond N were written"
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_gemm_batched_strided_heads(hip, oracle, dtype):
+    # attention layout: packed qkv [B, T, 3, H, hd]; S = Q K^T per (b, h); then P V
+    B, T, H, hd = 2, 197, 3, 64
+    C = H * hd
+    qkv = rnd((B, T, 3 * C), dtype, 1, 0.5)
+    Tp = 200
+    s = torch.zeros(B, H, T, Tp, dtype=F32)
+    q, k, v = qkv[:, :, 0:C], qkv[:, :, C:2 * C], qkv[:, :, 2 * C:]
+    for tab, dev_t in ((hip, "cuda"), (oracle, "cpu")):
+        pass
+    res = {}
+    for name, tab, dev in (("hip", hip, "cuda"), ("oracle", oracle, "cpu")):
+        t = qkv.to(dev)
+        S = s.to(dev)
+        tab.run("gemm", t[:, :, 0:C], t[:, :, C:2 * C], S, M=T, N=T, K=hd, lda=3 * C, ldb=3 * C, ldc=Tp,
+                batch=(B, H), sa=(T * 3 * C, hd), sb=(T * 3 * C, hd), sc=(H * T * Tp, T * Tp), alpha=hd ** -0.5)
+        P = torch.softmax(S[..., :T].float().cpu(), -1).to(dtype)
+        Pp = torch.zeros(B, H, T, Tp, dtype=dtype)
+        Pp[..., :T] = P
+        Pp = Pp.to(dev)
+        O = torch.zeros(B, T, C, dtype=dtype, device=dev)
+        tab.run("gemm", Pp, t[:, :, 2 * C:], O, M=T, N=hd, K=T, lda=Tp, ldb=3 * C, ldc=C, b_trans=1, batch=(B, H),
+                sa=(H * T * Tp, T * Tp), sb=(T * 3 * C, hd), sc=(T * C, hd))
+        if dev == "cuda":
+            torch.cuda.synchronize()
+        res[name] = (S.cpu(), O.cpu())
+    close((res["hip"][0], res["oracle"][0]), rtol=1e-4, atol=1e-3)
+    close((res["hip"][1], res["oracle"][1]), *TOL[dtype])
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        *(x.reshape(B, T, H, hd).transpose(1, 2).float() for x in (q, k, v))).transpose(1, 2).reshape(B, T, C)
+    torch.testing.assert_close(res["hip"][1].float(), ref, rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_gemm_epilogues(hip, oracle, dtype):
+    M, N, K = 300, 264, 136
+    x, w = rnd((M, K), dtype, 1), rnd((N, K), dtype, 2, 0.1)
+    bias = rnd((N,), dtype, 3)
+    rt, at = TOL[dtype]
+    # forward linear + bias + GELU, pre-activation kept
+    r = both(hip, oracle, "gemm", dict(a=x, b=w, c=torch.zeros(M, N, dtype=dtype), bias=bias,
+                                      aux_out=torch.zeros(M, N, dtype=dtype)), ["c", "aux_out"],
+             M=M, N=N, K=K, lda=K, ldb=K, ldc=N, round_mid=1, act=1, ld_aux_out=N)
+    close(r["c"], rt, at)
+    close(r["aux_out"], rt, at)
+    # backward through GELU: dH = (dY W) * gelu'(h)
+    dy = rnd((M, N), dtype, 4)
+    h = rnd((M, K), dtype, 5)
+    r = both(hip, oracle, "gemm", dict(a=dy, b=w, c=torch.zeros(M, K, dtype=dtype), aux_in=h), ["c"],
+             M=M, N=K, K=N, lda=N, ldb=K, ldc=K, b_trans=1, dact=1, ld_aux_in=K)
+    close(r["c"], rt, at * 4)
+    # residual add into an fp32 stream
+    res = rnd((M, N), F32, 6)
+    r = both(hip, oracle, "gemm", dict(a=x, b=w, c=torch.zeros(M, N, dtype=F32), bias=bias, residual=res), ["c"],
+             M=M, N=N, K=K, lda=K, ldb=K, ldc=N, round_mid=1, ld_res=N)
+    close(r["c"], rt, at)
+    # weight gradient accumulated into fp32 (beta = 1)
+    acc = rnd((N, K), F32, 7)
+    r = both(hip, oracle, "gemm", dict(a=dy, b=x, c=acc), ["c"], M=N, N=K, K=M, lda=N, ldb=K, ldc=K, a_trans=1,
+             b_trans=1, beta=1)
+    close(r["c"], rtol=1e-4, atol=2e-3)
+
+
+def test_gemm_full_size_vit_l(hip, oracle):
+    # qkv projection of ViT-L/16 at micro-batch 16: [3152 x 1024] . [1024 x 3072]
+    M, N, K = 3152, 3072, 1024
+    x, w = rnd((M, K), F16, 1), rnd((N, K), F16, 2, 0.03)
+    r = both(hip, oracle, "gemm", dict(a=x, b=w, c=torch.zeros(M, N, dtype=F16)), ["c"], M=M, N=N, K=K, lda=K,
+             ldb=K, ldc=N)
+    close(r["c"], *TOL[F16])
+
+
+def test_gemm_rejects_bad_arguments(hip):
+    a = torch.zeros(8, 12, dtype=F16, device="cuda")
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        hip.run("gemm", a, a, torch.zeros(8, 8, device="cuda"), M=8, N=8, K=12, lda=12, ldb=12, ldc=8)
+    with pytest.raises(RuntimeError, match="lda"):
+        hip.run("gemm", a, a, torch.zeros(8, 8, device="cuda"), M=8, N=8, K=16, lda=8, ldb=16, ldc=8)
+
+
+@pytest.mark.parametrize("xdt,ydt", [(F32, F16), (F32, BF16), (F32, F32), (F16, F16), (BF16, BF16)])
+@pytest.mark.parametrize("rows,d", [(37, 1024), (5, 1408), (9, 100), (3, 2048)])
+def test_layernorm_rmsnorm(hip, oracle, xdt, ydt, rows, d):
+    x = rnd((rows, d), xdt, 1) + 0.5
+    gamma, beta = rnd((d,), F32, 2) + 1, rnd((d,), F32, 3)
+    rt, at = TOL[ydt]
+    t = dict(x=x, gamma=gamma, beta=beta, y=torch.zeros(rows, d, dtype=ydt), mean=torch.zeros(rows),
+             rstd=torch.zeros(rows))
+    r = both(hip, oracle, "layernorm_fwd", t, ["y", "mean", "rstd"], rows=rows, d=d, eps=1e-5)
+    close(r["y"], rt, at)
+    close(r["mean"], 1e-5, 1e-5)
+    close(r["rstd"], 1e-5, 1e-5)
+    mean, rstd = r["mean"][1], r["rstd"][1]
+    dy = rnd((rows, d), ydt, 4)
+    add = rnd((rows, d), xdt, 5)
+    ws = torch.zeros(2 * 512 * d)
+    t = dict(dy=dy, x=x, gamma=gamma, mean=mean, rstd=rstd, dx_add=add, dx=torch.zeros(rows, d, dtype=xdt),
+             dgamma=rnd((d,), F32, 6), dbeta=rnd((d,), F32, 7), ws=ws)
+    r = both(hip, oracle, "layernorm_bwd", t, ["dx", "dgamma", "dbeta"], rows=rows, d=d)
+    close(r["dx"], *TOL[xdt])
+    close(r["dgamma"], 1e-4, 1e-4 * rows ** 0.5)
+    close(r["dbeta"], 1e-4, 1e-4 * rows ** 0.5)
+    # RMSNorm
+    t = dict(x=x, gamma=gamma, y=torch.zeros(rows, d, dtype=ydt), rstd=torch.zeros(rows))
+    r = both(hip, oracle, "rmsnorm_fwd", t, ["y", "rstd"], rows=rows, d=d, eps=1e-6)
+    close(r["y"], rt, at)
+    close(r["rstd"], 1e-5, 1e-5)
+    t = dict(dy=dy, x=x, gamma=gamma, rstd=r["rstd"][1], dx_add=None, dx=torch.zeros(rows, d, dtype=xdt),
+             dgamma=rnd((d,), F32, 6), ws=ws)
+    r = both(hip, oracle, "rmsnorm_bwd", t, ["dx", "dgamma"], rows=rows, d=d)
+    close(r["dx"], *TOL[xdt])
+    close(r["dgamma"], 1e-4, 1e-4 * rows ** 0.5)
+
+
+def test_layernorm_many_rows_param_grads(hip, oracle):
+    rows, d = 3152, 1024  # ViT-L residual stream at micro-batch 16: more rows than reduction workgroups
+    x, dy = rnd((rows, d), F32, 1), rnd((rows, d), F16, 2)
+    gamma = rnd((d,), F32, 3) + 1
+    mean, rstd = x.mean(1), 1 / torch.sqrt(x.var(1, unbiased=False) + 1e-5)
+    t = dict(dy=dy, x=x, gamma=gamma, mean=mean, rstd=rstd, dx_add=None, dx=torch.zeros(rows, d),
+             dgamma=torch.zeros(d), dbeta=torch.zeros(d), ws=torch.zeros(2 * 512 * d))
+    r = both(hip, oracle, "layernorm_bwd", t, ["dx", "dgamma", "dbeta"], rows=rows, d=d)
+    close(r["dx"], 1e-4, 1e-4)
+    close(r["dgamma"], 1e-4, 2e-2)
+    close(r["dbeta"], 1e-4, 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_colsum(hip, oracle, dtype):
+    for rows, cols, ld in [(3152, 1024, 1024), (77, 1000, 1000), (5, 13, 16), (4096, 96, 104)]:
+        x = rnd((rows, ld), dtype, 1)
+        t = dict(x=x, acc=rnd((cols,), F32, 2), ws=torch.zeros(2 * 512 * cols))
+        r = both(hip, oracle, "colsum_accumulate", t, ["acc"], rows=rows, cols=cols, ld=ld)
+        close(r["acc"], 1e-4, 1e-4 * rows ** 0.5 + 1e-3)
+
+
+@pytest.mark.parametrize("pdt", [F16, BF16, F32])
+@pytest.mark.parametrize("causal", [0, 1])
+def test_softmax(hip, oracle, pdt, causal):
+    for B, T, Tk in [(6, 197, 197), (2, 128, 128), (3, 64, 77)]:
+        if causal and T != Tk:
+            continue
+        rows, ldp = B * T, (Tk + 7) // 8 * 8
+        s = rnd((rows, Tk), F32, 1, 3.0)
+        t = dict(s=s, p=torch.full((rows, ldp), 7.0, dtype=pdt))
+        r = both(hip, oracle, "softmax_fwd", t, ["p"], ld_s=Tk, ld_p=ldp, rows=rows, cols=Tk, q_len=T, causal=causal)
+        close(r["p"], *TOL[pdt])
+        p = r["p"][1]
+        dp = rnd((rows, Tk), F32, 2)
+        t = dict(dp=dp, p=p, ds=torch.full((rows, ldp), 7.0, dtype=pdt))
+        r = both(hip, oracle, "softmax_bwd", t, ["ds"], ld_dp=Tk, ld_p=ldp, ld_ds=ldp, rows=rows, cols=Tk, scale=0.125)
+        close(r["ds"], *TOL[pdt])
+
+
+@pytest.mark.parametrize("ldt", [F16, BF16, F32])
+def test_cross_entropy(hip, oracle, ldt):
+    for rows, classes in [(16, 1000), (37, 32000), (4, 7)]:
+        logits = rnd((rows, classes), ldt, 1, 2.0)
+        g = torch.Generator().manual_seed(5)
+        targets = torch.randint(0, classes, (rows,), generator=g)
+        targets[rows // 2] = -100
+        t = dict(logits=logits, targets=targets, row_loss=torch.zeros(rows), row_lse=torch.zeros(rows),
+                 loss=torch.zeros(2))
+        r = both(hip, oracle, "cross_entropy_fwd", t, ["loss", "row_lse", "row_loss"], rows=rows, classes=classes,
+                 ignore_index=-100)
+        close(r["loss"], 1e-5, 1e-5)
+        close(r["row_lse"], 1e-5, 1e-5)
+        ref = torch.nn.functional.cross_entropy(logits.float(), targets, ignore_index=-100)
+        torch.testing.assert_close(r["loss"][0][0], ref, rtol=1e-5, atol=1e-5)
+        t = dict(logits=logits, targets=targets, row_lse=r["row_lse"][1], dloss=torch.tensor([1.7]),
+                 loss=r["loss"][1], dlogits=torch.zeros(rows, classes, dtype=ldt))
+        r = both(hip, oracle, "cross_entropy_bwd", t, ["dlogits"], rows=rows, classes=classes, ignore_index=-100)
+        close(r["dlogits"], TOL[ldt][0], 1e-5 if ldt == F32 else 1e-3)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_mse_sum(hip, oracle, dtype):
+    n = 4 * 4 * 32 * 32 + 3
+    a, b = rnd((n,), dtype, 1), rnd((n,), dtype, 2)
+    t = dict(a=a, b=b, partial=torch.zeros(1024), loss=torch.zeros(1))
+    r = both(hip, oracle, "mse_fwd", t, ["loss"], n=n)
+    close(r["loss"], 1e-5, 1e-6)
+    t = dict(a=a, b=b, dloss=torch.tensor([0.5]), da=torch.zeros(n, dtype=dtype))
+    r = both(hip, oracle, "mse_bwd", t, ["da"], n=n)
+    close(r["da"], TOL[dtype][0], 1e-6)
+    t = dict(x=a, partial=torch.zeros(1024), loss=torch.zeros(1))
+    r = both(hip, oracle, "sum_fwd", t, ["loss"], n=n)
+    close(r["loss"], 1e-4, 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+@pytest.mark.parametrize("act", [1, 2, 3, 4])
+def test_activations_and_glu(hip, oracle, dtype, act):
+    n = 8 * 1000 + 5
+    x, dy = rnd((n,), dtype, 1, 2.0), rnd((n,), dtype, 2)
+    rt, at = TOL[dtype]
+    r = both(hip, oracle, "act_fwd", dict(x=x, y=torch.zeros(n, dtype=dtype)), ["y"], act=act, n=n)
+    close(r["y"], rt, at)
+    r = both(hip, oracle, "act_bwd", dict(dy=dy, x=x, dx=torch.zeros(n, dtype=dtype)), ["dx"], act=act, n=n)
+    close(r["dx"], rt, at)
+    rows, cols, ld = 33, 264, 2 * 264
+    gu = rnd((rows, ld), dtype, 3)
+    res = {}
+    for name, tab, dev in (("hip", hip, "cuda"), ("oracle", oracle, "cpu")):
+        t = gu.to(dev)
+        y = torch.zeros(rows, cols, dtype=dtype, device=dev)
+        tab.run("glu_fwd", t, ld, t[:, cols:], ld, y, cols, act=act, rows=rows, cols=cols)
+        d = torch.zeros(rows, ld, dtype=dtype, device=dev)
+        dyy = rnd((rows, cols), dtype, 4).to(dev)
+        tab.run("glu_bwd", dyy, cols, t, ld, t[:, cols:], ld, d, ld, d[:, cols:], ld, act=act, rows=rows, cols=cols)
+        res[name] = (y.cpu(), d.cpu())
+    close((res["hip"][0], res["oracle"][0]), rt, at)
+    close((res["hip"][1], res["oracle"][1]), rt, at * 2)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_streaming_kernels(hip, oracle, dtype):
+    n = 3152 * 1024 + 7
+    a, b = rnd((n,), dtype, 1), rnd((n,), F32, 2)
+    rt, at = TOL[dtype]
+    r = both(hip, oracle, "axpby", dict(a=a, b=b, out=torch.zeros(n, dtype=F32)), ["out"], alpha=1.0, beta=1.0, n=n)
+    close(r["out"], 1e-6, 1e-6)
+    r = both(hip, oracle, "axpby", dict(a=b, b=None, out=torch.zeros(n, dtype=dtype)), ["out"], alpha=0.5, beta=0.0,
+             n=n)
+    close(r["out"], rt, at)
+    r = both(hip, oracle, "cast", dict(src=b, dst=torch.zeros(n, dtype=dtype)), ["dst"], n=n)
+    assert torch.equal(r["dst"][0], r["dst"][1]), "cast must round exactly like torch"
+    r = both(hip, oracle, "fill", dict(dst=torch.ones(n, dtype=dtype)), ["dst"], value=0.0, n=n)
+    assert torch.equal(r["dst"][0], r["dst"][1])
+    # fp32 gradient accumulation: identical single additions -> bit-exact
+    r = both(hip, oracle, "grad_accumulate", dict(acc=b.clone(), g=a), ["acc"], n=n)
+    assert torch.equal(r["acc"][0], r["acc"][1]), "grad accumulate must be bit-exact"
+    m = 1024 * 77
+    x, bias = rnd((m,), dtype, 3), rnd((1024,), F32, 4)
+    r = both(hip, oracle, "bias_add", dict(x=x, bias=bias, y=torch.zeros(m, dtype=F32)), ["y"], n=m, bias_len=1024)
+    close(r["y"], 1e-6, 1e-6)
+
+
+@pytest.mark.parametrize("dtype", [F16, F32])
+def test_copy_strided_and_rope(hip, oracle, dtype):
+    # patch extraction [B, C, Hp, p, Wp, p] -> [B, Hp, Wp, C, p, p]
+    B, C, Hp, p = 2, 3, 4, 16
+    img = rnd((B, C, Hp * p, Hp * p), F32, 1)
+    sizes = (B, Hp, Hp, C, p, p)
+    s = img.stride()
+    ss = (s[0], s[2] * p, s[3] * p, s[1], s[2], s[3])
+    out = torch.zeros(B * Hp * Hp, C * p * p, dtype=dtype)
+    ds = (Hp * Hp * C * p * p, Hp * C * p * p, C * p * p, p * p, p, 1)
+    r = both(hip, oracle, "copy_strided", dict(src=img, dst=out), ["dst"], src_strides=ss, dst_strides=ds, sizes=sizes)
+    assert torch.equal(r["dst"][0], r["dst"][1])
+    ref = img.reshape(B, C, Hp, p, Hp, p).permute(0, 2, 4, 1, 3, 5).reshape(B * Hp * Hp, -1).to(dtype)
+    assert torch.equal(r["dst"][0], ref)
+    # scalar path + accumulate
+    src = rnd((5, 7, 3), dtype, 2)
+    dst = rnd((3, 5, 7), dtype, 3)
+    r = both(hip, oracle, "copy_strided", dict(src=src, dst=dst), ["dst"], src_strides=(21, 3, 1),
+             dst_strides=(7, 1, 35), sizes=(5, 7, 3), accumulate=1)
+    close(r["dst"], *TOL[dtype])
+    # rotary embedding on q inside a packed [B, T, 3, H, D] tensor, forward then inverse = identity
+    Bq, T, H, D = 2, 33, 4, 64
+    qkv = rnd((Bq, T, 3 * H * D), dtype, 4)
+    inv_freq = 1.0 / (10000 ** (torch.arange(0, D, 2).float() / D))
+    ang = torch.arange(T).float()[:, None] * inv_freq[None, :]
+    cos_t, sin_t = ang.cos().contiguous(), ang.sin().contiguous()
+    xs = (T * 3 * H * D, 3 * H * D, D)
+    y = torch.zeros(Bq, T, H, D, dtype=dtype)
+    r = both(hip, oracle, "rope", dict(x=qkv, y=y, cos_t=cos_t, sin_t=sin_t), ["y"], B=Bq, T=T, H=H, D=D, xs=xs,
+             ys=(T * H * D, H * D, D), inverse=0)
+    close(r["y"], *TOL[dtype])
+    back = both(hip, oracle, "rope", dict(x=r["y"][1], y=torch.zeros_like(y), cos_t=cos_t, sin_t=sin_t), ["y"], B=Bq,
+                T=T, H=H, D=D, xs=(T * H * D, H * D, D), ys=(T * H * D, H * D, D), inverse=1)
+    close((back["y"][0], qkv.view(Bq, T, 3, H, D)[:, :, 0].contiguous()), TOL[dtype][0] * 3, TOL[dtype][1] * 3)
+
+
+def test_split_merge_bit_exact(hip, oracle):
+    g = torch.Generator().manual_seed(3)
+    for N, n, shape_tail, dtype in [(64, 4, (3, 8, 8), F32), (10, 4, (5,), torch.int64), (7, 3, (3,), torch.uint8),
+                                    (5, 8, (2, 2), F16), (16, 4, (), torch.int64)]:
+        if dtype in (F32, F16):
+            full = torch.randn((N,) + shape_tail, generator=g).to(dtype)
+        else:
+            full = torch.randint(0, 200, (N,) + shape_tail, generator=g).to(dtype)
+        row_bytes = full[0].numel() * full.element_size() if N else 0
+        chunks = torch.tensor_split(full, n, 0)
+        merged = {"hip": torch.zeros_like(full).cuda(), "oracle": torch.zeros_like(full)}
+        start = 0
+        for ch in chunks:
+            rows = ch.shape[0]
+            for name, tab, dev in (("hip", hip, "cuda"), ("oracle", oracle, "cpu")):
+                slab = torch.zeros_like(ch).to(dev)
+                tab.run("split_gather", full.to(dev), slab, row_bytes=row_bytes, row_start=start, n_rows=rows)
+                assert torch.equal(slab.cpu(), ch), (name, N, n, start)
+                tab.run("merge_scatter", slab, merged[name], row_bytes=row_bytes, row_start=start, n_rows=rows)
+            start += rows
+        assert start == N
+        torch.cuda.synchronize()
+        assert torch.equal(merged["hip"].cpu(), full) and torch.equal(merged["oracle"], full)
+    # indexed gather / scatter
+    full = torch.randn(33, 24, generator=g)
+    idx = torch.randperm(33, generator=g)[:9]
+    for name, tab, dev in (("hip", hip, "cuda"), ("oracle", oracle, "cpu")):
+        out = torch.zeros(9, 24, device=dev)
+        tab.run("split_gather", full.to(dev), out, row_bytes=96, row_start=0, n_rows=9, index=idx.to(dev))
+        assert torch.equal(out.cpu(), full[idx]), name
+        back = torch.zeros(33, 24, device=dev)
+        tab.run("merge_scatter", out, back, row_bytes=96, row_start=0, n_rows=9, index=idx.to(dev))
+        ref = torch.zeros(33, 24)
+        ref[idx] = full[idx]
+        assert torch.equal(back.cpu(), ref), name
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_embedding(hip, oracle, dtype):
+    vocab, dim, n = 1000, 264, 300
+    table = rnd((vocab, dim), F32, 1)
+    g = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, 50, (n,), generator=g)  # heavy collisions
+    r = both(hip, oracle, "embedding_fwd", dict(table=table, ids=ids, out=torch.zeros(n, dim, dtype=dtype)), ["out"],
+             n_ids=n, dim=dim, vocab=vocab)
+    assert torch.equal(r["out"][0], r["out"][1])
+    dout = rnd((n, dim), dtype, 3)
+    r = both(hip, oracle, "embedding_bwd", dict(dout=dout, ids=ids, dtable=rnd((vocab, dim), F32, 4)), ["dtable"],
+             n_ids=n, dim=dim, vocab=vocab)
+    close(r["dtable"], 1e-5, 1e-5)
