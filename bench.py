@@ -1,0 +1,264 @@
+"""Headline benchmark: train samples/sec of the pipeline-stage hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vit_l16_fp16]
+
+One "step" is one PartialRunner.step(): micro-batch split, forward + backward of
+every stage in the looped schedule's order for every micro-batch, fp32 gradient
+accumulation, loss, optimizer step.  Inputs are resident in HBM before the timed
+region.  Prints ONE JSON line (the last line of stdout).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}
+PEAK_HBM_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+WORKLOADS = {
+    # name: (model family, config attr, global batch, batch_cnt, split points, device_cnt, mixed precision)
+    "vit_l16_fp16": ("vit", "VIT_L16", 64, 4, ["blocks.12"], 2, "fp16"),
+    "vit_s16_fp32": ("vit", "VIT_S16", 16, 4, ["blocks.6"], 2, None),
+}
+
+
+def build_workload(name, device):
+    import torch
+
+    from pfeife_amd.bench_models import vit
+    from pfeife_amd.loss import CrossEntropyLoss
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife, partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
+    cfg = getattr(vit, cfg_name)
+    torch.manual_seed(42)
+    model = vit.VisionTransformer(cfg)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(batch, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
+    y = torch.randint(0, cfg.num_classes, (batch,), generator=g)
+    initialize_pfeife()
+    option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
+                        split_points=splits, mixed_precision=mixed, optimizer=dict(type="adam", lr=1e-5))
+    runner = PartialRunner(option)
+    model.to(device)
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = CrossEntropyLoss(cfg.num_classes)
+
+    def exec_fn(px, labels):
+        out = cmodel(px)
+        loss = crit(out, labels)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(exec_fn)
+    info = dict(cfg=cfg, batch=batch, batch_cnt=batch_cnt, splits=splits, device_cnt=device_cnt, mixed=mixed,
+                model=model, family=family)
+    return runner, (x.to(device), y.to(device)), info
+
+
+def gemm_roofline(runner, mixed, reps=3):
+    """Replays every matrix-product launch of one step, grouped by kernel
+    instantiation, between HIP events on the launch stream; returns the roofline
+    record of the instantiation that takes the most time plus an all-GEMM summary."""
+    import torch
+
+    groups = {}
+    for slot in runner.worker.mbs.values():
+        for prog in slot.stage_programs.values():
+            for launch in list(prog.fwd) + list(prog.bwd):
+                if getattr(launch, "kernel", "") == "pf_gemm":
+                    g = groups.setdefault(launch.variant, dict(launches=[], flops=0.0))
+                    g["launches"].append(launch)
+                    g["flops"] += launch.flops
+    stream = torch.cuda.current_stream()
+    sp = stream.cuda_stream
+    out = {}
+    for name, g in groups.items():
+        for launch in g["launches"]:  # warm
+            launch(sp)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(stream)
+        for _ in range(reps):
+            for launch in g["launches"]:
+                launch(sp)
+        ev1.record(stream)
+        ev1.synchronize()
+        ms = ev0.elapsed_time(ev1) / reps
+        n = len(g["launches"])
+        out[name] = dict(ms_per_step=ms, launches_per_step=n, flops_per_step=g["flops"],
+                         avg_launch_us=1e3 * ms / n, tflops=g["flops"] / (ms * 1e-3) / 1e12)
+    if not out:
+        return None, {}
+    dom = max(out, key=lambda k: out[k]["ms_per_step"])
+    peak = PEAK_TFLOPS[mixed or "fp32"]
+    d = out[dom]
+    tot_ms = sum(v["ms_per_step"] for v in out.values())
+    tot_fl = sum(v["flops_per_step"] for v in out.values())
+    roof = dict(bound="mfma", achieved=round(d["tflops"], 2), peak=peak, unit="TFLOP/s",
+                frac=round(d["tflops"] / peak, 4), traffic=None, kernel=dom,
+                avg_launch_us=round(d["avg_launch_us"], 2), launches_per_step=d["launches_per_step"],
+                flops_per_launch=d["flops_per_step"] / d["launches_per_step"],
+                all_gemm_tflops=round(tot_fl / (tot_ms * 1e-3) / 1e12, 2), all_gemm_ms_per_step=round(tot_ms, 3))
+    return roof, out
+
+
+def hbm_kernel_rates(runner, reps=3):
+    """Achieved HBM GB/s of the fp32 gradient-accumulate kernel at the size of the
+    largest weight matrix (12 bytes per element: read g, read acc, write acc)."""
+    import torch
+
+    k = runner.worker.kernels
+    n = 4096 * 1024 * 16
+    acc = torch.zeros(n, device="cuda")
+    g = torch.ones(n, device="cuda")
+    launch = k.grad_accumulate(acc, g, n)
+    stream = torch.cuda.current_stream()
+    launch(stream.cuda_stream)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record(stream)
+    for _ in range(reps * 5):
+        launch(stream.cuda_stream)
+    ev1.record(stream)
+    ev1.synchronize()
+    ms = ev0.elapsed_time(ev1) / (reps * 5)
+    gbs = 12.0 * n / (ms * 1e-3) / 1e9
+    return dict(kernel="pf_grad_accumulate_f32", elements=n, avg_launch_us=round(ms * 1e3, 2),
+                achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4))
+
+
+def cpu_baseline(name):
+    """The oracle's restatement of the reference's stage execution on the host
+    cores, fp32, on a bounded sample of the workload (2 micro-batches of 4)."""
+    import torch
+    import torch.nn as nn
+
+    from oracle.stage_oracle import run_pipeline_step
+    from pfeife_amd.bench_models import vit
+
+    family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
+    cfg = getattr(vit, cfg_name)
+    cores = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env:
+        cores = min(cores, int(env))
+    torch.set_num_threads(cores)
+    torch.manual_seed(42)
+    model = vit.VisionTransformer(cfg)
+    k = int(splits[0].split(".")[1])
+    stages = vit.split_stages(model, k)
+    mb, cnt = 4, 2
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(mb * cnt, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
+    y = torch.randint(0, cfg.num_classes, (mb * cnt,), generator=g)
+    crit = nn.CrossEntropyLoss()
+    times = []
+    for _ in range(2):  # first pass warms the allocator and the thread pool
+        t0 = time.perf_counter()
+        run_pipeline_step(stages, lambda o, t: crit(o, t), x, y, cnt, device_cnt=device_cnt)
+        times.append(time.perf_counter() - t0)
+    sps = mb * cnt / times[-1]
+    return dict(value=round(sps, 3), unit="samples/s", cores=cores, kind="port",
+                sample="%s fp32 on CPU: %d micro-batches x %d samples, %d stages, forward+backward+grad-accumulate "
+                       "(no optimizer step), oracle stage executor; %.1f s" % (cfg_name, cnt, mb, len(stages),
+                                                                                  times[-1]))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="vit_l16_fp16", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-roofline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs every pipeline stage on ONE GPU; --gpus %d is not supported "
+              "(no collectives, no second device)." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda", 0)
+    runner, batch, info = build_workload(args.workload, device)
+    log("[bench] workload", args.workload, "building stage programs (first step) ...")
+    t0 = time.perf_counter()
+    losses = runner.step(*batch)
+    torch.cuda.synchronize()
+    log("[bench] first step %.1f s, losses %s" % (time.perf_counter() - t0, [round(float(l), 4) for l in losses]))
+    log("[bench]", runner.worker.memory_report())
+    for _ in range(max(0, args.warmup - 1)):
+        runner.step(*batch)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        losses = runner.step(*batch)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = 1e3 * dt / args.steps
+    samples = info["batch"]
+    value = samples * args.steps / dt
+    log("[bench] %.2f ms/step, %.1f samples/s, last losses %s" % (ms, value, [round(float(l), 4) for l in losses]))
+
+    roof, per_variant = (None, {}) if args.no_roofline else gemm_roofline(runner, info["mixed"])
+    for k, v in sorted(per_variant.items(), key=lambda kv: -kv[1]["ms_per_step"]):
+        log("[bench] %-46s %4d launches/step %8.3f ms/step %8.1f us/launch %7.1f TFLOP/s"
+            % (k, v["launches_per_step"], v["ms_per_step"], v["avg_launch_us"], v["tflops"]))
+    hbm = None if args.no_roofline else hbm_kernel_rates(runner)
+    if hbm:
+        log("[bench] grad-accumulate: %.1f GB/s (%.1f%% of %d)" % (hbm["achieved"], 100 * hbm["frac"], PEAK_HBM_GBS))
+    cpu = None
+    if not args.no_cpu_baseline:
+        log("[bench] timing the CPU baseline ...")
+        cpu = cpu_baseline(args.workload)
+        log("[bench] cpu baseline", cpu)
+
+    cfg = info["cfg"]
+    flops_step = None
+    if info["family"] == "vit":
+        T, d, ff, L = cfg.tokens, cfg.dim, cfg.mlp_dim, cfg.depth
+        per_block = 2 * T * d * 3 * d + 2 * T * d * d + 4 * T * d * ff + 4 * T * T * d
+        patch = 2 * (T - 1) * (cfg.channels * cfg.patch_size ** 2) * d
+        flops_step = 3.0 * samples * (L * per_block + patch + 2 * d * cfg.num_classes)
+    rec = {
+        "metric": "train samples/sec on 1 MI355X; MFMA util % (GEMMs), HBM GB/s % (elementwise)",
+        "value": round(value, 2),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": info["mixed"] or "fp32",
+        "data": "synthetic (images ~N(0,1), labels uniform int, random-init weights, seed 42)",
+        "config": {"workload": "%s: %s micro-batch %d x %d, %d stages split at %s, schedule drawn for %d ranks, "
+                               "all stages on one GPU, CE loss, Adam" % (
+                                   args.workload, type(cfg).__name__, samples // info["batch_cnt"], info["batch_cnt"],
+                                   len(info["splits"]) + 1, info["splits"], info["device_cnt"]),
+                   "global_batch": samples, "batch_cnt": info["batch_cnt"]},
+        "roofline": roof,
+        "hbm_kernel": hbm,
+        "cpu_baseline": cpu,
+        "model_tflops": None if flops_step is None else round(flops_step / (ms * 1e-3) / 1e12, 2),
+    }
+    print(json.dumps(rec), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -114,6 +114,11 @@ typedef struct pf_gemm_desc {
 } pf_gemm_desc;
 
 int pf_gemm(const pf_gemm_desc* desc, void* stream);
+/* Name of the kernel instantiation pf_gemm would launch for `desc`, spelled the
+ * way a profiler prints it (e.g. "gemm16_kernel<1, 128, 128, false, false>":
+ * dtype, tile M, tile N, a_trans, b_trans).  Lets a harness attribute measured
+ * kernel time to problem shapes.  No counterpart in the reference. */
+int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap);
 
 /* ---- normalisation (HBM-bound, one wavefront per row) ---------------------
  * LayerNorm over the last dimension d of a [rows, d] matrix; gamma/beta are

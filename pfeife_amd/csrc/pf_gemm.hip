@@ -349,17 +349,27 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
   return PF_OK;
 }
 
+// Tile choice: the largest tile that still yields at least ~one workgroup per
+// CU (256 CUs); small problems (attention heads, narrow projections) take
+// smaller tiles so the launch fills the chip.  tile = 0: 256x128, 1: 128x128,
+// 2: 128x64, 3: 64x64.
+int choose_tile(const pf_gemm_desc& d) {
+  const int64_t nb = (d.batch1 > 0 ? d.batch1 : 1) * (d.batch2 > 0 ? d.batch2 : 1);
+  auto tiles = [&](int bm, int bn) { return ((d.M + bm - 1) / bm) * ((d.N + bn - 1) / bn) * nb; };
+  if (tiles(256, 128) >= 512 && d.M >= 256) return 0;
+  if (tiles(128, 128) >= 256 && d.M >= 128 && d.N >= 128) return 1;
+  if (tiles(128, 64) >= 256 && d.M >= 128) return 2;
+  return 3;
+}
+
 template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
-  // Tile choice: the largest tile that still yields at least ~one workgroup per
-  // CU (256 CUs); small problems (attention heads, narrow projections) take
-  // smaller tiles so the launch fills the chip.
-  const int64_t nb = d.batch1 * d.batch2;
-  auto tiles = [&](int bm, int bn) { return ((d.M + bm - 1) / bm) * ((d.N + bn - 1) / bn) * nb; };
-  if (tiles(256, 128) >= 512 && d.M >= 256) return launch16<DT, 256, 128>(d, st);
-  if (tiles(128, 128) >= 256 && d.M >= 128 && d.N >= 128) return launch16<DT, 128, 128>(d, st);
-  if (tiles(128, 64) >= 256 && d.M >= 128) return launch16<DT, 128, 64>(d, st);
-  return launch16<DT, 64, 64>(d, st);
+  switch (choose_tile(d)) {
+    case 0: return launch16<DT, 256, 128>(d, st);
+    case 1: return launch16<DT, 128, 128>(d, st);
+    case 2: return launch16<DT, 128, 64>(d, st);
+    default: return launch16<DT, 64, 64>(d, st);
+  }
 }
 
 }  // namespace
@@ -407,4 +417,16 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
              "pf_gemm: batch strides of 16-bit operands must be multiples of 8");
   if (d.in_dtype == PF_F16) return dispatch16<PF_F16>(d, st);
   return dispatch16<PF_BF16>(d, st);
+}
+
+extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
+  PF_REQUIRE(desc && out && cap > 0, "pf_gemm_variant: bad arguments");
+  static const char* tile_names[4] = {"256, 128", "128, 128", "128, 64", "64, 64"};
+  if (desc->in_dtype == PF_F32) {
+    snprintf(out, (size_t)cap, "gemm32_kernel");
+  } else {
+    snprintf(out, (size_t)cap, "gemm16_kernel<%d, %s, %s, %s>", desc->in_dtype, tile_names[choose_tile(*desc)],
+             desc->a_trans ? "true" : "false", desc->b_trans ? "true" : "false");
+  }
+  return PF_OK;
 }

@@ -1,0 +1,1349 @@
+"""Turns one pipeline-stage FX graph into prepared HIP launch lists.
+
+This module occupies the seam where the reference calls the stage submodule
+(`self.mods[node.idx](*inputs)`, pfeife/mp/worker.py:1457-1494) and
+`torch.autograd.backward` (pfeife/mp/worker.py:1585-1587): instead of running
+ATen kernels under autograd, the stage graph is lowered ONCE per (stage,
+micro-batch) to
+
+    program.fwd : [launch, ...]     forward kernels on preallocated buffers
+    program.bwd : [launch, ...]     hand-derived backward kernels
+
+and a step replays those lists.  Stage inputs are used in place (the reference
+clones them, worker.py:1442-1455) and the gradient of a stage input is written
+straight into the buffer the producing stage reads as its output gradient (the
+reference copies twice, worker.py:1096-1151): the handoff moves no bytes.
+
+Numerics follow torch.autocast's policy when `compute_dtype` is fp16/bf16
+(reference: `get_mp_ctx`, worker.py:675-680): matrix products take 16-bit
+operands with fp32 accumulation and give 16-bit results, normalisations,
+softmax and losses are computed in fp32, the residual stream stays fp32 and
+parameter gradients are accumulated in fp32.
+"""
+import math
+import operator
+
+import torch
+import torch.nn.functional as F
+
+from .values import Val, as_matrix, collapse_for_copy, dense_like, is_dense
+
+ACT_NONE, ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU = 0, 1, 2, 3, 4
+
+
+class Unsupported(RuntimeError):
+    """A graph node for which no HIP lowering exists. There is no eager fallback."""
+
+
+# ---------------------------------------------------------------------------
+# parameter store: fp32 masters, 16-bit shadows, fp32 gradient accumulators
+# ---------------------------------------------------------------------------
+class ParamStore:
+    def __init__(self, kernels, device):
+        self.kernels = kernels
+        self.device = device
+        self._shadow = {}      # (id(param), dtype) -> tensor
+        self._grads = {}       # id(param) -> fp32 grad tensor (== param.grad)
+        self.refresh = []      # launches: master -> shadow casts (once per step)
+        self.zero = []         # launches: zero-fill of every gradient accumulator (once per step)
+        self.params = []       # parameters that receive gradients, in first-use order
+        self._keep = []
+
+    def shadow(self, tensor, dtype):
+        if tensor.dtype == dtype:
+            return tensor
+        key = (tensor.data_ptr(), tuple(tensor.shape), tensor.dtype, dtype)
+        sh = self._shadow.get(key)
+        if sh is None:
+            sh = torch.empty(tensor.shape, dtype=dtype, device=tensor.device)
+            src = tensor.detach()
+            if not src.is_contiguous():
+                raise Unsupported("non-contiguous parameter %s" % (tuple(tensor.shape),))
+            self.refresh.append(self.kernels.cast(src, sh, src.numel()))
+            self._shadow[key] = sh
+            self._keep.append(tensor)
+        return sh
+
+    def grad(self, param):
+        g = self._grads.get(id(param))
+        if g is None:
+            if param.grad is None or param.grad.dtype != torch.float32 or not param.grad.is_contiguous():
+                param.grad = torch.zeros(param.shape, dtype=torch.float32, device=param.device)
+            g = param.grad
+            self._grads[id(param)] = g
+            self.zero.append(self.kernels.fill(g, 0.0, g.numel()))
+            self.params.append(param)
+        elif param.grad is not g:
+            # user code replaced .grad (e.g. zero_grad(set_to_none=True)); programs hold raw pointers
+            param.grad = g
+        return g
+
+    def rebind_grads(self):
+        for p in self.params:
+            g = self._grads[id(p)]
+            if p.grad is not g:
+                p.grad = g
+
+
+class BufferPool:
+    """Named scratch and per-stage backward buffers, shared wherever lifetimes cannot overlap."""
+
+    def __init__(self, device):
+        self.device = device
+        self._scratch = {}
+        self._bwd = {}
+        self.bytes = 0
+
+    def scratch(self, slot, shape, dtype):
+        key = (slot, tuple(shape), dtype)
+        t = self._scratch.get(key)
+        if t is None:
+            t = torch.empty(tuple(shape), dtype=dtype, device=self.device)
+            self._scratch[key] = t
+            self.bytes += t.numel() * t.element_size()
+        return t
+
+    def bwd_like(self, seq, like):
+        """Buffer number `seq` of a backward job.  Backward jobs never overlap in
+        time (one stream, one job at a time) and their temporaries die with the
+        job, so all stages and micro-batches share one set of buffers."""
+        key = (seq, tuple(like.shape), tuple(like.stride()), like.dtype)
+        t = self._bwd.get(key)
+        if t is None:
+            t = torch.empty_like(like, device=self.device)
+            self._bwd[key] = t
+            self.bytes += t.numel() * t.element_size()
+        return t
+
+    def fresh_like(self, like):
+        t = torch.empty_like(like, device=self.device)
+        self.bytes += t.numel() * t.element_size()
+        return t
+
+
+class StageProgram:
+    def __init__(self, stage, mb):
+        self.stage = stage
+        self.mb = mb
+        self.inputs = []       # [Val] in stage-placeholder order
+        self.outputs = []      # [Val or python constant]
+        self.fwd = []
+        self.bwd = []
+        self.backward_fns = []  # build-time closures, one per lowered node, in forward order
+        self.input_grads = []   # filled by lower_backward: gradient tensor (or None) per input
+        self.fwd_bytes = 0
+        self.tile_groups = []   # sibling regions that must all be written for the zero-fill to be skipped
+
+    def run_forward(self, stream):
+        for launch in self.fwd:
+            launch(stream)
+
+    def run_backward(self, stream):
+        for launch in self.bwd:
+            launch(stream)
+
+
+def _dtype_promote(a, b):
+    return torch.promote_types(a, b)
+
+
+# ---------------------------------------------------------------------------
+# backward build context
+# ---------------------------------------------------------------------------
+class BwdCtx:
+    def __init__(self, lowerer, program):
+        self.L = lowerer
+        self.k = lowerer.kernels
+        self.program = program
+        self.out = program.bwd
+        self._seq = 0
+        self._pending = {}
+
+    def emit(self, launch):
+        self.out.append(launch)
+
+    def new_like(self, like, private=False):
+        if private:
+            # gradients that outlive this job (they cross a stage boundary) get their own storage
+            return self.L.pool.fresh_like(like)
+        self._seq += 1
+        return self.L.pool.bwd_like(self._seq, like)
+
+    def temp(self, shape, dtype):
+        self._seq += 1
+        return self.L.pool.bwd_like(self._seq, torch.empty(tuple(shape), dtype=dtype, device="meta"))
+
+    # -- reading -------------------------------------------------------------
+    def grad_of(self, val):
+        """Accumulated gradient of `val` (None: nothing contributed, i.e. zero)."""
+        if val.kind == "base":
+            return val.grad
+        g = self.grad_of(val.base)
+        return None if g is None else val.view_fn(g)
+
+    # -- writing -------------------------------------------------------------
+    def _own_base_grad(self, val, zero_fill):
+        """Make sure `val` (kind base) has a private, writable gradient buffer."""
+        if val.param is not None:
+            return self.L.params.grad(val.param)
+        if val.grad is None:
+            val.grad = self.new_like(val.buf, val.boundary)
+            val.grad_shared = False
+            val.partial_only = True
+            if zero_fill:
+                self._zero(val.grad)
+        elif val.grad_shared:
+            fresh = self.new_like(val.buf, val.boundary)
+            self.copy(val.grad, fresh)
+            val.grad, val.grad_shared = fresh, False
+        return val.grad
+
+    def _zero(self, t):
+        if is_dense(t):
+            self.emit(self.k.fill(t, 0.0, t.numel()))
+        else:
+            raise Unsupported("zero-fill of a non-dense gradient buffer")
+
+    def _writable(self, val, zero_fill):
+        """Gradient tensor laid out like val.buf that may be written in place."""
+        if val.kind == "base":
+            return self._own_base_grad(val, zero_fill)
+        return val.view_fn(self._writable(val.base, zero_fill))
+
+    def grad_target(self, val):
+        """-> (dst, prev): write the NEW TOTAL gradient of `val` into dst; prev is the
+        total so far (None: nothing yet; `prev is dst`: accumulate in place)."""
+        if not val.req_grad:
+            raise RuntimeError("gradient requested for a value that does not require one: %r" % val)
+        if val.kind == "view":
+            dst_b, prev_b = self.grad_target(val.base)
+            self._pending[id(val)] = dst_b
+            return val.view_fn(dst_b), (None if prev_b is None else val.view_fn(prev_b))
+        if val.kind == "part":
+            parent = val.base
+            had_full = self._has_full_contribution(parent)
+            pg = self._writable(parent, zero_fill=not val.tiled)
+            region = val.view_fn(pg)
+            if val.written or had_full:
+                return region, region
+            return region, None
+        if val.param is not None:
+            g = self.L.params.grad(val.param)  # AccumulateGrad: always += into the fp32 accumulator
+            return g, g
+        if val.grad is None:
+            return self.new_like(val.buf, val.boundary), None
+        if val.grad_shared:
+            return self.new_like(val.buf, val.boundary), val.grad
+        return val.grad, val.grad
+
+    def _has_full_contribution(self, val):
+        if val.kind == "base":
+            return val.grad is not None and not val.partial_only
+        if val.kind == "view":
+            return self._has_full_contribution(val.base)
+        return val.written or self._has_full_contribution(val.base)
+
+    def commit(self, val, dst):
+        if val.param is not None:
+            return
+        if val.kind == "view":
+            self.commit(val.base, self._pending.pop(id(val)))
+        elif val.kind == "part":
+            val.written = True
+        else:
+            if val.grad is not dst:
+                val.grad, val.grad_shared = dst, False
+            val.partial_only = False
+
+    # -- generic contributions -------------------------------------------------
+    def copy(self, src, dst, accumulate=False):
+        """dst (=|+=) src for same-shape tensors of any strides / float dtypes."""
+        if src.shape != dst.shape:
+            raise RuntimeError("copy: shape mismatch %s vs %s" % (tuple(src.shape), tuple(dst.shape)))
+        if src.numel() == 0:
+            return
+        if is_dense(src) and is_dense(dst) and src.stride() == dst.stride():
+            n = src.numel()
+            if accumulate:
+                self.emit(self.k.axpby(dst, 1.0, src, 1.0, dst, n))
+            else:
+                self.emit(self.k.cast(src, dst, n))
+            return
+        sizes, ss, ds = collapse_for_copy(src.shape, src.stride(), dst.stride())
+        if len(sizes) > 6:
+            raise Unsupported("strided copy over %d dimensions" % len(sizes))
+        self.emit(self.k.copy_strided(src, ss, dst, ds, sizes, 1 if accumulate else 0))
+
+    def contribute(self, val, t):
+        """Add tensor t (val's shape, any strides/dtype) to val's gradient."""
+        if not val.req_grad:
+            return
+        if (val.kind == "base" and val.param is None and not val.boundary and val.grad is None
+                and t.dtype == val.buf.dtype and t.stride() == val.buf.stride()):
+            val.grad, val.grad_shared, val.partial_only = t, True, False  # alias, no bytes moved
+            return
+        dst, prev = self.grad_target(val)
+        if prev is None:
+            self.copy(t, dst)
+        elif prev is dst:
+            self.copy(t, dst, accumulate=True)
+        else:
+            if is_dense(t) and is_dense(prev) and t.stride() == prev.stride() == dst.stride():
+                self.emit(self.k.axpby(prev, 1.0, t, 1.0, dst, t.numel()))
+            else:
+                self.copy(prev, dst)
+                self.copy(t, dst, accumulate=True)
+        self.commit(val, dst)
+
+    def matrix_in(self, t, dtype):
+        """t as a row-major matrix of `dtype` (cast / compact into a temp when needed)."""
+        if t.dtype == dtype and as_matrix(t) is not None:
+            return t
+        tmp = self.temp(t.shape, dtype)
+        self.copy(t, tmp)
+        return tmp
+
+
+# ---------------------------------------------------------------------------
+# the lowerer
+# ---------------------------------------------------------------------------
+class Lowerer:
+    def __init__(self, kernels, device, compute_dtype=None, params=None, pool=None):
+        self.kernels = kernels
+        self.device = torch.device(device)
+        self.cd = compute_dtype or torch.float32
+        self.mixed = self.cd != torch.float32
+        self.params = params or ParamStore(kernels, self.device)
+        self.pool = pool or BufferPool(self.device)
+        self._ws = None
+
+    # -- buffers -------------------------------------------------------------
+    def alloc(self, shape, dtype):
+        t = torch.empty(tuple(int(s) for s in shape), dtype=dtype, device=self.device)
+        self.cur.fwd_bytes += t.numel() * t.element_size()
+        return t
+
+    def workspace(self, cols):
+        need = self.kernels.colreduce_workspace(0, cols)
+        if self._ws is None or self._ws.numel() < need:
+            if self._ws is not None:
+                raise RuntimeError("column-reduction workspace grew after launches were prepared")
+            self._ws = torch.empty(max(need, 2 * 512 * 32768), dtype=torch.float32, device=self.device)
+        return self._ws
+
+    def emit(self, launch):
+        self.cur.fwd.append(launch)
+
+    # -- entry points ----------------------------------------------------------
+    def lower_forward(self, part_node, mb, input_vals):
+        """Build the forward launch list of one stage for one micro-batch.
+        `input_vals` are the Vals (or constants) bound to the stage placeholders."""
+        prog = StageProgram(part_node.idx, mb)
+        self.cur = prog
+        gm = part_node.graph_module
+        self.env = {}
+        self.fused = {}
+        placeholders = [n for n in gm.graph.nodes if n.op == "placeholder"]
+        if len(placeholders) != len(input_vals):
+            raise RuntimeError("stage %d expects %d inputs, got %d" % (part_node.idx, len(placeholders), len(input_vals)))
+        for n, v in zip(placeholders, input_vals):
+            self.env[n] = v
+            if isinstance(v, Val):
+                v.name = v.name or n.name
+        prog.inputs = list(input_vals)
+        for node in gm.graph.nodes:
+            if node.op == "placeholder":
+                continue
+            if node.op == "output":
+                res = node.args[0]
+                outs = list(res) if isinstance(res, (tuple, list)) else [res]
+                prog.outputs = [self.arg(o) for o in outs]
+                continue
+            if node in self.fused:
+                self.env[node] = self.fused[node]
+                continue
+            handler = self._handler(node)
+            out = handler(self, node)
+            self.env[node] = out
+            if isinstance(out, Val) and not out.name:
+                out.name = node.name
+        self.cur = None
+        return prog
+
+    def lower_backward(self, prog, output_grads):
+        """Build the backward launch list.  `output_grads[i]` is the (preallocated)
+        gradient tensor of prog.outputs[i] or None; the tensors are only read."""
+        B = BwdCtx(self, prog)
+        for v, gs in zip(prog.outputs, output_grads):
+            if gs is None or not isinstance(v, Val) or not v.req_grad:
+                continue
+            for g in ([gs] if torch.is_tensor(gs) else gs):  # several consumers: fan-out sum
+                B.contribute(v, g)
+        for fn in reversed(prog.backward_fns):
+            fn(B)
+        prog.input_grads = []
+        for v in prog.inputs:
+            if isinstance(v, Val) and v.req_grad and v.param is None:
+                prog.input_grads.append(B.grad_of(v))
+            else:
+                prog.input_grads.append(None)
+        for group in prog.tile_groups:
+            w = [p.written for p in group]
+            if any(w) and not all(w):
+                raise RuntimeError("stage %d: a split/unbind piece received no gradient while its siblings did; "
+                                   "the unwritten region would hold garbage" % prog.stage)
+        prog.backward_fns = []  # closures keep build-time state alive; not needed any more
+        return prog
+
+    # -- helpers for handlers ----------------------------------------------------
+    def arg(self, a):
+        if isinstance(a, torch.fx.Node):
+            return self.env[a]
+        if isinstance(a, (tuple, list)):
+            return type(a)(self.arg(x) for x in a)
+        return a
+
+    def add_backward(self, fn):
+        self.cur.backward_fns.append(fn)
+
+    def _handler(self, node):
+        if node.op == "call_function":
+            h = FUNCTION_HANDLERS.get(node.target)
+            if h is None:
+                h = FUNCTION_HANDLERS.get(getattr(node.target, "__name__", None))
+        elif node.op == "call_method":
+            h = METHOD_HANDLERS.get(node.target)
+        else:
+            h = None
+        if h is None:
+            raise Unsupported("no HIP lowering for graph node %s (target %s)" % (node.format_node(), node.target))
+        return h
+
+    def sole_user(self, node):
+        if len(node.users) != 1:
+            return None
+        return next(iter(node.users))
+
+    def matrix_in(self, t, dtype):
+        """Forward-side: t as a matrix of dtype, materialising a saved copy when needed."""
+        if t.dtype == dtype and as_matrix(t) is not None:
+            return t
+        tmp = self.alloc(t.shape, dtype)
+        self.copy(t, tmp)
+        return tmp
+
+    def copy(self, src, dst):
+        if src.numel() == 0:
+            return
+        if is_dense(src) and is_dense(dst) and src.stride() == dst.stride():
+            self.emit(self.kernels.cast(src, dst, src.numel()))
+            return
+        sizes, ss, ds = collapse_for_copy(src.shape, src.stride(), dst.stride())
+        if len(sizes) > 6:
+            raise Unsupported("strided copy over %d dimensions" % len(sizes))
+        self.emit(self.kernels.copy_strided(src, ss, dst, ds, sizes, 0))
+
+    def consumers_cast_to_cd(self, node):
+        """True when every user of `node` is an op that autocast would feed 16-bit inputs."""
+        if not self.mixed or not node.users:
+            return False
+        for u in node.users:
+            if u.op == "call_function" and u.target in CAST_TO_CD_TARGETS:
+                continue
+            return False
+        return True
+
+
+# ---------------------------------------------------------------------------
+# handlers
+# ---------------------------------------------------------------------------
+def _kw(node, idx, name, default=None):
+    if len(node.args) > idx:
+        return node.args[idx]
+    return node.kwargs.get(name, default)
+
+
+def _act_of_node(n):
+    """(act code) if node n is a supported unary activation, else None."""
+    if n.op != "call_function":
+        return None
+    t = n.target
+    if t in (F.gelu, torch._C._nn.gelu):
+        approx = n.kwargs.get("approximate", "none")
+        return ACT_GELU_TANH if approx == "tanh" else ACT_GELU
+    if t in (F.silu,):
+        return ACT_SILU
+    if t in (F.relu, torch.relu):
+        return ACT_RELU
+    return None
+
+
+def _is_add_node(n):
+    return n.op == "call_function" and n.target in (operator.add, operator.iadd, torch.add)
+
+
+def lower_linear(L, node):
+    x = L.arg(node.args[0])
+    w = L.arg(node.args[1])
+    b = L.arg(_kw(node, 2, "bias"))
+    cd = L.cd
+    K = x.shape[-1]
+    N = w.shape[0]
+    if w.shape[1] != K:
+        raise RuntimeError("linear: weight %s does not match input %s" % (w.shape, x.shape))
+    xm = L.matrix_in(x.buf, cd)
+    M, _, lda = as_matrix(xm)
+    w_cd = L.params.shadow(w.buf, cd) if w.param is not None or not w.req_grad else None
+    if w_cd is None:
+        raise Unsupported("linear with a non-parameter weight that requires grad")
+    if not w_cd.is_contiguous():
+        raise Unsupported("linear with a non-contiguous weight")
+    b_cd = None if b is None else L.params.shadow(b.buf, cd)
+
+    # fusions: linear -> activation, or linear -> (+ residual)
+    act, res, out_node = ACT_NONE, None, node
+    user = L.sole_user(node)
+    if user is not None:
+        a = _act_of_node(user)
+        if a is not None and user.args[0] is node:
+            act, out_node = a, user
+        elif _is_add_node(user) and not user.kwargs:
+            other = user.args[1] if user.args[0] is node else user.args[0]
+            if isinstance(other, torch.fx.Node) and other in L.env and isinstance(L.env[other], Val):
+                ov = L.env[other]
+                if ov.shape == tuple(x.shape[:-1]) + (N,) and as_matrix(ov.buf) is not None \
+                        and ov.dtype.is_floating_point:
+                    res, out_node = ov, user
+    out_shape = tuple(x.shape[:-1]) + (N,)
+    out_dtype = cd if res is None else _dtype_promote(cd, res.dtype)
+    out = L.alloc(out_shape, out_dtype)
+    h = L.alloc(out_shape, cd) if act != ACT_NONE else None
+    kw = dict(M=M, N=N, K=K, lda=lda, ldb=K, ldc=N, bias=b_cd, round_mid=1 if L.mixed else 0)
+    if act != ACT_NONE:
+        kw.update(aux_out=h, ld_aux_out=N, act=act)
+    if res is not None:
+        kw.update(residual=res.buf, ld_res=as_matrix(res.buf)[2])
+    L.emit(L.kernels.gemm(xm, w_cd, out, **kw))
+    req = x.req_grad or w.req_grad or (b is not None and b.req_grad) or (res is not None and res.req_grad)
+    outv = Val(out, req_grad=req, name=out_node.name)
+    if act != ACT_NONE:
+        outv.preact = (act, h)
+    if out_node is not node:
+        L.fused[out_node] = outv
+    x_users = len(node.args[0].users) if isinstance(node.args[0], torch.fx.Node) else 0
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        if res is not None:
+            B.contribute(res, g)
+        if act != ACT_NONE and not outv.grad_is_preact:
+            gm_ = B.matrix_in(g, cd)
+            dy = B.temp(out_shape, cd)
+            if not (gm_.is_contiguous() and h.is_contiguous()):
+                raise Unsupported("activation backward on non-contiguous gradient")
+            B.emit(B.k.act_bwd(gm_, h, dy, act, dy.numel()))
+        else:
+            dy = B.matrix_in(g, cd)
+        _, _, ld_dy = as_matrix(dy)
+        if w.req_grad and w.param is not None:
+            B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
+                            b_trans=1, beta=1))
+        if b is not None and b.req_grad and b.param is not None:
+            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(N)))
+        if x.req_grad:
+            dst, prev = B.grad_target(x)
+            dm = as_matrix(dst)
+            kw2 = dict(M=M, N=K, K=N, lda=ld_dy, ldb=K, b_trans=1)
+            if x.preact is not None and x_users == 1 and prev is None:
+                kw2.update(dact=x.preact[0], aux_in=x.preact[1], ld_aux_in=K)
+                x.grad_is_preact = True
+            if dm is not None:
+                if prev is dst:
+                    kw2["beta"] = 1
+                elif prev is not None:
+                    pm = as_matrix(prev)
+                    if pm is None:
+                        raise Unsupported("accumulating into a non-matrix gradient")
+                    kw2.update(residual=prev, ld_res=pm[2])
+                B.emit(B.k.gemm(dy, w_cd, dst, ldc=dm[2], **kw2))
+                B.commit(x, dst)
+            else:
+                # target is not a plain matrix (e.g. a permuted view): go through a temp
+                tmp = B.temp(tuple(x.shape), x.dtype)
+                B.emit(B.k.gemm(dy, w_cd, tmp, ldc=K, **kw2))
+                if prev is None:
+                    B.copy(tmp, dst)
+                elif prev is dst:
+                    B.copy(tmp, dst, accumulate=True)
+                else:
+                    B.copy(prev, dst)
+                    B.copy(tmp, dst, accumulate=True)
+                B.commit(x, dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv if out_node is node else outv
+
+
+def lower_layer_norm(L, node, rms=False):
+    x = L.arg(node.args[0])
+    shape = _kw(node, 1, "normalized_shape")
+    gamma = L.arg(_kw(node, 2, "weight"))
+    if rms:
+        beta = None
+        eps = _kw(node, 3, "eps", None)
+        if eps is None:
+            eps = torch.finfo(torch.float32).eps
+    else:
+        beta = L.arg(_kw(node, 3, "bias"))
+        eps = _kw(node, 4, "eps", 1e-5)
+    if len(tuple(shape)) != 1 or shape[0] != x.shape[-1]:
+        raise Unsupported("normalisation over other than the last dimension: %s" % (shape,))
+    if gamma is None:
+        raise Unsupported("normalisation without a weight")
+    d = x.shape[-1]
+    if not x.buf.is_contiguous():
+        raise Unsupported("normalisation of a non-contiguous input")
+    rows = x.buf.numel() // d
+    y_dtype = L.cd if L.consumers_cast_to_cd(node) else (torch.float32 if L.mixed else x.dtype)
+    y = L.alloc(x.shape, y_dtype)
+    rstd = L.alloc((rows,), torch.float32)
+    g32 = gamma.buf if gamma.dtype == torch.float32 else L.params.shadow(gamma.buf, torch.float32)
+    if rms:
+        mean = None
+        L.emit(L.kernels.rmsnorm_fwd(x.buf, g32, y, rstd, rows, d, float(eps)))
+    else:
+        mean = L.alloc((rows,), torch.float32)
+        b32 = None if beta is None else (beta.buf if beta.dtype == torch.float32 else L.params.shadow(beta.buf, torch.float32))
+        L.emit(L.kernels.layernorm_fwd(x.buf, g32, b32, y, mean, rstd, rows, d, float(eps)))
+    req = x.req_grad or gamma.req_grad or (beta is not None and beta.req_grad)
+    outv = Val(y, req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        if not g.is_contiguous():
+            t = B.temp(g.shape, g.dtype)
+            B.copy(g, t)
+            g = t
+        dgamma = L.params.grad(gamma.param) if gamma.req_grad and gamma.param is not None else None
+        dbeta = L.params.grad(beta.param) if beta is not None and beta.req_grad and beta.param is not None else None
+        ws = L.workspace(d) if (dgamma is not None or dbeta is not None) else None
+        if x.req_grad:
+            dst, prev = B.grad_target(x)
+            if not dst.is_contiguous() or (prev is not None and not prev.is_contiguous()):
+                raise Unsupported("normalisation backward into a non-contiguous gradient")
+        else:
+            dst, prev = B.temp(x.shape, x.dtype), None
+        if rms:
+            B.emit(B.k.rmsnorm_bwd(g, x.buf, g32, rstd, prev, dst, dgamma, ws, rows, d))
+        else:
+            B.emit(B.k.layernorm_bwd(g, x.buf, g32, mean, rstd, prev, dst, dgamma, dbeta, ws, rows, d))
+        if x.req_grad:
+            B.commit(x, dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_rms_norm(L, node):
+    return lower_layer_norm(L, node, rms=True)
+
+
+def lower_sdpa(L, node):
+    q, k, v = (L.arg(a) for a in node.args[:3])
+    mask = _kw(node, 3, "attn_mask")
+    drop = _kw(node, 4, "dropout_p", 0.0)
+    causal = bool(_kw(node, 5, "is_causal", False))
+    scale = _kw(node, 6, "scale", None)
+    if mask is not None:
+        raise Unsupported("scaled_dot_product_attention with an explicit mask")
+    if drop:
+        raise Unsupported("attention dropout")
+    if node.kwargs.get("enable_gqa"):
+        raise Unsupported("grouped-query attention")
+    cd = L.cd
+    if q.buf.dim() != 4:
+        raise Unsupported("attention on %d-d tensors" % q.buf.dim())
+    Bn, H, Tq, hd = q.shape
+    Tk = k.shape[2]
+    if k.shape != (Bn, H, Tk, hd) or v.shape[:3] != (Bn, H, Tk):
+        raise Unsupported("attention with mismatched head layout %s %s %s" % (q.shape, k.shape, v.shape))
+    hv = v.shape[3]
+    scale = float(scale) if scale is not None else 1.0 / math.sqrt(hd)
+    Tkp = (Tk + 7) // 8 * 8
+
+    def head_tensor(val):
+        t = val.buf
+        if t.dtype != cd or t.stride(3) != 1 or any(s % 8 for s in t.stride()[:3] if cd != torch.float32):
+            c = L.alloc(t.shape, cd)
+            L.copy(t, c)
+            return c
+        return t
+
+    qt, kt, vt = head_tensor(q), head_tensor(k), head_tensor(v)
+    S = L.pool.scratch("attn_s", (Bn, H, Tq, Tkp), torch.float32)
+    P = L.alloc((Bn, H, Tq, Tkp), cd)
+    O = L.alloc((Bn, Tq, H, hv), cd)           # token-major, so that transpose(1,2).reshape is a view
+    Ov = O.permute(0, 2, 1, 3)
+    bs = lambda t: (t.stride(0), t.stride(1))
+    kern = L.kernels
+    L.emit(kern.gemm(qt, kt, S, M=Tq, N=Tk, K=hd, lda=qt.stride(2), ldb=kt.stride(2), ldc=Tkp, batch=(Bn, H),
+                     sa=bs(qt), sb=bs(kt), sc=bs(S), alpha=scale))
+    L.emit(kern.softmax_fwd(S, Tkp, P, Tkp, Bn * H * Tq, Tk, Tq, 1 if causal else 0))
+    L.emit(kern.gemm(P, vt, Ov, M=Tq, N=hv, K=Tk, lda=Tkp, ldb=vt.stride(2), ldc=Ov.stride(2), b_trans=1,
+                     batch=(Bn, H), sa=bs(P), sb=bs(vt), sc=bs(Ov)))
+    req = q.req_grad or k.req_grad or v.req_grad
+    outv = Val(Ov, req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        if g.dtype != cd or g.stride(3) != 1:
+            t = B.new_like(Ov)
+            B.copy(g, t)
+            g = t
+        dP = L.pool.scratch("attn_dp", (Bn, H, Tq, Tkp), torch.float32)
+        dS = L.pool.scratch("attn_ds", (Bn, H, Tq, Tkp), cd)
+        kb = B.k
+        B.emit(kb.gemm(g, vt, dP, M=Tq, N=Tk, K=hv, lda=g.stride(2), ldb=vt.stride(2), ldc=Tkp, batch=(Bn, H),
+                       sa=bs(g), sb=bs(vt), sc=bs(dP)))
+        B.emit(kb.softmax_bwd(dP, Tkp, P, Tkp, dS, Tkp, Bn * H * Tq, Tk, scale))
+
+        def into(val, emit_fn, like_t):
+            if not val.req_grad:
+                return
+            dst, prev = B.grad_target(val)
+            direct = dst.dtype == cd and dst.stride(3) == 1 and (prev is None or prev is dst)
+            if direct:
+                emit_fn(dst, 1 if prev is dst else 0)
+                B.commit(val, dst)
+            else:
+                tmp = B.temp(val.shape, cd)
+                emit_fn(tmp, 0)
+                if prev is None:
+                    B.copy(tmp, dst)
+                elif prev is dst:
+                    B.copy(tmp, dst, accumulate=True)
+                else:
+                    B.copy(prev, dst)
+                    B.copy(tmp, dst, accumulate=True)
+                B.commit(val, dst)
+
+        # dQ = dS K ; dK = dS^T Q ; dV = P^T dO
+        into(q, lambda dst, beta: B.emit(kb.gemm(dS, kt, dst, M=Tq, N=hd, K=Tk, lda=Tkp, ldb=kt.stride(2),
+                                                  ldc=dst.stride(2), b_trans=1, batch=(Bn, H), sa=bs(dS), sb=bs(kt),
+                                                  sc=bs(dst), beta=beta)), qt)
+        into(k, lambda dst, beta: B.emit(kb.gemm(dS, qt, dst, M=Tk, N=hd, K=Tq, lda=Tkp, ldb=qt.stride(2),
+                                                  ldc=dst.stride(2), a_trans=1, b_trans=1, batch=(Bn, H), sa=bs(dS),
+                                                  sb=bs(qt), sc=bs(dst), beta=beta)), kt)
+        into(v, lambda dst, beta: B.emit(kb.gemm(P, g, dst, M=Tk, N=hv, K=Tq, lda=Tkp, ldb=g.stride(2),
+                                                  ldc=dst.stride(2), a_trans=1, b_trans=1, batch=(Bn, H), sa=bs(P),
+                                                  sb=bs(g), sc=bs(dst), beta=beta)), vt)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_conv2d(L, node):
+    x = L.arg(node.args[0])
+    w = L.arg(node.args[1])
+    b = L.arg(_kw(node, 2, "bias"))
+    stride = _kw(node, 3, "stride", (1, 1))
+    padding = _kw(node, 4, "padding", (0, 0))
+    dilation = _kw(node, 5, "dilation", (1, 1))
+    groups = _kw(node, 6, "groups", 1)
+    pair = lambda v: (v, v) if isinstance(v, int) else tuple(v)
+    stride, padding, dilation = pair(stride), pair(padding), pair(dilation)
+    O, C, kh, kw_ = w.shape
+    if groups != 1 or dilation != (1, 1) or padding != (0, 0) or stride != (kh, kw_):
+        raise Unsupported("conv2d other than a non-overlapping patch projection (kernel == stride, no padding)")
+    Bn, Cx, H, W = x.shape
+    if Cx != C or H % kh or W % kw_:
+        raise Unsupported("conv2d patch projection with ragged image size")
+    Hp, Wp = H // kh, W // kw_
+    cd = L.cd
+    cols = L.alloc((Bn * Hp * Wp, C * kh * kw_), cd)
+    xs = x.buf.stride()
+    src_strides = (xs[0], xs[2] * kh, xs[3] * kw_, xs[1], xs[2], xs[3])
+    sizes = (Bn, Hp, Wp, C, kh, kw_)
+    cview = cols.view(Bn, Hp, Wp, C, kh, kw_)
+    s2, ss2, ds2 = collapse_for_copy(sizes, src_strides, cview.stride())
+    L.emit(L.kernels.copy_strided(x.buf, ss2, cols, ds2, s2, 0))
+    M, K, N = Bn * Hp * Wp, C * kh * kw_, O
+    w_cd = L.params.shadow(w.buf, cd)
+    b_cd = None if b is None else L.params.shadow(b.buf, cd)
+    out = L.alloc((Bn, Hp, Wp, O), cd)
+    L.emit(L.kernels.gemm(cols, w_cd, out, M=M, N=N, K=K, lda=K, ldb=K, ldc=N, bias=b_cd,
+                          round_mid=1 if L.mixed else 0))
+    req = x.req_grad or w.req_grad or (b is not None and b.req_grad)
+    outv = Val(out.permute(0, 3, 1, 2), req_grad=req)   # logical NCHW, channels-last memory
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        gm_ = g.permute(0, 2, 3, 1)
+        dy = B.matrix_in(gm_, cd)
+        _, _, ld_dy = as_matrix(dy)
+        if w.req_grad and w.param is not None:
+            B.emit(B.k.gemm(dy, cols, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
+                            b_trans=1, beta=1))
+        if b is not None and b.req_grad and b.param is not None:
+            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(N)))
+        if x.req_grad:
+            dcols = B.temp((M, K), cd)
+            B.emit(B.k.gemm(dy, w_cd, dcols, M=M, N=K, K=N, lda=ld_dy, ldb=K, ldc=K, b_trans=1))
+            dst, prev = B.grad_target(x)
+            dview = torch.as_strided(dst, sizes, tuple(
+                s * m for s, m in zip((dst.stride(0), dst.stride(2), dst.stride(3), dst.stride(1), dst.stride(2),
+                                       dst.stride(3)), (1, kh, kw_, 1, 1, 1))), dst.storage_offset())
+            if prev is not None and prev is not dst:
+                B.copy(prev, dst)
+            B.copy(dcols.view(sizes), dview, accumulate=prev is not None)
+            B.commit(x, dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def _view_handler(fn_of_node):
+    """Builds a handler for an op that is a pure view of its first argument."""
+
+    def handler(L, node):
+        x = L.arg(node.args[0])
+        if not isinstance(x, Val):
+            raise Unsupported("view of a non-tensor: %s" % node.format_node())
+        fn = fn_of_node(L, node)
+        out = fn(x.buf)
+        if out.untyped_storage().data_ptr() != x.buf.untyped_storage().data_ptr():
+            # the op had to copy (reshape of a non-viewable layout): materialise with the copy kernel
+            shape = tuple(out.shape)
+            dense = L.alloc(x.shape, x.dtype)
+            L.copy(x.buf, dense)
+            outbuf = dense.view(shape)
+            outv = Val(outbuf, req_grad=x.req_grad)
+
+            def bwd(B):
+                g = B.grad_of(outv)
+                if g is not None:
+                    B.contribute(x, g.reshape(x.shape) if g.is_contiguous() else _compact(B, g).view(x.shape))
+
+            if x.req_grad:
+                L.add_backward(bwd)
+            return outv
+        return Val(out, req_grad=x.req_grad, kind="view", base=x, view_fn=fn)
+
+    return handler
+
+
+def _compact(B, g):
+    t = B.temp(g.shape, g.dtype)
+    B.copy(g, t)
+    return t
+
+
+def _shape_args(L, node):
+    a = [L.arg(v) for v in node.args[1:]]
+    if len(a) == 1 and isinstance(a[0], (tuple, list, torch.Size)):
+        a = list(a[0])
+    return tuple(int(v) for v in a)
+
+
+lower_reshape = _view_handler(lambda L, n: (lambda t, s=_shape_args(L, n): t.reshape(s)))
+lower_view = _view_handler(lambda L, n: (lambda t, s=_shape_args(L, n): t.view(s)))
+lower_permute = _view_handler(lambda L, n: (lambda t, s=_shape_args(L, n): t.permute(s)))
+lower_transpose = _view_handler(lambda L, n: (lambda t, a=int(n.args[1]), b=int(n.args[2]): t.transpose(a, b)))
+lower_flatten = _view_handler(
+    lambda L, n: (lambda t, a=int(_kw(n, 1, "start_dim", 0)), b=int(_kw(n, 2, "end_dim", -1)): t.flatten(a, b)))
+lower_unsqueeze = _view_handler(lambda L, n: (lambda t, d=int(n.args[1]): t.unsqueeze(d)))
+lower_squeeze = _view_handler(
+    lambda L, n: (lambda t, d=(n.args[1] if len(n.args) > 1 else None): t.squeeze() if d is None else t.squeeze(d)))
+
+
+def lower_contiguous(L, node):
+    x = L.arg(node.args[0])
+    if x.buf.is_contiguous():
+        return Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
+    dense = L.alloc(x.shape, x.dtype)
+    L.copy(x.buf, dense)
+    outv = Val(dense, req_grad=x.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is not None:
+            B.contribute(x, g)
+
+    if x.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def _chain_single_user(node):
+    """True when node and the chain of view nodes above it each have exactly one user."""
+    n = node
+    while isinstance(n, torch.fx.Node) and n.op in ("call_method", "call_function"):
+        if len(n.users) != 1:
+            return False
+        name = n.target if n.op == "call_method" else getattr(n.target, "__name__", "")
+        if name not in ("reshape", "view", "permute", "transpose", "flatten", "unsqueeze", "squeeze"):
+            return True
+        n = n.args[0]
+    return True
+
+
+def lower_unbind(L, node):
+    x = L.arg(node.args[0])
+    dim = int(_kw(node, 1, "dim", 0))
+    n = x.shape[dim]
+    all_used = len(node.users) == n and all(
+        u.op == "call_function" and u.target is operator.getitem and len(u.users) > 0 for u in node.users)
+    tiled = all_used and _chain_single_user(node.args[0]) and len(node.args[0].users) == 1
+    parts = []
+    for i in range(n):
+        fn = (lambda t, i=i: t.select(dim, i))
+        p = Val(fn(x.buf), req_grad=x.req_grad, kind="part", base=x, view_fn=fn)
+        p.tiled = tiled
+        parts.append(p)
+    if tiled:
+        L.cur.tile_groups.append(parts)
+    return parts
+
+
+def lower_split_like(L, node, pieces_fn):
+    x = L.arg(node.args[0])
+    bufs = pieces_fn(x.buf)
+    n_total = sum(1 for _ in bufs)
+    all_used = len(node.users) == n_total and all(
+        u.op == "call_function" and u.target is operator.getitem and len(u.users) > 0 for u in node.users)
+    tiled = all_used and _chain_single_user(node.args[0]) and len(node.args[0].users) == 1
+    parts = []
+    for i in range(n_total):
+        fn = (lambda t, i=i: pieces_fn(t)[i])
+        p = Val(bufs[i], req_grad=x.req_grad, kind="part", base=x, view_fn=fn)
+        p.tiled = tiled
+        parts.append(p)
+    if tiled:
+        L.cur.tile_groups.append(parts)
+    return parts
+
+
+def lower_chunk(L, node):
+    n = int(node.args[1])
+    dim = int(_kw(node, 2, "dim", 0))
+    return lower_split_like(L, node, lambda t: t.chunk(n, dim))
+
+
+def lower_split(L, node):
+    sz = node.args[1]
+    dim = int(_kw(node, 2, "dim", 0))
+    return lower_split_like(L, node, lambda t: t.split(sz, dim))
+
+
+def lower_getitem(L, node):
+    src = L.arg(node.args[0])
+    idx = node.args[1]
+    if isinstance(src, (list, tuple)):
+        return src[idx]
+    if not isinstance(src, Val):
+        raise Unsupported("getitem on %s" % type(src))
+    idx_t = idx if isinstance(idx, tuple) else (idx,)
+    for i in idx_t:
+        if not (isinstance(i, (int, slice)) or i is None or i is Ellipsis):
+            raise Unsupported("advanced indexing is not lowered: %s" % (idx,))
+    fn = (lambda t, idx=idx: t[idx])
+    out = fn(src.buf)
+    full = out.numel() == src.buf.numel()
+    return Val(out, req_grad=src.req_grad, kind="view" if full else "part", base=src, view_fn=fn)
+
+
+def lower_expand(L, node):
+    x = L.arg(node.args[0])
+    sizes = _shape_args(L, node)
+    out = x.buf.expand(*sizes)
+    if out.numel() == x.buf.numel():
+        return Val(out, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t.expand(*sizes))
+    # broadcasting view; its gradient is a sum over the expanded (leading) dimensions
+    lead = out.dim() - x.buf.dim()
+    exp_dims = [i for i in range(out.dim()) if i < lead or (x.buf.shape[i - lead] == 1 and out.shape[i] != 1)]
+    inner_start = max(exp_dims) + 1
+    if exp_dims != list(range(inner_start)) and any(out.shape[i] != 1 for i in range(inner_start) if i not in exp_dims):
+        raise Unsupported("expand over non-leading dimensions: %s -> %s" % (x.shape, sizes))
+    outv = Val(out, req_grad=x.req_grad)
+    rows = 1
+    for i in range(inner_start):
+        rows *= out.shape[i]
+    cols = out.numel() // rows
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        gc = B.matrix_in(g.reshape(rows, cols) if g.is_contiguous() else _compact(B, g).view(rows, cols), torch.float32)
+        dst, prev = B.grad_target(x)
+        if dst.dtype != torch.float32 or not dst.is_contiguous():
+            raise Unsupported("expand backward into a non-fp32 gradient")
+        if prev is None:
+            B.emit(B.k.fill(dst, 0.0, dst.numel()))
+        elif prev is not dst:
+            B.copy(prev, dst)
+        B.emit(B.k.colsum_accumulate(gc, rows, cols, as_matrix(gc)[2], dst, L.workspace(cols)))
+        B.commit(x, dst)
+
+    if x.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_cat(L, node):
+    tensors = L.arg(node.args[0])
+    dim = int(_kw(node, 1, "dim", 0))
+    vals = [t for t in tensors]
+    dt = vals[0].dtype
+    for v in vals[1:]:
+        dt = _dtype_promote(dt, v.dtype)
+    shape = list(vals[0].shape)
+    if dim < 0:
+        dim += len(shape)
+    shape[dim] = sum(v.shape[dim] for v in vals)
+    out = L.alloc(shape, dt)
+    off = 0
+    regions = []
+    for v in vals:
+        n = v.shape[dim]
+        region = out.narrow(dim, off, n)
+        L.copy(v.buf, region)
+        regions.append((off, n))
+        off += n
+    req = any(v.req_grad for v in vals)
+    outv = Val(out, req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        for v, (o, n) in zip(vals, regions):
+            if v.req_grad:
+                B.contribute(v, g.narrow(dim, o, n))
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_add(L, node):
+    a, b = L.arg(node.args[0]), L.arg(node.args[1])
+    alpha = node.kwargs.get("alpha", 1)
+    if alpha != 1:
+        raise Unsupported("add with alpha")
+    if not isinstance(a, Val) or not isinstance(b, Val):
+        raise Unsupported("add of a tensor and a python scalar")
+    if b.buf.numel() > a.buf.numel():
+        a, b = b, a
+    out_dtype = _dtype_promote(a.dtype, b.dtype)
+    req = a.req_grad or b.req_grad
+    if a.shape == b.shape:
+        if not (is_dense(a.buf) and is_dense(b.buf) and a.buf.stride() == b.buf.stride()):
+            raise Unsupported("add of differently laid out tensors")
+        out = torch.empty_like(a.buf, dtype=out_dtype)
+        L.cur.fwd_bytes += out.numel() * out.element_size()
+        L.emit(L.kernels.axpby(a.buf, 1.0, b.buf, 1.0, out, out.numel()))
+        outv = Val(out, req_grad=req)
+
+        def bwd(B):
+            g = B.grad_of(outv)
+            if g is None:
+                return
+            B.contribute(a, g)
+            B.contribute(b, g)
+
+        if req:
+            L.add_backward(bwd)
+        return outv
+    # broadcast of b over the leading dimensions of a
+    bshape = tuple(b.shape)
+    while bshape and bshape[0] == 1:
+        bshape = bshape[1:]
+    if tuple(a.shape[len(a.shape) - len(bshape):]) != bshape or not a.buf.is_contiguous() or not b.buf.is_contiguous():
+        raise Unsupported("add with general broadcasting %s + %s" % (a.shape, b.shape))
+    n, blen = a.buf.numel(), b.buf.numel()
+    out = L.alloc(a.shape, out_dtype)
+    L.emit(L.kernels.bias_add(a.buf, b.buf, out, n, blen))
+    outv = Val(out, req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        B.contribute(a, g)
+        if b.req_grad:
+            gc = g if g.is_contiguous() else _compact(B, g)
+            dst, prev = B.grad_target(b)
+            if dst.dtype != torch.float32 or not dst.is_contiguous():
+                raise Unsupported("broadcast-add backward into a non-fp32 gradient")
+            if prev is None:
+                B.emit(B.k.fill(dst, 0.0, dst.numel()))
+            elif prev is not dst:
+                B.copy(prev, dst)
+            B.emit(B.k.colsum_accumulate(gc, n // blen, blen, blen, dst, L.workspace(blen)))
+            B.commit(b, dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_unary_act(L, node):
+    act = _act_of_node(node)
+    x = L.arg(node.args[0])
+    if not x.buf.is_contiguous():
+        raise Unsupported("activation on a non-contiguous tensor")
+    y = L.alloc(x.shape, x.dtype)
+    L.emit(L.kernels.act_fwd(x.buf, y, act, y.numel()))
+    outv = Val(y, req_grad=x.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        gc = g if (g.is_contiguous() and g.dtype == x.dtype) else _compact(B, g)
+        dst, prev = B.grad_target(x)
+        if prev is None and dst.is_contiguous():
+            B.emit(B.k.act_bwd(gc, x.buf, dst, act, y.numel()))
+        else:
+            tmp = B.temp(x.shape, x.dtype)
+            B.emit(B.k.act_bwd(gc, x.buf, tmp, act, y.numel()))
+            if prev is None:
+                B.copy(tmp, dst)
+            elif prev is dst:
+                B.copy(tmp, dst, accumulate=True)
+            else:
+                B.copy(prev, dst)
+                B.copy(tmp, dst, accumulate=True)
+        B.commit(x, dst)
+
+    if x.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_dropout(L, node):
+    p = _kw(node, 1, "p", 0.5)
+    training = _kw(node, 2, "training", True)
+    if p and training:
+        raise Unsupported("dropout with p > 0 in training mode")
+    x = L.arg(node.args[0])
+    return Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
+
+
+def lower_cross_entropy(L, node):
+    logits = L.arg(node.args[0])
+    target = L.arg(node.args[1])
+    if _kw(node, 2, "weight") is not None or node.kwargs.get("label_smoothing", 0.0):
+        raise Unsupported("weighted / label-smoothed cross entropy")
+    ignore_index = int(node.kwargs.get("ignore_index", -100))
+    if node.kwargs.get("reduction", "mean") != "mean":
+        raise Unsupported("cross entropy with reduction other than mean")
+    if logits.buf.dim() != 2 or not logits.buf.is_contiguous() or target.dtype != torch.int64:
+        raise Unsupported("cross entropy expects contiguous [rows, classes] logits and int64 targets")
+    rows, classes = logits.shape
+    tgt = target.buf if target.buf.is_contiguous() else None
+    if tgt is None:
+        raise Unsupported("non-contiguous cross entropy targets")
+    row_loss = L.alloc((rows,), torch.float32)
+    row_lse = L.alloc((rows,), torch.float32)
+    loss2 = L.alloc((2,), torch.float32)
+    L.emit(L.kernels.cross_entropy_fwd(logits.buf, tgt, row_loss, row_lse, loss2, rows, classes, ignore_index))
+    outv = Val(loss2[0], req_grad=logits.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        if g.dtype != torch.float32:
+            raise Unsupported("loss gradient must be fp32")
+        dst, prev = B.grad_target(logits)
+        if prev is not None or not dst.is_contiguous():
+            raise Unsupported("cross entropy backward into an already written gradient")
+        B.emit(B.k.cross_entropy_bwd(logits.buf, tgt, row_lse, g, loss2, dst, rows, classes, ignore_index))
+        B.commit(logits, dst)
+
+    if logits.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_float(L, node):
+    """x.float() / x.to(float32): under the mixed-precision policy a no-op for fp32 values,
+    a cast kernel otherwise."""
+    x = L.arg(node.args[0])
+    return _lower_cast(L, x, torch.float32)
+
+
+def _lower_cast(L, x, dtype):
+    if x.dtype == dtype:
+        return Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
+    out = torch.empty_like(x.buf, dtype=dtype) if is_dense(x.buf) else L.alloc(x.shape, dtype)
+    L.copy(x.buf, out)
+    outv = Val(out, req_grad=x.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is not None:
+            B.contribute(x, g)
+
+    if x.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_to(L, node):
+    x = L.arg(node.args[0])
+    dtype = node.kwargs.get("dtype")
+    for a in node.args[1:]:
+        if isinstance(a, torch.dtype):
+            dtype = a
+    if dtype is None:
+        return Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
+    return _lower_cast(L, x, dtype)
+
+
+def lower_embedding(L, node):
+    ids = L.arg(node.args[0])
+    table = L.arg(node.args[1])
+    if _kw(node, 2, "padding_idx") is not None and False:
+        raise Unsupported("embedding with padding_idx")
+    if ids.dtype != torch.int64 or not ids.buf.is_contiguous() or not table.buf.is_contiguous():
+        raise Unsupported("embedding expects contiguous int64 ids")
+    vocab, dim = table.shape
+    n = ids.buf.numel()
+    out_dtype = table.dtype  # autocast leaves embedding outputs in the table's dtype (fp32 residual stream)
+    out = L.alloc(tuple(ids.shape) + (dim,), out_dtype)
+    L.emit(L.kernels.embedding_fwd(table.buf, ids.buf, out, n, dim, vocab))
+    outv = Val(out, req_grad=table.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None or table.param is None:
+            return
+        gc = g if g.is_contiguous() else _compact(B, g)
+        B.emit(B.k.embedding_bwd(gc, ids.buf, L.params.grad(table.param), n, dim, vocab))
+
+    if table.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_mul(L, node):
+    a, b = L.arg(node.args[0]), L.arg(node.args[1])
+    if isinstance(a, Val) and isinstance(b, Val):
+        # gated MLP: act(gate) * up, with the activation node fused here
+        for gate_v, up_v, gate_n in ((a, b, node.args[0]), (b, a, node.args[1])):
+            info = gate_v.pending_act
+            if info is not None and len(gate_n.users) == 1 and gate_v.shape == up_v.shape:
+                act, gsrc = info
+                return _lower_glu(L, gsrc, up_v, act)
+        raise Unsupported("elementwise tensor*tensor outside the gated-MLP pattern")
+    v, s = (a, b) if isinstance(a, Val) else (b, a)
+    if not isinstance(v, Val) or not isinstance(s, (int, float)):
+        raise Unsupported("mul operands %s" % (node.format_node(),))
+    if not is_dense(v.buf):
+        raise Unsupported("scaling a non-dense tensor")
+    out = torch.empty_like(v.buf)
+    L.cur.fwd_bytes += out.numel() * out.element_size()
+    L.emit(L.kernels.axpby(v.buf, float(s), None, 0.0, out, out.numel()))
+    outv = Val(out, req_grad=v.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        gc = g if is_dense(g) and g.stride() == v.buf.stride() else _compact(B, g)
+        t = B.new_like(v.buf)
+        B.emit(B.k.axpby(gc, float(s), None, 0.0, t, t.numel()))
+        B.contribute(v, t)
+
+    if v.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
+def _lower_glu(L, gate, up, act):
+    rows_cols = as_matrix(gate.buf), as_matrix(up.buf)
+    if rows_cols[0] is None or rows_cols[1] is None or gate.dtype != up.dtype:
+        raise Unsupported("gated MLP on non-matrix operands")
+    rows, cols, ldg = rows_cols[0]
+    _, _, ldu = rows_cols[1]
+    y = L.alloc(gate.shape, gate.dtype)
+    L.emit(L.kernels.glu_fwd(gate.buf, ldg, up.buf, ldu, y, cols, act, rows, cols))
+    req = gate.req_grad or up.req_grad
+    outv = Val(y, req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        gc = B.matrix_in(g, gate.dtype)
+        dg_dst, dg_prev = B.grad_target(gate)
+        du_dst, du_prev = B.grad_target(up)
+        mg, mu = as_matrix(dg_dst), as_matrix(du_dst)
+        if dg_prev is not None or du_prev is not None or mg is None or mu is None:
+            raise Unsupported("gated MLP backward into already written / non-matrix gradients")
+        B.emit(B.k.glu_bwd(gc, as_matrix(gc)[2], gate.buf, ldg, up.buf, ldu, dg_dst, mg[2], du_dst, mu[2], act, rows,
+                           cols))
+        B.commit(gate, dg_dst)
+        B.commit(up, du_dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_act_maybe_gate(L, node):
+    """silu/gelu whose single user is a tensor*tensor product is the gate of a gated MLP:
+    defer it to the product so that one kernel computes act(gate) * up."""
+    user = L.sole_user(node)
+    x = L.arg(node.args[0])
+    if (user is not None and user.op == "call_function" and user.target in (operator.mul, torch.mul)
+            and all(isinstance(a, torch.fx.Node) for a in user.args[:2])):
+        v = Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
+        v.pending_act = (_act_of_node(node), x)
+        return v
+    return lower_unary_act(L, node)
+
+
+FUNCTION_HANDLERS = {
+    F.linear: lower_linear, torch._C._nn.linear: lower_linear,
+    F.layer_norm: lower_layer_norm, torch.layer_norm: lower_layer_norm,
+    F.rms_norm: lower_rms_norm,
+    F.scaled_dot_product_attention: lower_sdpa, torch._C._nn.scaled_dot_product_attention: lower_sdpa,
+    F.conv2d: lower_conv2d, torch.conv2d: lower_conv2d,
+    F.gelu: lower_act_maybe_gate, torch._C._nn.gelu: lower_act_maybe_gate,
+    F.silu: lower_act_maybe_gate,
+    F.relu: lower_unary_act, torch.relu: lower_unary_act,
+    F.dropout: lower_dropout,
+    F.cross_entropy: lower_cross_entropy,
+    F.embedding: lower_embedding,
+    operator.add: lower_add, operator.iadd: lower_add, torch.add: lower_add,
+    operator.mul: lower_mul, torch.mul: lower_mul,
+    operator.getitem: lower_getitem,
+    torch.cat: lower_cat,
+    torch.flatten: lower_flatten, torch.transpose: lower_transpose, torch.permute: lower_permute,
+    torch.reshape: lower_reshape, torch.unsqueeze: lower_unsqueeze, torch.squeeze: lower_squeeze,
+    torch.unbind: lower_unbind, torch.chunk: lower_chunk, torch.split: lower_split,
+}
+METHOD_HANDLERS = {
+    "reshape": lower_reshape, "view": lower_view, "permute": lower_permute, "transpose": lower_transpose,
+    "flatten": lower_flatten, "unsqueeze": lower_unsqueeze, "squeeze": lower_squeeze,
+    "contiguous": lower_contiguous, "unbind": lower_unbind, "chunk": lower_chunk, "split": lower_split,
+    "expand": lower_expand, "float": lower_float, "to": lower_to, "add": lower_add, "mul": lower_mul,
+}
+CAST_TO_CD_TARGETS = {F.linear, torch._C._nn.linear, F.conv2d, torch.conv2d,
+                      F.scaled_dot_product_attention, torch._C._nn.scaled_dot_product_attention, torch.matmul}

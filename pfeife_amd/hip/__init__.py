@@ -66,6 +66,7 @@ _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
     "pf_init": [_I],
     "pf_gemm": [POINTER(GemmDesc), _P],
+    "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
     "pf_layernorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _F, _P],
     "pf_layernorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P],
     "pf_rmsnorm_fwd": [_P, _I, _P, _P, _I, _P, _L, _L, _F, _P],
@@ -210,7 +211,12 @@ class HipKernels:
         for t in (aux_out, aux_in):
             if t is not None and t.dtype != a.dtype:
                 raise RuntimeError("gemm: aux tensors must have the operand dtype")
-        return self._prep("pf_gemm", (byref(d),), (d, a, b, c, bias, aux_out, aux_in, residual))
+        launch = self._prep("pf_gemm", (byref(d),), (d, a, b, c, bias, aux_out, aux_in, residual))
+        name = ctypes.create_string_buffer(96)
+        self.lib.pf_gemm_variant(byref(d), name, 96)
+        launch.variant = name.value.decode()
+        launch.flops = 2.0 * M * N * K * batch[0] * batch[1]
+        return launch
 
     # -- normalisation -----------------------------------------------------------
     def layernorm_fwd(self, x, gamma, beta, y, mean, rstd, rows, d, eps):

@@ -1,0 +1,292 @@
+"""Public front-end: `PartialRunner`, `PartialModule`, `partial_compiler`.
+
+Same contract as pfeife/mp/partial/module.py:37-438:
+
+    runner = PartialRunner(option, optimizer)
+    model = torch.compile(model, backend=partial_compiler)
+    runner.set_exec_fn(fn)            # fn(*micro_batch) calls model, computes a loss, calls loss.backward()
+    losses = runner.step(*batch)      # list of fn's return values, one per micro-batch, in order
+
+`step` splits the batch (pfeife/batch.py), runs `fn` once per micro-batch on a
+helper thread that parks inside the compiled model until the schedule has
+produced that micro-batch's outputs (module.py:161-166, 417-433), and executes
+the stage jobs on the calling thread in the schedule's order.  Exactly one
+thread is runnable at any time, as in the reference (module.py:87-89, 145-159).
+
+What differs: the first `step` does not profile the model.  The probe call of
+`fn` (module.py:168-170) only records the captured graph and the micro-batch's
+input signature, builds the stage programs, and hands `fn` zero-valued outputs
+of the right shape so that user code can run through its loss once; like the
+reference's probe it contributes nothing to the gradients.
+"""
+import threading
+from functools import partial
+from queue import Queue
+from typing import List
+
+import torch
+import torch.fx as fx
+import torch.nn as nn
+
+from ...batch import split_args_kwargs
+from ...executor.values import Val
+from ...graph.partition_graph import compute_nodes, partition_by_split_points
+from ...option import PipeOption
+from ...utils import get_logger, to_device
+from ..net_states import get_state
+from ..worker import StageWorker
+
+STEP_TOKEN = "###<<STEP_TOKEN>>###"
+
+
+class _ExecError:
+    def __init__(self, exc):
+        self.exc = exc
+
+
+class PartialRunner:
+    def __init__(self, option: PipeOption = None, optimizer=None, kernels=None):
+        """`kernels` is for tests of the host logic only (a kernel table double);
+        user code never passes it and the HIP table is the only one shipped."""
+        self.option = option if option is not None else PipeOption()
+        self.optimizer = optimizer
+        self.exec_fn = None
+        self.net_state = get_state()
+        self._compiled = False
+        self._probing = False
+        self._train_queues = [Queue() for _ in range(self.option.batch_cnt)]
+        self._return_queues = [Queue() for _ in range(self.option.batch_cnt)]
+        self._batch_threads = []
+        self.results = []
+        self.worker = StageWorker(self, self.option, self.net_state.device, kernels)
+        PartialModule.set_runner(self)
+        for i in range(self.option.batch_cnt):
+            t = threading.Thread(target=self._exec_loop, args=(i,), daemon=True, name="pfeife-mb%d" % i)
+            self._batch_threads.append(t)
+            t.start()
+
+    def set_exec_fn(self, exec_fn):
+        self.exec_fn = exec_fn
+
+    # -- one optimisation step ---------------------------------------------------
+    def step(self, *args, **kwargs):
+        if self.exec_fn is None:
+            raise RuntimeError("call set_exec_fn() before step()")
+        option = self.option
+        args, kwargs = split_args_kwargs(args, kwargs, option.batch_cnt)
+
+        if not self._compiled:
+            self._probe_forward(args[0], kwargs[0])
+            if option.print_graph:
+                print("Found %d graphs in the main module" % len(PartialModule._all_modules))
+
+        self.reset()
+        pp = PartialModule._pp_modules[0] if PartialModule._pp_modules else None
+        worker = self.worker
+        self.results = []
+
+        # every micro-batch thread runs user code up to the compiled model, hands its
+        # inputs to the worker and parks there
+        for bid in range(option.batch_cnt):
+            self._train_queues[bid].put((args[bid], kwargs[bid]))
+            tok = self._return_queues[bid].get()
+            if isinstance(tok, _ExecError):
+                raise tok.exc
+            if tok is not STEP_TOKEN:
+                # exec_fn returned without reaching a pipelined graph: nothing to schedule for it
+                self.results.append(tok)
+                if pp is not None:
+                    raise RuntimeError("exec_fn finished without calling the compiled model")
+
+        if pp is None:
+            return self._take_results()
+
+        worker.begin_step()
+        for i, (stage, mb, is_fwd) in enumerate(worker.order):
+            worker.run_job(stage, mb, is_fwd)
+            if is_fwd and worker.last_forward.get(i) == mb:
+                self.finalize_output(mb)
+        worker.optimizer_step()
+        return self._take_results()
+
+    def _take_results(self):
+        results, self.results = self.results, []
+        return results
+
+    def finalize_output(self, batch_idx):
+        """Wake micro-batch `batch_idx`: its outputs exist; wait until its exec_fn has
+        returned (loss computed, backward hooks fired)."""
+        PartialModule._module_queues[batch_idx].put(None)
+        ret = self._return_queues[batch_idx].get()
+        if isinstance(ret, _ExecError):
+            raise ret.exc
+        self.worker.finish_micro_batch(batch_idx)
+        self.results.append(ret)
+
+    def backward_hook(self, batch_idx, output_idx, grad):
+        self.worker.recv_loss_grad(batch_idx, output_idx, grad)
+
+    def reset(self):
+        for pm in PartialModule._all_modules:
+            pm.reset()
+
+    def gather_params(self):
+        """Parameters never leave the user's module on a single GPU; kept for API parity
+        (module.py:115-117)."""
+        return None
+
+    def log_memory_usage(self):
+        get_logger().info(self.worker.memory_report())
+
+    def train(self):
+        pass
+
+    def eval(self):
+        pass
+
+    # -- helpers --------------------------------------------------------------------
+    def _exec_loop(self, batch_idx):
+        q = self._train_queues[batch_idx]
+        while True:
+            args, kwargs = q.get()
+            try:
+                if self.net_state.device.type == "cuda":
+                    torch.cuda.set_device(self.net_state.device)
+                ret = self.exec_fn(*args, **kwargs)
+            except BaseException as e:  # surfaced on the thread that called step()
+                ret = _ExecError(e)
+            self._return_queues[batch_idx].put(ret)
+
+    def _probe_forward(self, args, kwargs):
+        self._probing = True
+        try:
+            self.exec_fn(*args, **kwargs)
+        finally:
+            self._probing = False
+        self._compiled = True
+        self.worker.init_optimizer(self.optimizer)
+
+
+class PartialModule(nn.Module):
+    _module_queues: List[Queue] = []
+    _runner: PartialRunner = None
+    _all_modules: List["PartialModule"] = []
+    _pp_modules: List["PartialModule"] = []
+    _option: PipeOption = None
+
+    def __init__(self, gm: fx.GraphModule, example_inputs=None):
+        super().__init__()
+        self.gm = gm
+        self.example_inputs = list(example_inputs) if example_inputs is not None else None
+        self.curr_batch = 0
+        self.net_state = get_state()
+        self.device = self.net_state.device
+        self.probed = False
+        n_compute = len(compute_nodes(gm))
+        has_params = any(isinstance(e, nn.Parameter) for e in (self.example_inputs or []))
+        can_pp = all(not m.should_pp for m in self._all_modules)
+        # pipeline the first captured graph that has real work in it (reference: node-count test,
+        # module.py:205-216)
+        self.should_pp = can_pp and n_compute >= 2 * self.net_state.pp_size and has_params
+        if self._option is not None and self._option.print_graph:
+            print("================ GRAPH %d: %d nodes / PP enabled: %s ================"
+                  % (len(self._all_modules) + 1, len(gm.graph.nodes), self.should_pp))
+            gm.graph.print_tabular()
+        self.partition_graph = None
+        self._all_modules.append(self)
+
+    @staticmethod
+    def set_runner(runner: PartialRunner):
+        PartialModule._runner = runner
+        PartialModule._option = runner.option
+        PartialModule._module_queues = [Queue() for _ in range(runner.option.batch_cnt)]
+        PartialModule._all_modules = []
+        PartialModule._pp_modules = []
+
+    def reset(self):
+        self.curr_batch = 0
+
+    # -- compilation --------------------------------------------------------------------
+    def _compile(self, args):
+        option = self._option
+        worker = self._runner.worker
+        ex = self.example_inputs if self.example_inputs is not None else list(args)
+        # module state is identified on the real call arguments (they are the live tensors)
+        live = list(args)
+        self.partition_graph = partition_by_split_points(self.gm, live, option.split_points, option.device_cnt)
+        if option.print_graph:
+            for idx, st in self.partition_graph.nodes.items():
+                print("================ PARTITION GRAPH %d: %d nodes ================"
+                      % (idx, len(st.graph_module.graph.nodes)))
+                st.graph_module.graph.print_tabular()
+        worker.set_partition_graph(self.partition_graph, live)
+        self._pp_modules.append(self)
+        del ex
+
+    def _dynamic_inputs(self, args):
+        pg = self.partition_graph
+        return {i: (to_device(a, self.device) if not torch.is_tensor(a) else a)
+                for i, a in enumerate(args) if not pg.static_placeholder[i]}
+
+    def _ensure_programs(self, mb, args):
+        worker = self._runner.worker
+        dyn = self._dynamic_inputs(args)
+        sig = worker._signature([dyn[i] for i in sorted(dyn)])
+        slot = worker.mbs.get(mb)
+        if slot is None or slot.input_sig != sig:
+            worker.build_micro_batch(mb, dyn)
+        return dyn
+
+    def _outputs_for_user(self, mb, probe):
+        worker = self._runner.worker
+        slot = worker.mbs[mb]
+        outs = []
+        for oi, v in enumerate(slot.outputs):
+            if isinstance(v, Val):
+                if probe:
+                    t = torch.zeros_like(v.buf)
+                else:
+                    t = v.buf.detach()
+                if v.req_grad:
+                    t.requires_grad_()
+                    if not probe:
+                        t.register_hook(partial(self._runner.backward_hook, mb, oi))
+                outs.append(t)
+            else:
+                outs.append(v)
+        spec = self.partition_graph.output_spec
+        if spec == "single":
+            return outs[0]
+        return tuple(outs) if spec == "tuple" else outs
+
+    # -- call ----------------------------------------------------------------------------
+    def forward(self, *args):
+        if not self.should_pp:
+            return self.gm(*to_device(args, self.device))
+        runner = self._runner
+        if runner._probing:
+            if self.partition_graph is None:
+                self._compile(args)
+            self._ensure_programs(0, args)
+            return self._outputs_for_user(0, probe=True)
+        if self.partition_graph is None:
+            raise RuntimeError("the compiled model was called outside PartialRunner.step()")
+
+        mb = self.curr_batch
+        self.curr_batch += 1
+        if mb >= self._option.batch_cnt:
+            raise RuntimeError("the compiled model was called more than batch_cnt times in one step")
+        dyn = self._ensure_programs(mb, args)
+        worker = runner.worker
+        for i, v in dyn.items():
+            if torch.is_tensor(v):
+                worker.distribute_input(mb, i, v)
+        runner._return_queues[mb].put(STEP_TOKEN)   # inputs are in place; main thread may schedule
+        self._module_queues[mb].get()               # parked until this micro-batch's outputs exist
+        return self._outputs_for_user(mb, probe=False)
+
+
+def partial_compiler(gm: fx.GraphModule, example_inputs: List[torch.Tensor]):
+    if PartialModule._runner is None:
+        raise RuntimeError("create a PartialRunner before the compiled model is first called")
+    return PartialModule(gm, example_inputs)

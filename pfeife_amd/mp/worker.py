@@ -1,0 +1,257 @@
+"""Single-GPU stage worker: owns the stage programs and runs the job loop of a step.
+
+Counterpart of `ProcessWorker` in pfeife/mp/worker.py for one rank that holds
+every stage:
+  * `set_partition_graph`  (worker.py:682-758): here it lowers each (stage,
+    micro-batch) to prepared launch lists on preallocated buffers instead of
+    allocating per-edge copy buffers;
+  * `distribute_input`     (worker.py:818-840): micro-batch slab -> stage input
+    buffer through the split/gather kernel (or one H2D copy for host tensors);
+  * `run_with_module`      (worker.py:912-940) + `_handle_job_with_comm`
+    (:978-1006): the schedule's jobs in one serial order;
+  * `send_same_node`       (worker.py:1096-1151): nothing to do, a stage reads its
+    producer's output buffer and writes the gradient buffer its producer reads;
+  * `_init_optimizer` / `optimizer_step` (worker.py:583-597, 1432-1436).
+"""
+import torch
+
+from ..executor.lowering import BufferPool, Lowerer, ParamStore
+from ..executor.values import Val
+from ..option import get_optimizer_cls
+from ..schedule.scheduler import PipeSchedParams, SingleCommScheduler, StepWork, serialize_ranks
+from ..utils import fmem, get_logger
+
+
+class MicroBatchPrograms:
+    """Everything that was built for one micro-batch slot."""
+
+    def __init__(self):
+        self.stage_programs = {}   # stage -> StageProgram
+        self.input_buffers = {}    # graph placeholder index -> static device buffer
+        self.input_sig = None      # shapes/dtypes the programs were built for
+        self.outputs = []          # per graph output: Val | python constant
+        self.loss_grads = {}       # graph output index -> static gradient buffer
+        self.grad_seen = set()
+
+
+class StageWorker:
+    def __init__(self, runner, option, device, kernels=None):
+        self.runner = runner
+        self.option = option
+        self.device = torch.device(device)
+        if kernels is None:
+            from ..hip import HipKernels  # raises when the library or the GPU is missing
+
+            kernels = HipKernels(self.device.index)
+        self.kernels = kernels
+        self.log = get_logger()
+        self.params = ParamStore(kernels, self.device)
+        self.pool = BufferPool(self.device)
+        self.lowerer = Lowerer(kernels, self.device, option.mixed_precision, self.params, self.pool)
+        self.part_graph = None
+        self.static_inputs = {}
+        self.mbs = {}
+        self.order = []
+        self.optimizer = None
+        self.mem_usage_info = {}
+
+    # -- graph ---------------------------------------------------------------------
+    def set_partition_graph(self, part_graph, example_inputs):
+        self.part_graph = pg = part_graph
+        self.static_inputs = {}
+        for i, (is_static, ex) in enumerate(zip(pg.static_placeholder, example_inputs)):
+            if not is_static:
+                continue
+            if ex.device != self.device:
+                ex.data = ex.data.to(self.device)  # stage parameters live on the worker's device
+            param = ex if isinstance(ex, torch.nn.Parameter) else None
+            self.static_inputs[i] = Val(ex.detach(), req_grad=bool(ex.requires_grad), param=param,
+                                        name=pg.placeholder_names[i])
+        node_cnt = len(pg.nodes)
+        opt = self.option
+        device_cnt = max(1, min(opt.device_cnt, node_cnt))
+        loop_batch = opt.loop_batch if opt.loop_batch is not None else device_cnt
+        loop_batch = max(1, min(loop_batch, opt.batch_cnt))
+        prefetch = opt.prefetch_fwd if opt.prefetch_fwd is not None else 0
+        for st in pg.nodes.values():
+            st.rank = st.idx % device_cnt
+        self.sched_params = PipeSchedParams(device_cnt, opt.batch_cnt, node_cnt, loop_batch, prefetch)
+        self.scheduler = SingleCommScheduler(self.sched_params)
+        self.order = serialize_ranks(self.sched_params.rank_works, node_cnt)
+        last = {}
+        for i, (stage, mb, is_fwd) in enumerate(self.order):
+            if is_fwd:
+                last[mb] = i
+        self.last_forward = {i: mb for mb, i in last.items()}
+
+    def stage_parameters(self):
+        seen, out = set(), []
+        for v in self.static_inputs.values():
+            if v.param is not None and id(v.param) not in seen:
+                seen.add(id(v.param))
+                out.append(v.param)
+        return out
+
+    @staticmethod
+    def _signature(values):
+        sig = []
+        for v in values:
+            if torch.is_tensor(v):
+                sig.append((tuple(v.shape), v.dtype))
+            else:
+                sig.append(("const", repr(v)))
+        return tuple(sig)
+
+    def build_micro_batch(self, mb, dynamic_inputs):
+        """Lower every stage for micro-batch slot `mb`; `dynamic_inputs` maps graph
+        placeholder index -> the value user code passed (tensor chunk or constant)."""
+        pg = self.part_graph
+        slot = MicroBatchPrograms()
+        slot.input_sig = self._signature([dynamic_inputs[i] for i in sorted(dynamic_inputs)])
+        graph_vals = {}
+        for i, v in dynamic_inputs.items():
+            if torch.is_tensor(v):
+                buf = torch.empty(v.shape, dtype=v.dtype, device=self.device)
+                slot.input_buffers[i] = buf
+                graph_vals[i] = Val(buf, req_grad=False, name=pg.placeholder_names[i])
+            else:
+                graph_vals[i] = v
+        for i, v in self.static_inputs.items():
+            graph_vals[i] = v
+        L = self.lowerer
+        stage_out = {}
+        for sid in sorted(pg.nodes):
+            st = pg.nodes[sid]
+            ins = []
+            for k, name in enumerate(st.inputs):
+                gi = st.input_placeholder[k]
+                if gi >= 0:
+                    ins.append(graph_vals[gi])
+                else:
+                    src_stage, oi = st.input_source[k]
+                    pv = stage_out[src_stage][oi]
+                    if isinstance(pv, Val):
+                        bv = Val(pv.buf, req_grad=pv.req_grad, name=name)  # same storage: the handoff is a pointer
+                        bv.boundary = True
+                        ins.append(bv)
+                    else:
+                        ins.append(pv)
+            prog = L.lower_forward(st, mb, ins)
+            slot.stage_programs[sid] = prog
+            stage_out[sid] = prog.outputs
+        # graph outputs and the buffers their loss gradients arrive in
+        for oi, ref in enumerate(pg.outputs):
+            if ref[0] == "const":
+                slot.outputs.append(ref[1])
+            elif ref[0] == "input":
+                slot.outputs.append(graph_vals[ref[1]])
+            else:
+                v = stage_out[ref[0]][ref[1]]
+                slot.outputs.append(v)
+                if isinstance(v, Val) and v.req_grad:
+                    slot.loss_grads[oi] = torch.zeros_like(v.buf)
+        # backward, last stage first: a stage's output gradients are its consumers' input gradients
+        for sid in sorted(pg.nodes, reverse=True):
+            st = pg.nodes[sid]
+            prog = slot.stage_programs[sid]
+            out_grads = [[] for _ in st.outputs]
+            for tid in sorted(pg.nodes):
+                if tid <= sid:
+                    continue
+                tst = pg.nodes[tid]
+                tprog = slot.stage_programs[tid]
+                for k, src in enumerate(tst.input_source):
+                    if src is not None and src[0] == sid and tprog.input_grads[k] is not None:
+                        out_grads[src[1]].append(tprog.input_grads[k])
+            for oi, ref in enumerate(pg.outputs):
+                if ref[0] == sid and oi in slot.loss_grads:
+                    out_grads[ref[1]].append(slot.loss_grads[oi])
+            L.lower_backward(prog, out_grads)
+        self.mbs[mb] = slot
+        return slot
+
+    # -- per step --------------------------------------------------------------------
+    def stream(self):
+        if self.device.type == "cuda":
+            return torch.cuda.current_stream(self.device).cuda_stream
+        return None
+
+    def distribute_input(self, mb, placeholder_idx, value):
+        """Copy one micro-batch slab into the stage input buffer it was built for."""
+        slot = self.mbs[mb]
+        buf = slot.input_buffers.get(placeholder_idx)
+        if buf is None:
+            return
+        if value.device == buf.device and value.is_contiguous() and value.numel() > 0:
+            rows = value.shape[0] if value.dim() > 0 else 1
+            row_bytes = value.numel() * value.element_size() // max(rows, 1)
+            self.kernels.split_gather(value, buf, row_bytes, 0, rows)(self.stream())
+        elif value.numel() > 0:
+            buf.copy_(value, non_blocking=True)  # host -> device (or a layout change): PyTorch plumbing
+
+    def begin_step(self):
+        s = self.stream()
+        self.params.rebind_grads()
+        for launch in self.params.zero:      # optimizer.zero_grad(set_to_none=False)
+            launch(s)
+        for launch in self.params.refresh:   # one master -> 16-bit cast per step, not per micro-batch
+            launch(s)
+        for slot in self.mbs.values():
+            slot.grad_seen.clear()
+
+    def recv_loss_grad(self, mb, out_idx, grad):
+        slot = self.mbs[mb]
+        buf = slot.loss_grads.get(out_idx)
+        if buf is None:
+            return
+        slot.grad_seen.add(out_idx)
+        if grad is None:
+            return
+        g = grad.detach()
+        if g.shape != buf.shape:
+            raise RuntimeError("loss gradient of output %d has shape %s, expected %s"
+                               % (out_idx, tuple(g.shape), tuple(buf.shape)))
+        if g.device == buf.device and g.is_contiguous() and buf.is_contiguous() and g.dtype.is_floating_point:
+            self.kernels.cast(g, buf, g.numel())(self.stream())
+        else:
+            buf.copy_(g)
+
+    def finish_micro_batch(self, mb):
+        """Outputs whose hook never fired: zero gradient, except scalars which get 1
+        (the implicit gradient the reference keeps, worker.py:1568-1573)."""
+        slot = self.mbs[mb]
+        for oi, buf in slot.loss_grads.items():
+            if oi not in slot.grad_seen:
+                self.kernels.fill(buf, 1.0 if buf.dim() == 0 else 0.0, buf.numel())(self.stream())
+
+    def run_job(self, stage, mb, is_fwd):
+        prog = self.mbs[mb].stage_programs[stage]
+        if is_fwd:
+            prog.run_forward(self.stream())
+        else:
+            prog.run_backward(self.stream())
+
+    def init_optimizer(self, optimizer):
+        if optimizer is not None:
+            self.optimizer = optimizer
+        elif self.optimizer is None:
+            params = [p for p in self.stage_parameters() if p.requires_grad]
+            if params:
+                cls = get_optimizer_cls(self.option.optimizer_type)
+                self.optimizer = cls(params, **self.option.optimizer_kwargs)
+
+    def optimizer_step(self):
+        if self.optimizer is not None:
+            self.optimizer.step()
+
+    # -- reporting -----------------------------------------------------------------------
+    def memory_report(self):
+        fwd = sum(p.fwd_bytes for s in self.mbs.values() for p in s.stage_programs.values())
+        return "forward buffers %s, backward/scratch buffers %s" % (fmem(fwd), fmem(self.pool.bytes))
+
+    def launch_counts(self):
+        out = {}
+        for mb, slot in self.mbs.items():
+            for sid, p in slot.stage_programs.items():
+                out[(sid, mb)] = (len(p.fwd), len(p.bwd))
+        return out

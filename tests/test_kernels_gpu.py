@@ -44,9 +44,11 @@ GEMM_SHAPES = [(197, 197, 64), (130, 72, 200), (257, 1000, 88), (512, 384, 1024)
 @pytest.mark.parametrize("a_trans,b_trans", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_gemm_layouts(hip, oracle, dtype, a_trans, b_trans):
     for i, (M, N, K) in enumerate(GEMM_SHAPES):
-        pad = 8
-        lda = (M if a_trans else K) + pad
-        ldb = (N if b_trans else K) + pad
+        def ld8(v):  # 16-bit operands need leading dimensions that are multiples of 8
+            return (v + 7) // 8 * 8 + 8
+
+        lda = ld8(M if a_trans else K)
+        ldb = ld8(N if b_trans else K)
         ldc = N + 3
         a = rnd((K if a_trans else M, lda), dtype, 10 + i)
         b = rnd((K if b_trans else N, ldb), dtype, 20 + i)
@@ -67,8 +69,6 @@ def test_gemm_batched_strided_heads(hip, oracle, dtype):
     Tp = 200
     s = torch.zeros(B, H, T, Tp, dtype=F32)
     q, k, v = qkv[:, :, 0:C], qkv[:, :, C:2 * C], qkv[:, :, 2 * C:]
-    for tab, dev_t in ((hip, "cuda"), (oracle, "cpu")):
-        pass
     res = {}
     for name, tab, dev in (("hip", hip, "cuda"), ("oracle", oracle, "cpu")):
         t = qkv.to(dev)

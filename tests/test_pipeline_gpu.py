@@ -1,0 +1,153 @@
+"""End-to-end parity of the HIP stage executor (PartialRunner.step on the GPU)
+against the CPU oracle of the reference's stage execution (oracle/stage_oracle.py)
+on identical seeded inputs and weights.
+
+Tolerances (from the task's north star): micro-batch split bit-exact; loss within
+1e-5 relative in fp32 and 2e-2 relative in bf16/fp16; gradients: fp32
+max|d| <= 1e-4 * max|g| per tensor, 16-bit relative L2 <= 2e-2 per tensor
+(fp32 accumulation of 16-bit products on both sides)."""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+pytestmark = pytest.mark.gpu
+
+
+def _fresh_runner(option):
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife
+    from pfeife_amd.mp import net_states
+
+    torch._dynamo.reset()
+    net_states._reset_state_for_tests()
+    initialize_pfeife()
+    return PartialRunner(option)
+
+
+def _run_vit(cfg, batch, batch_cnt, split, mixed, device_cnt=2, steps=1, seed=0):
+    from oracle.stage_oracle import run_pipeline_step
+    from pfeife_amd.bench_models.vit import VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    torch.manual_seed(seed)
+    model = VisionTransformer(cfg)
+    ref = copy.deepcopy(model)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(batch, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
+    y = torch.randint(0, cfg.num_classes, (batch,), generator=g)
+
+    option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
+                        split_points=[split] if split else None, mixed_precision=mixed,
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+
+    def fn(px, labels):
+        out = cmodel(px)
+        loss = crit(out.float(), labels)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    xd, yd = x.cuda(), y.cuda()
+    for _ in range(steps):
+        losses = runner.step(xd, yd)
+    torch.cuda.synchronize()
+
+    # oracle: the reference's stage semantics on CPU (autocast for mixed precision)
+    k = int(split.split(".")[1]) if split else cfg.depth
+
+    class Stage0(nn.Module):
+        def __init__(self, m):
+            super().__init__()
+            self.m = m
+
+        def forward(self, px):
+            m = self.m
+            t = m.patch_embed(px).flatten(2).transpose(1, 2)
+            t = torch.cat([m.cls_token.expand(t.shape[0], -1, -1), t], dim=1) + m.pos_embed
+            for blk in m.blocks[:k]:
+                t = blk(t)
+            return t
+
+    class Stage1(nn.Module):
+        def __init__(self, m):
+            super().__init__()
+            self.m = m
+
+        def forward(self, t):
+            m = self.m
+            for blk in m.blocks[k:]:
+                t = blk(t)
+            return m.head(m.norm(t)[:, 0])
+
+    adt = {"fp16": torch.float16, "bf16": torch.bfloat16}.get(mixed)
+    stages = [Stage0(ref), Stage1(ref)] if split else [nn.Sequential(Stage0(ref), Stage1(ref))]
+    ref_losses = run_pipeline_step(stages, lambda o, t: crit(o.float(), t), x, y, batch_cnt,
+                                   device_cnt=device_cnt, autocast_dtype=adt)
+    return model, ref, losses, ref_losses, runner
+
+
+def _check(model, ref, losses, ref_losses, mixed):
+    assert len(losses) == len(ref_losses)
+    ltol = 1e-5 if mixed is None else 2e-2
+    for a, b in zip(losses, ref_losses):
+        a, b = float(a), float(b)
+        assert abs(a - b) <= ltol * abs(b), ("loss", a, b)
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        gp, gq = p.grad.float().cpu(), q.grad.float()
+        assert torch.isfinite(gp).all(), n
+        if mixed is None:
+            assert (gp - gq).abs().max() <= 1e-4 * gq.abs().max() + 1e-9, (n, float((gp - gq).abs().max()))
+        else:
+            rel = (gp - gq).norm() / (gq.norm() + 1e-12)
+            assert rel <= 2e-2, (n, float(rel))
+
+
+def test_vit_tiny_fp32_two_stages():
+    from pfeife_amd.bench_models.vit import ViTConfig
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=4, heads=4, mlp_dim=128, num_classes=10)
+    m, r, l, rl, runner = _run_vit(cfg, 8, 4, "blocks.2", None)
+    _check(m, r, l, rl, None)
+
+
+@pytest.mark.parametrize("mixed", [None, "fp16", "bf16"])
+def test_vit_s16_config_c1(mixed):
+    """BASELINE config 0: ViT-S/16, micro-batch 4 x 4, two stages split at block 6, CE loss."""
+    from pfeife_amd.bench_models.vit import VIT_S16
+
+    m, r, l, rl, _ = _run_vit(VIT_S16, 16, 4, "blocks.6", mixed)
+    _check(m, r, l, rl, mixed)
+
+
+def test_vit_single_stage_and_repeatability():
+    from pfeife_amd.bench_models.vit import ViTConfig
+
+    cfg = ViTConfig(image_size=64, patch_size=16, dim=128, depth=2, heads=4, mlp_dim=256, num_classes=16)
+    m, r, l, rl, runner = _run_vit(cfg, 6, 3, None, None, device_cnt=1, steps=3)
+    _check(m, r, l, rl, None)
+
+
+def test_loss_wrappers_match_torch():
+    from pfeife_amd.loss import CrossEntropyLoss, RescaleLoss, SumLoss
+
+    g = torch.Generator().manual_seed(1)
+    logits = torch.randn(16, 1000, generator=g).cuda().requires_grad_()
+    target = torch.randint(0, 1000, (16,), generator=g).cuda()
+    ref_in = logits.detach().clone().requires_grad_()
+    loss = RescaleLoss(CrossEntropyLoss(1000), 0.5)(logits, target)
+    ref = nn.CrossEntropyLoss()(ref_in, target) * 0.5
+    loss.backward()
+    ref.backward()
+    torch.testing.assert_close(loss, ref, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(logits.grad, ref_in.grad, rtol=1e-4, atol=1e-7)
+    x = torch.randn(33, 7, generator=g).cuda().requires_grad_()
+    s = SumLoss()(x, None)
+    s.backward()
+    torch.testing.assert_close(s, x.detach().sum(), rtol=1e-5, atol=1e-4)
+    assert torch.equal(x.grad, torch.ones_like(x))
