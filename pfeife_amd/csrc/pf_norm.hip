@@ -197,6 +197,13 @@ __global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, in
   }
 }
 
+inline int64_t colsum_chunks(int64_t rows) {
+  int64_t chunks = (rows + 31) / 32;
+  if (chunks > 256) chunks = 256;
+  if (chunks < 1) chunks = 1;
+  return chunks;
+}
+
 inline int norm_bwd_blocks(int64_t rows) {
   int64_t b = (rows + 3) / 4;
   if (b < 1) b = 1;
@@ -264,9 +271,15 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
 
 }  // namespace
 
+// fp32 elements needed by the two-stage column reductions over a [rows, cols]
+// matrix: the norm backward writes 2 partial rows per workgroup, the column sum
+// one partial row per row chunk.
 extern "C" int64_t pf_colreduce_workspace(int64_t rows, int64_t cols) {
-  (void)rows;
-  return 2 * (int64_t)COLRED_MAX_BLOCKS * (cols > 0 ? cols : 1);
+  if (cols < 1) cols = 1;
+  if (rows < 1) rows = 1;
+  const int64_t norm = 2 * (int64_t)norm_bwd_blocks(rows) * cols;
+  const int64_t colsum = colsum_chunks(rows) * cols;
+  return norm > colsum ? norm : colsum;
 }
 
 extern "C" int pf_layernorm_fwd(const void* x, int x_dtype, const float* gamma, const float* beta, void* y,
@@ -305,8 +318,7 @@ extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, in
   if (rows == 0 || cols == 0) return PF_OK;
   PF_REQUIRE(x && acc && workspace, "pf_colsum_accumulate: null pointer");
   PF_REQUIRE(pf_is_float_dtype(x_dtype), "pf_colsum_accumulate: bad dtype");
-  int64_t chunks = (rows + 31) / 32;
-  if (chunks > 256) chunks = 256;
+  int64_t chunks = colsum_chunks(rows);
   const int64_t rpc = (rows + chunks - 1) / chunks;
   chunks = (rows + rpc - 1) / rpc;
   const bool v = vec_ok(x, x_dtype, ld) && cols % 8 == 0;

@@ -323,13 +323,10 @@ class Lowerer:
         self.cur.fwd_bytes += t.numel() * t.element_size()
         return t
 
-    def workspace(self, cols):
-        need = self.kernels.colreduce_workspace(0, cols)
-        if self._ws is None or self._ws.numel() < need:
-            if self._ws is not None:
-                raise RuntimeError("column-reduction workspace grew after launches were prepared")
-            self._ws = torch.empty(max(need, 2 * 512 * 32768), dtype=torch.float32, device=self.device)
-        return self._ws
+    def workspace(self, rows, cols):
+        """fp32 scratch for the two-stage column reductions (shared by every launch of that size)."""
+        need = max(1, self.kernels.colreduce_workspace(rows, cols))
+        return self.pool.scratch("colreduce_ws", (need,), torch.float32)
 
     def emit(self, launch):
         self.cur.fwd.append(launch)
@@ -551,7 +548,7 @@ def lower_linear(L, node):
             B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
                             b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
-            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(N)))
+            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(M, N)))
         if x.req_grad:
             dst, prev = B.grad_target(x)
             dm = as_matrix(dst)
@@ -631,7 +628,7 @@ def lower_layer_norm(L, node, rms=False):
             g = t
         dgamma = L.params.grad(gamma.param) if gamma.req_grad and gamma.param is not None else None
         dbeta = L.params.grad(beta.param) if beta is not None and beta.req_grad and beta.param is not None else None
-        ws = L.workspace(d) if (dgamma is not None or dbeta is not None) else None
+        ws = L.workspace(rows, d) if (dgamma is not None or dbeta is not None) else None
         if x.req_grad:
             dst, prev = B.grad_target(x)
             if not dst.is_contiguous() or (prev is not None and not prev.is_contiguous()):
@@ -796,7 +793,7 @@ def lower_conv2d(L, node):
             B.emit(B.k.gemm(dy, cols, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
                             b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
-            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(N)))
+            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(M, N)))
         if x.req_grad:
             dcols = B.temp((M, K), cd)
             B.emit(B.k.gemm(dy, w_cd, dcols, M=M, N=K, K=N, lda=ld_dy, ldb=K, ldc=K, b_trans=1))
@@ -994,7 +991,7 @@ def lower_expand(L, node):
             B.emit(B.k.fill(dst, 0.0, dst.numel()))
         elif prev is not dst:
             B.copy(prev, dst)
-        B.emit(B.k.colsum_accumulate(gc, rows, cols, as_matrix(gc)[2], dst, L.workspace(cols)))
+        B.emit(B.k.colsum_accumulate(gc, rows, cols, as_matrix(gc)[2], dst, L.workspace(rows, cols)))
         B.commit(x, dst)
 
     if x.req_grad:
@@ -1092,7 +1089,7 @@ def lower_add(L, node):
                 B.emit(B.k.fill(dst, 0.0, dst.numel()))
             elif prev is not dst:
                 B.copy(prev, dst)
-            B.emit(B.k.colsum_accumulate(gc, n // blen, blen, blen, dst, L.workspace(blen)))
+            B.emit(B.k.colsum_accumulate(gc, n // blen, blen, blen, dst, L.workspace(n // blen, blen)))
             B.commit(b, dst)
 
     if req:
