@@ -156,13 +156,24 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
   }
 }
 
-// acc[c] += sum_p ws[p*stride + c]
-__global__ void colreduce_finalize_kernel(const float* ws, int n_partials, int64_t stride, int64_t cols, float* acc) {
-  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= cols) return;
+// acc[c] += sum_p ws[p*stride + c].  A block owns 32 columns; its 8 groups of 32
+// threads split the partials, then combine through LDS in a fixed order.
+__global__ __launch_bounds__(256) void colreduce_finalize_kernel(const float* ws, int n_partials, int64_t stride,
+                                                                 int64_t cols, float* acc) {
+  __shared__ float red[8][32];
+  const int cl = threadIdx.x & 31, part = threadIdx.x >> 5;
+  const int64_t c = (int64_t)blockIdx.x * 32 + cl;
   float s = 0.f;
-  for (int p = 0; p < n_partials; ++p) s += ws[(int64_t)p * stride + c];
-  acc[c] += s;
+  if (c < cols)
+    for (int p = part; p < n_partials; p += 8) s += ws[(int64_t)p * stride + c];
+  red[part][cl] = s;
+  __syncthreads();
+  if (part == 0 && c < cols) {
+    float t = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) t += red[q][cl];
+    acc[c] += t;
+  }
 }
 
 // column sums of x[rows, cols]: block = 4 wavefronts sharing one 64*W column
@@ -261,7 +272,7 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
 #undef PF_NB
   PF_CHECK_LAUNCH(name);
   if (want) {
-    const dim3 fg((unsigned)((d + 255) / 256));
+    const dim3 fg((unsigned)((d + 31) / 32));
     if (dgamma) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws, blocks, 2 * d, d, dgamma);
     if (dbeta) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws + d, blocks, 2 * d, d, dbeta);
     PF_CHECK_LAUNCH(name);
@@ -330,7 +341,7 @@ extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, in
     hipLaunchKernelGGL(colsum_kernel<1>, grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc);
   }
   PF_CHECK_LAUNCH("pf_colsum_accumulate");
-  hipLaunchKernelGGL(colreduce_finalize_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, st, workspace,
+  hipLaunchKernelGGL(colreduce_finalize_kernel, dim3((unsigned)((cols + 31) / 32)), dim3(256), 0, st, workspace,
                      (int)chunks, cols, cols, acc);
   PF_CHECK_LAUNCH("pf_colsum_accumulate(finalize)");
   return PF_OK;
