@@ -59,6 +59,9 @@ class PartialRunner:
         self._batch_threads = []
         self.results = []
         self.worker = StageWorker(self, self.option, self.net_state.device, kernels)
+        # stage programs are built for concrete shapes: a new micro-batch shape must give a new static
+        # graph (handled as an alias of the pipelined one), not a symbolic-shape graph
+        torch._dynamo.config.automatic_dynamic_shapes = False
         PartialModule.set_runner(self)
         for i in range(self.option.batch_cnt):
             t = threading.Thread(target=self._exec_loop, args=(i,), daemon=True, name="pfeife-mb%d" % i)
@@ -193,7 +196,21 @@ class PartialModule(nn.Module):
                   % (len(self._all_modules) + 1, len(gm.graph.nodes), self.should_pp))
             gm.graph.print_tabular()
         self.partition_graph = None
+        # TorchDynamo recompiles when a micro-batch arrives with a new shape (ragged last chunk);
+        # a structurally identical graph is the same pipeline, run by the module that owns the programs
+        self.alias_of = None
+        if not self.should_pp:
+            sig = self._structure(gm)
+            for m in self._all_modules:
+                if m.should_pp and m._sig == sig:
+                    self.alias_of = m
+                    break
+        self._sig = self._structure(gm) if self.should_pp else None
         self._all_modules.append(self)
+
+    @staticmethod
+    def _structure(gm):
+        return tuple((n.op, str(n.target)) for n in gm.graph.nodes)
 
     @staticmethod
     def set_runner(runner: PartialRunner):
@@ -220,7 +237,8 @@ class PartialModule(nn.Module):
                       % (idx, len(st.graph_module.graph.nodes)))
                 st.graph_module.graph.print_tabular()
         worker.set_partition_graph(self.partition_graph, live)
-        self._pp_modules.append(self)
+        if self.alias_of is None:
+            self._pp_modules.append(self)
         del ex
 
     def _dynamic_inputs(self, args):
@@ -233,8 +251,8 @@ class PartialModule(nn.Module):
         dyn = self._dynamic_inputs(args)
         sig = worker._signature([dyn[i] for i in sorted(dyn)])
         slot = worker.mbs.get(mb)
-        if slot is None or slot.input_sig != sig:
-            worker.build_micro_batch(mb, dyn)
+        if slot is None or slot.input_sig != sig or slot.graph is not self.partition_graph:
+            worker.build_micro_batch(mb, dyn, self.partition_graph).graph = self.partition_graph
         return dyn
 
     def _outputs_for_user(self, mb, probe):
@@ -261,7 +279,8 @@ class PartialModule(nn.Module):
 
     # -- call ----------------------------------------------------------------------------
     def forward(self, *args):
-        if not self.should_pp:
+        owner = self.alias_of if self.alias_of is not None else self
+        if not owner.should_pp:
             return self.gm(*to_device(args, self.device))
         runner = self._runner
         if runner._probing:
@@ -269,11 +288,13 @@ class PartialModule(nn.Module):
                 self._compile(args)
             self._ensure_programs(0, args)
             return self._outputs_for_user(0, probe=True)
-        if self.partition_graph is None:
+        if owner.partition_graph is None:
             raise RuntimeError("the compiled model was called outside PartialRunner.step()")
+        if self.partition_graph is None:
+            self._compile(args)  # same pipeline, captured again for another micro-batch shape
 
-        mb = self.curr_batch
-        self.curr_batch += 1
+        mb = owner.curr_batch
+        owner.curr_batch += 1
         if mb >= self._option.batch_cnt:
             raise RuntimeError("the compiled model was called more than batch_cnt times in one step")
         dyn = self._ensure_programs(mb, args)

@@ -31,6 +31,7 @@ class MicroBatchPrograms:
         self.input_sig = None      # shapes/dtypes the programs were built for
         self.outputs = []          # per graph output: Val | python constant
         self.loss_grads = {}       # graph output index -> static gradient buffer
+        self.graph = None          # the partition graph the programs were lowered from
         self.grad_seen = set()
 
 
@@ -57,16 +58,29 @@ class StageWorker:
 
     # -- graph ---------------------------------------------------------------------
     def set_partition_graph(self, part_graph, example_inputs):
-        self.part_graph = pg = part_graph
-        self.static_inputs = {}
+        """Register a stage partition.  The first one fixes the schedule; later ones are
+        the same pipeline captured again for another micro-batch shape (TorchDynamo
+        recompiles with the new sizes baked in) and must have the same stage count."""
+        pg = part_graph
+        static = {}
         for i, (is_static, ex) in enumerate(zip(pg.static_placeholder, example_inputs)):
             if not is_static:
                 continue
             if ex.device != self.device:
                 ex.data = ex.data.to(self.device)  # stage parameters live on the worker's device
             param = ex if isinstance(ex, torch.nn.Parameter) else None
-            self.static_inputs[i] = Val(ex.detach(), req_grad=bool(ex.requires_grad), param=param,
-                                        name=pg.placeholder_names[i])
+            static[i] = Val(ex.detach(), req_grad=bool(ex.requires_grad), param=param,
+                            name=pg.placeholder_names[i])
+        pg.static_vals = static
+        if self.part_graph is not None:
+            if len(pg.nodes) != len(self.part_graph.nodes):
+                raise RuntimeError("recaptured graph splits into %d stages, the pipeline has %d"
+                                   % (len(pg.nodes), len(self.part_graph.nodes)))
+            for st in pg.nodes.values():
+                st.rank = self.part_graph.nodes[st.idx].rank
+            return
+        self.part_graph = pg
+        self.static_inputs = static
         node_cnt = len(pg.nodes)
         opt = self.option
         device_cnt = max(1, min(opt.device_cnt, node_cnt))
@@ -102,10 +116,10 @@ class StageWorker:
                 sig.append(("const", repr(v)))
         return tuple(sig)
 
-    def build_micro_batch(self, mb, dynamic_inputs):
+    def build_micro_batch(self, mb, dynamic_inputs, part_graph=None):
         """Lower every stage for micro-batch slot `mb`; `dynamic_inputs` maps graph
         placeholder index -> the value user code passed (tensor chunk or constant)."""
-        pg = self.part_graph
+        pg = part_graph if part_graph is not None else self.part_graph
         slot = MicroBatchPrograms()
         slot.input_sig = self._signature([dynamic_inputs[i] for i in sorted(dynamic_inputs)])
         graph_vals = {}
@@ -116,7 +130,7 @@ class StageWorker:
                 graph_vals[i] = Val(buf, req_grad=False, name=pg.placeholder_names[i])
             else:
                 graph_vals[i] = v
-        for i, v in self.static_inputs.items():
+        for i, v in pg.static_vals.items():
             graph_vals[i] = v
         L = self.lowerer
         stage_out = {}

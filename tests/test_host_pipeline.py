@@ -1,0 +1,143 @@
+"""Host logic of the executor on CPU: graph capture, stage partition, lowering to
+launch programs, schedule-ordered job loop, micro-batch threads.  The kernel
+table is replaced by the CPU oracle of the kernels (a test double injected
+through PartialRunner's `kernels` argument; the product only ships the HIP
+table), so these tests check everything EXCEPT the HIP code."""
+import copy
+
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle.kernels_oracle import OracleKernels
+from oracle.stage_oracle import run_pipeline_step, run_unpipelined
+from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer, split_stages
+from pfeife_amd.mp import net_states
+from pfeife_amd.option import PipeOption
+
+CFG = ViTConfig(image_size=32, patch_size=16, dim=64, depth=4, heads=4, mlp_dim=128, num_classes=10)
+
+
+def make_runner(option):
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife
+
+    torch._dynamo.reset()
+    net_states._reset_state_for_tests()
+    initialize_pfeife(device="cpu")
+    return PartialRunner(option, kernels=OracleKernels("cpu"))
+
+
+def run_case(mixed, batch=8, batch_cnt=4, device_cnt=2, split=("blocks.2",), steps=1, lr=0.0, opt_type="sgd"):
+    from pfeife_amd.mp import partial_compiler
+
+    torch.manual_seed(0)
+    model = VisionTransformer(CFG)
+    ref = copy.deepcopy(model)
+    option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
+                        split_points=list(split) if split else None, mixed_precision=mixed,
+                        optimizer=dict(type=opt_type, lr=lr))
+    runner = make_runner(option)
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+
+    def fn(x, y):
+        loss = crit(cmodel(x).float(), y)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(batch, 3, 32, 32, generator=g)
+    y = torch.randint(0, 10, (batch,), generator=g)
+    out = [runner.step(x, y) for _ in range(steps)]
+    return model, ref, out, (x, y), runner, crit
+
+
+def test_fp32_matches_reference_stage_semantics():
+    model, ref, out, (x, y), runner, crit = run_case(None)
+    want = run_pipeline_step(split_stages(ref, 2), crit, x, y, 4, device_cnt=2)
+    for a, b in zip(out[0], want):
+        assert abs(float(a) - float(b)) <= 1e-5 * abs(float(b))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+    # the job order is the serialised looped schedule: F00 F01 | F10 ... and ends with the last backward of stage 0
+    order = runner.worker.order
+    assert order[0] == (0, 0, True) and order[-1] == (0, 3, False)
+    assert len(order) == 2 * 2 * 4
+
+
+@pytest.mark.parametrize("mixed,tol", [("bf16", 3e-2), ("fp16", 5e-3)])
+def test_mixed_precision_follows_autocast(mixed, tol):
+    model, ref, out, (x, y), _, crit = run_case(mixed)
+    adt = {"bf16": torch.bfloat16, "fp16": torch.float16}[mixed]
+    want = run_unpipelined(ref, lambda o, t: crit(o.float(), t), x, y, 4, autocast_dtype=adt)
+    for a, b in zip(out[0], want):
+        assert abs(float(a) - float(b)) <= 2e-2 * abs(float(b))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        rel = (p.grad - q.grad).norm() / (q.grad.norm() + 1e-12)
+        assert rel <= tol, (n, float(rel))
+
+
+def test_single_stage_ragged_batch_and_repeat():
+    # 7 samples over 3 micro-batches -> 3, 2, 2 rows; same result on every repetition (lr = 0)
+    model, ref, out, (x, y), runner, crit = run_case(None, batch=7, batch_cnt=3, device_cnt=1, split=None, steps=3)
+    want = run_unpipelined(ref, crit, x, y, 3)
+    assert [float(a) for a in out[0]] == [float(a) for a in out[2]]
+    for a, b in zip(out[0], want):
+        assert abs(float(a) - float(b)) <= 1e-5 * abs(float(b))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+
+
+def test_optimizer_step_updates_parameters_like_eager_training():
+    model, ref, out, (x, y), runner, crit = run_case(None, steps=2, lr=0.05)
+    opt = torch.optim.SGD(ref.parameters(), lr=0.05)
+    ref_losses = []
+    for _ in range(2):
+        ref_losses.append(run_unpipelined(ref, crit, x, y, 4))
+        opt.step()
+    for a, b in zip(out[1], ref_losses[1]):
+        assert abs(float(a) - float(b)) <= 1e-4 * abs(float(b))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        torch.testing.assert_close(p.detach(), q.detach(), rtol=1e-4, atol=1e-6, msg=n)
+
+
+def test_three_stages_integer_split_points_and_errors():
+    from pfeife_amd.graph.partition_graph import compute_nodes, resolve_split_points
+    from pfeife_amd.mp import partial_compiler
+
+    model, ref, out, (x, y), runner, crit = run_case(None, split=("blocks.1", "blocks.3"), device_cnt=3, batch_cnt=4)
+    want = run_unpipelined(ref, crit, x, y, 4)
+    for a, b in zip(out[0], want):
+        assert abs(float(a) - float(b)) <= 1e-5 * abs(float(b))
+    pg = runner.worker.part_graph
+    assert sorted(pg.nodes) == [0, 1, 2]
+    # each cross-stage value appears once as a producer output and once per consumer input
+    for sid, st in pg.nodes.items():
+        for k, src in enumerate(st.input_source):
+            if src is not None:
+                assert sid in pg.nodes[src[0]].output_map[pg.nodes[src[0]].outputs[src[1]]]
+    assert pg.outputs == [(2, 0)]
+    with pytest.raises(RuntimeError, match="matches no module path"):
+        resolve_split_points(pg.nodes[0].graph_module, ["nonexistent.9"])
+
+
+def test_unsupported_node_fails_loudly():
+    from pfeife_amd.executor.lowering import Unsupported
+    from pfeife_amd.mp import partial_compiler
+
+    class Odd(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = nn.Linear(8, 8)
+
+        def forward(self, x):
+            return torch.cumsum(self.fc(x), dim=1)
+
+    option = PipeOption(device_cnt=1, batch_cnt=1, batch_size=2)
+    runner = make_runner(option)
+    m = torch.compile(Odd(), backend=partial_compiler)
+    runner.set_exec_fn(lambda x: m(x).sum())
+    with pytest.raises(Exception) as ei:
+        runner.step(torch.randn(2, 8))
+    assert "no HIP lowering" in str(ei.value) or isinstance(ei.value, Unsupported)
