@@ -26,45 +26,67 @@ def log(*a):
 
 
 WORKLOADS = {
-    # name: (model family, config attr, global batch, batch_cnt, split points, device_cnt, mixed precision)
+    # name: (family, config attr, global batch, batch_cnt, split points, device_cnt, mixed precision)
     "vit_l16_fp16": ("vit", "VIT_L16", 64, 4, ["blocks.12"], 2, "fp16"),
     "vit_s16_fp32": ("vit", "VIT_S16", 16, 4, ["blocks.6"], 2, None),
+    "llama_1b_bf16": ("llama", "LLAMA_1B", 16, 8, ["layers.4", "layers.8", "layers.12"], 2, "bf16"),
+    "vit_g14_share_bf16": ("vit_share", "VIT_G14_SHARE", 96, 4, [], 1, "bf16"),
 }
 
 
 def build_workload(name, device):
     import torch
 
-    from pfeife_amd.bench_models import vit
+    from pfeife_amd.bench_models import llama, vit
     from pfeife_amd.loss import CrossEntropyLoss
     from pfeife_amd.mp import PartialRunner, initialize_pfeife, partial_compiler
     from pfeife_amd.option import PipeOption
 
     family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
-    cfg = getattr(vit, cfg_name)
     torch.manual_seed(42)
-    model = vit.VisionTransformer(cfg)
     g = torch.Generator().manual_seed(42)
-    x = torch.randn(batch, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
-    y = torch.randint(0, cfg.num_classes, (batch,), generator=g)
+    if family == "vit":
+        cfg = getattr(vit, cfg_name)
+        model = vit.VisionTransformer(cfg)
+        inputs = (torch.randn(batch, cfg.channels, cfg.image_size, cfg.image_size, generator=g),
+                  torch.randint(0, cfg.num_classes, (batch,), generator=g))
+    elif family == "vit_share":
+        cfg = getattr(vit, cfg_name)
+        model = vit.BlockStack(cfg)
+        inputs = (torch.randn(batch, cfg.tokens, cfg.dim, generator=g),
+                  torch.randn(batch, cfg.tokens, cfg.dim, generator=g) * 1e-2)
+    else:
+        cfg = getattr(llama, cfg_name)
+        model = llama.LlamaForCausalLM(cfg)
+        inputs = (torch.randint(0, cfg.vocab, (batch, cfg.max_seq), generator=g),)
     initialize_pfeife()
     option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
-                        split_points=splits, mixed_precision=mixed, optimizer=dict(type="adam", lr=1e-5))
+                        split_points=splits or None, mixed_precision=mixed, optimizer=dict(type="adam", lr=1e-5))
     runner = PartialRunner(option)
     model.to(device)
     cmodel = torch.compile(model, backend=partial_compiler)
-    crit = CrossEntropyLoss(cfg.num_classes)
+    if family == "vit":
+        crit = CrossEntropyLoss(cfg.num_classes)
 
-    def exec_fn(px, labels):
-        out = cmodel(px)
-        loss = crit(out, labels)
-        loss.backward()
-        return loss.detach()
+        def exec_fn(px, labels):
+            loss = crit(cmodel(px), labels)
+            loss.backward()
+            return loss.detach()
+    elif family == "vit_share":
+        def exec_fn(act, grad_out):
+            out = cmodel(act)
+            out.backward(grad_out.to(out.dtype))   # supplied upstream gradient of this GPU's block share
+            return out.detach()[0, 0, 0]
+    else:
+        def exec_fn(ids):
+            loss = cmodel(ids, ids)                # next-token CE is inside the last stage
+            loss.backward()
+            return loss.detach()
 
     runner.set_exec_fn(exec_fn)
     info = dict(cfg=cfg, batch=batch, batch_cnt=batch_cnt, splits=splits, device_cnt=device_cnt, mixed=mixed,
                 model=model, family=family)
-    return runner, (x.to(device), y.to(device)), info
+    return runner, tuple(t.to(device) for t in inputs), info
 
 
 def gemm_roofline(runner, mixed, reps=3):
@@ -139,39 +161,60 @@ def hbm_kernel_rates(runner, reps=3):
 
 def cpu_baseline(name):
     """The oracle's restatement of the reference's stage execution on the host
-    cores, fp32, on a bounded sample of the workload (2 micro-batches of 4)."""
+    cores, fp32, on a bounded sample of the workload (2 micro-batches)."""
     import torch
     import torch.nn as nn
+    import torch.nn.functional as F
 
     from oracle.stage_oracle import run_pipeline_step
-    from pfeife_amd.bench_models import vit
+    from pfeife_amd.bench_models import llama, vit
 
     family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
-    cfg = getattr(vit, cfg_name)
     cores = os.cpu_count() or 1
     env = os.environ.get("OMP_NUM_THREADS")
     if env:
         cores = min(cores, int(env))
     torch.set_num_threads(cores)
     torch.manual_seed(42)
-    model = vit.VisionTransformer(cfg)
-    k = int(splits[0].split(".")[1])
-    stages = vit.split_stages(model, k)
-    mb, cnt = 4, 2
     g = torch.Generator().manual_seed(42)
-    x = torch.randn(mb * cnt, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
-    y = torch.randint(0, cfg.num_classes, (mb * cnt,), generator=g)
-    crit = nn.CrossEntropyLoss()
+    cnt = 2
+    if family == "vit":
+        cfg = getattr(vit, cfg_name)
+        model = vit.VisionTransformer(cfg)
+        stages = vit.split_stages(model, int(splits[0].split(".")[1]))
+        mb = 4
+        x = torch.randn(mb * cnt, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
+        y = torch.randint(0, cfg.num_classes, (mb * cnt,), generator=g)
+        loss_fn = nn.CrossEntropyLoss()
+        unit, per_sample = "samples/s", 1
+    elif family == "vit_share":
+        cfg = getattr(vit, cfg_name)
+        stages = [vit.BlockStack(cfg)]
+        mb = 4
+        x = torch.randn(mb * cnt, cfg.tokens, cfg.dim, generator=g)
+        y = torch.randn(mb * cnt, cfg.tokens, cfg.dim, generator=g) * 1e-2
+        loss_fn = lambda o, t: (o * t).sum()
+        unit, per_sample = "samples/s", 1
+    else:
+        cfg = getattr(llama, cfg_name)
+        model = llama.LlamaForCausalLM(cfg)
+        stages = llama.split_stages(model, [int(s.split(".")[1]) for s in splits])
+        mb, T = 1, 512   # bounded: 2 micro-batches of one 512-token sequence
+        x = torch.randint(0, cfg.vocab, (mb * cnt, T), generator=g)
+        y = x
+        loss_fn = lambda lg, t: F.cross_entropy(lg[:, :-1].reshape(-1, lg.shape[-1]), t[:, 1:].reshape(-1))
+        unit, per_sample = "samples/s (sequences of 2048 tokens; measured tokens/s / 2048)", T / float(cfg.max_seq)
     times = []
     for _ in range(2):  # first pass warms the allocator and the thread pool
         t0 = time.perf_counter()
-        run_pipeline_step(stages, lambda o, t: crit(o, t), x, y, cnt, device_cnt=device_cnt)
+        run_pipeline_step(stages, loss_fn, x, y, cnt, device_cnt=device_cnt)
         times.append(time.perf_counter() - t0)
-    sps = mb * cnt / times[-1]
-    return dict(value=round(sps, 3), unit="samples/s", cores=cores, kind="port",
+    sps = mb * cnt * per_sample / times[-1]
+    return dict(value=round(sps, 4), unit=unit, cores=cores, kind="port",
                 sample="%s fp32 on CPU: %d micro-batches x %d samples, %d stages, forward+backward+grad-accumulate "
-                       "(no optimizer step), oracle stage executor; %.1f s" % (cfg_name, cnt, mb, len(stages),
-                                                                                  times[-1]))
+                       "(no optimizer step), oracle stage executor; %.1f s%s" % (
+                           cfg_name, cnt, mb, len(stages), times[-1],
+                           "" if family != "llama" else "; 512-token sequences, attention cost scaled linearly"))
 
 
 def main():
@@ -229,11 +272,17 @@ def main():
 
     cfg = info["cfg"]
     flops_step = None
-    if info["family"] == "vit":
+    if info["family"] in ("vit", "vit_share"):
         T, d, ff, L = cfg.tokens, cfg.dim, cfg.mlp_dim, cfg.depth
         per_block = 2 * T * d * 3 * d + 2 * T * d * d + 4 * T * d * ff + 4 * T * T * d
-        patch = 2 * (T - 1) * (cfg.channels * cfg.patch_size ** 2) * d
-        flops_step = 3.0 * samples * (L * per_block + patch + 2 * d * cfg.num_classes)
+        extra = 0
+        if info["family"] == "vit":
+            extra = 2 * (T - 1) * (cfg.channels * cfg.patch_size ** 2) * d + 2 * d * cfg.num_classes
+        flops_step = 3.0 * samples * (L * per_block + extra)
+    else:
+        T, d, ff, L, V = cfg.max_seq, cfg.dim, cfg.ffn, cfg.layers, cfg.vocab
+        per_tok = L * (8 * d * d + 6 * d * ff + 4 * T * d) + 2 * d * V
+        flops_step = 3.0 * samples * T * per_tok
     rec = {
         "metric": "train samples/sec on 1 MI355X; MFMA util % (GEMMs), HBM GB/s % (elementwise)",
         "value": round(value, 2),
@@ -246,9 +295,9 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": info["mixed"] or "fp32",
-        "data": "synthetic (images ~N(0,1), labels uniform int, random-init weights, seed 42)",
+        "data": "synthetic (inputs ~N(0,1) / uniform int ids, random-init weights, seed 42)",
         "config": {"workload": "%s: %s micro-batch %d x %d, %d stages split at %s, schedule drawn for %d ranks, "
-                               "all stages on one GPU, CE loss, Adam" % (
+                               "all stages on one GPU, Adam" % (
                                    args.workload, type(cfg).__name__, samples // info["batch_cnt"], info["batch_cnt"],
                                    len(info["splits"]) + 1, info["splits"], info["device_cnt"]),
                    "global_batch": samples, "batch_cnt": info["batch_cnt"]},

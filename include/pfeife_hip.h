@@ -216,17 +216,19 @@ int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n,
 int pf_fill(void* dst, int dtype, float value, int64_t n, void* stream);
 /* Generic strided copy with dtype conversion of a tensor of up to 6 dims:
  * dst[idx . dst_strides] = src[idx . src_strides]  (strides in elements). Used
- * for layout changes that are not views: patch extraction, head merges, cat. */
+ * for layout changes that are not views: patch extraction, head merges, cat.
+ * Integer dtypes (token ids) are copied raw: same dtype on both sides, no accumulate. */
 int pf_copy_strided(const void* src, int src_dtype, const int64_t* src_strides, void* dst, int dst_dtype,
                     const int64_t* dst_strides, const int64_t* sizes, int ndim, int accumulate, void* stream);
 /* Rotary position embedding (rotate-half convention of HF Llama: element i
  * pairs with i + D/2): x and y are [B, T, H, D] tensors addressed with element
- * strides (sb, st, sh, 1); cos_t/sin_t are fp32 [T, D/2].
+ * strides (sb, st, sh, 1); cos_t/sin_t are fp32 tables with T rows of row
+ * stride tab_ld (>= D/2) whose first D/2 columns are used.
  *   y[i]       = x[i] cos[t,i] - x[i+D/2] sin[t,i]
  *   y[i+D/2]   = x[i+D/2] cos[t,i] + x[i] sin[t,i]
  * inverse != 0 applies the transposed rotation (the backward pass). y may alias x. */
-int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t B, int64_t T,
-            int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh, int64_t y_sb, int64_t y_st,
+int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t tab_ld, int64_t B,
+            int64_t T, int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh, int64_t y_sb, int64_t y_st,
             int64_t y_sh, int inverse, void* stream);
 
 /* ---- gradient accumulation --------------------------------------------------

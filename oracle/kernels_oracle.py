@@ -310,19 +310,23 @@ class OracleKernels:
         def launch(stream=None):
             s = _strided(src, tuple(sizes), tuple(src_strides))
             d = _strided(dst, tuple(sizes), tuple(dst_strides))
-            if accumulate:
+            if not src.dtype.is_floating_point:
+                assert src.dtype == dst.dtype and not accumulate
+                d.copy_(s)
+            elif accumulate:
                 d.copy_((d.float() + s.float()).to(dst.dtype))
             else:
                 d.copy_(s.to(dst.dtype))
 
         return launch
 
-    def rope(self, x, y, cos_t, sin_t, B, T, H, D, xs, ys, inverse):
+    def rope(self, x, y, cos_t, sin_t, B, T, H, D, xs, ys, inverse, tab_ld=None):
         def launch(stream=None):
             half = D // 2
+            ld = half if tab_ld is None else tab_ld
             X = _strided(x, (B, T, H, D), (xs[0], xs[1], xs[2], 1)).float()
-            c = _strided(cos_t, (T, half), (half, 1)).float()[None, :, None, :]
-            s = _strided(sin_t, (T, half), (half, 1)).float()[None, :, None, :]
+            c = _strided(cos_t, (T, half), (ld, 1)).float()[None, :, None, :]
+            s = _strided(sin_t, (T, half), (ld, 1)).float()[None, :, None, :]
             if inverse:
                 s = -s
             x1, x2 = X[..., :half], X[..., half:]

@@ -183,12 +183,31 @@ __global__ __launch_bounds__(EW_BLOCK) void copy_strided_kernel(const void* src,
   }
 }
 
+// same-dtype copy of non-float element types (token ids, masks): moves raw elements
+template <typename U>
+__global__ __launch_bounds__(EW_BLOCK) void copy_strided_raw_kernel(const U* src, U* dst, CopyDesc cd, int64_t total) {
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gsz) {
+    int64_t rem = i, so = 0, dof = 0;
+#pragma unroll
+    for (int k = 5; k >= 0; --k) {
+      if (k < cd.ndim) {
+        const int64_t idx = rem % cd.size[k];
+        rem /= cd.size[k];
+        so += idx * cd.ss[k];
+        dof += idx * cd.ds[k];
+      }
+    }
+    dst[dof] = src[so];
+  }
+}
+
 // ---- rotary embedding --------------------------------------------------------
 // one thread per (b, t, h, i) pair index i < D/2
 __global__ __launch_bounds__(EW_BLOCK) void rope_kernel(const void* x, void* y, int dt, const float* cos_t,
-                                                        const float* sin_t, int64_t B, int64_t T, int64_t H,
-                                                        int64_t D, int64_t xsb, int64_t xst, int64_t xsh, int64_t ysb,
-                                                        int64_t yst, int64_t ysh, int inverse) {
+                                                        const float* sin_t, int64_t tab_ld, int64_t B, int64_t T,
+                                                        int64_t H, int64_t D, int64_t xsb, int64_t xst, int64_t xsh,
+                                                        int64_t ysb, int64_t yst, int64_t ysh, int inverse) {
   const int64_t half = D / 2;
   const int64_t total = B * T * H * half;
   const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
@@ -200,8 +219,8 @@ __global__ __launch_bounds__(EW_BLOCK) void rope_kernel(const void* x, void* y, 
     const int64_t t = r % T, b = r / T;
     const int64_t xo = b * xsb + t * xst + h * xsh, yo = b * ysb + t * yst + h * ysh;
     const float x1 = pf_load_as_f32(x, xo + i, dt), x2 = pf_load_as_f32(x, xo + i + half, dt);
-    const float c = cos_t[t * half + i];
-    const float s = inverse ? -sin_t[t * half + i] : sin_t[t * half + i];
+    const float c = cos_t[t * tab_ld + i];
+    const float s = inverse ? -sin_t[t * tab_ld + i] : sin_t[t * tab_ld + i];
     pf_store_from_f32(y, yo + i, dt, x1 * c - x2 * s);
     pf_store_from_f32(y, yo + i + half, dt, x2 * c + x1 * s);
   }
@@ -306,7 +325,10 @@ extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* sr
                                void* stream) {
   PF_REQUIRE(ndim >= 1 && ndim <= 6, "pf_copy_strided: ndim %d outside 1..6", ndim);
   PF_REQUIRE(src_strides && dst_strides && sizes, "pf_copy_strided: null shape");
-  PF_REQUIRE(pf_is_float_dtype(src_dtype) && pf_is_float_dtype(dst_dtype), "pf_copy_strided: bad dtype");
+  const bool raw = !pf_is_float_dtype(src_dtype);
+  if (raw) PF_REQUIRE(src_dtype == dst_dtype && pf_dtype_size(src_dtype) > 0 && !accumulate,
+                      "pf_copy_strided: integer tensors can only be copied to the same dtype");
+  else PF_REQUIRE(pf_is_float_dtype(dst_dtype), "pf_copy_strided: bad dtype");
   CopyDesc cd;
   cd.ndim = ndim;
   int64_t total = 1;
@@ -326,7 +348,13 @@ extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* sr
   PF_REQUIRE(src && dst, "pf_copy_strided: null pointer");
   vec = vec && src_strides[ndim - 1] == 1 && dst_strides[ndim - 1] == 1 && sizes[ndim - 1] % 8 == 0;
   hipStream_t st = (hipStream_t)stream;
-  if (vec) {
+  if (raw) {
+    switch (pf_dtype_size(src_dtype)) {
+      case 8: hipLaunchKernelGGL(copy_strided_raw_kernel<uint64_t>, ew_grid(total), dim3(EW_BLOCK), 0, st, (const uint64_t*)src, (uint64_t*)dst, cd, total); break;
+      case 4: hipLaunchKernelGGL(copy_strided_raw_kernel<uint32_t>, ew_grid(total), dim3(EW_BLOCK), 0, st, (const uint32_t*)src, (uint32_t*)dst, cd, total); break;
+      default: hipLaunchKernelGGL(copy_strided_raw_kernel<uint8_t>, ew_grid(total), dim3(EW_BLOCK), 0, st, (const uint8_t*)src, (uint8_t*)dst, cd, total); break;
+    }
+  } else if (vec) {
     cd.size[ndim - 1] /= 8;
     total /= 8;
     hipLaunchKernelGGL(copy_strided_kernel<8>, ew_grid(total), dim3(EW_BLOCK), 0, st, src, src_dtype, dst, dst_dtype,
@@ -339,15 +367,16 @@ extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* sr
   return PF_OK;
 }
 
-extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t B,
-                       int64_t T, int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh, int64_t y_sb,
-                       int64_t y_st, int64_t y_sh, int inverse, void* stream) {
+extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t tab_ld,
+                       int64_t B, int64_t T, int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh,
+                       int64_t y_sb, int64_t y_st, int64_t y_sh, int inverse, void* stream) {
   PF_REQUIRE(B >= 0 && T >= 0 && H >= 0 && D >= 0 && D % 2 == 0 && pf_is_float_dtype(dtype), "pf_rope: bad arguments");
+  PF_REQUIRE(tab_ld >= D / 2, "pf_rope: table row stride %lld < D/2", (long long)tab_ld);
   const int64_t total = B * T * H * (D / 2);
   if (total == 0) return PF_OK;
   PF_REQUIRE(x && y && cos_t && sin_t, "pf_rope: null pointer");
-  hipLaunchKernelGGL(rope_kernel, ew_grid(total), dim3(EW_BLOCK), 0, (hipStream_t)stream, x, y, dtype, cos_t, sin_t, B,
-                     T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
+  hipLaunchKernelGGL(rope_kernel, ew_grid(total), dim3(EW_BLOCK), 0, (hipStream_t)stream, x, y, dtype, cos_t, sin_t,
+                     tab_ld, B, T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
   PF_CHECK_LAUNCH("pf_rope");
   return PF_OK;
 }

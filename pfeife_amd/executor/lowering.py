@@ -348,6 +348,7 @@ class Lowerer:
             if isinstance(v, Val):
                 v.name = v.name or n.name
         prog.inputs = list(input_vals)
+        self.patterns, self.pattern_skip = find_rope_patterns(gm)
         for node in gm.graph.nodes:
             if node.op == "placeholder":
                 continue
@@ -359,8 +360,12 @@ class Lowerer:
             if node in self.fused:
                 self.env[node] = self.fused[node]
                 continue
-            handler = self._handler(node)
-            out = handler(self, node)
+            if node in self.pattern_skip:
+                continue  # interior of a matched multi-node pattern, produced by the pattern's root
+            if node in self.patterns:
+                out = lower_rope(self, node, *self.patterns[node])
+            else:
+                out = self._handler(node)(self, node)
             self.env[node] = out
             if isinstance(out, Val) and not out.name:
                 out.name = node.name
@@ -432,7 +437,7 @@ class Lowerer:
     def copy(self, src, dst):
         if src.numel() == 0:
             return
-        if is_dense(src) and is_dense(dst) and src.stride() == dst.stride():
+        if src.dtype.is_floating_point and is_dense(src) and is_dense(dst) and src.stride() == dst.stride():
             self.emit(self.kernels.cast(src, dst, src.numel()))
             return
         sizes, ss, ds = collapse_for_copy(src.shape, src.stride(), dst.stride())
@@ -502,7 +507,12 @@ def lower_linear(L, node):
     user = L.sole_user(node)
     if user is not None:
         a = _act_of_node(user)
-        if a is not None and user.args[0] is node:
+        gate_of_glu = False
+        if a is not None and len(user.users) == 1:
+            uu = next(iter(user.users))
+            gate_of_glu = (uu.op == "call_function" and uu.target in (operator.mul, torch.mul)
+                           and all(isinstance(x, torch.fx.Node) for x in uu.args[:2]))
+        if a is not None and user.args[0] is node and not gate_of_glu:
             act, out_node = a, user
         elif _is_add_node(user) and not user.kwargs:
             other = user.args[1] if user.args[0] is node else user.args[0]
@@ -1181,6 +1191,9 @@ def lower_float(L, node):
     """x.float() / x.to(float32): under the mixed-precision policy a no-op for fp32 values,
     a cast kernel otherwise."""
     x = L.arg(node.args[0])
+    if L.mixed and node.users and all(u.op == "call_function" and u.target is F.cross_entropy for u in node.users):
+        # the loss kernels read 16-bit logits and do their arithmetic in fp32: no fp32 copy of the logits
+        return Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
     return _lower_cast(L, x, torch.float32)
 
 
@@ -1316,10 +1329,112 @@ def lower_act_maybe_gate(L, node):
     return lower_unary_act(L, node)
 
 
+def _is(node, *targets):
+    return isinstance(node, torch.fx.Node) and node.op == "call_function" and node.target in targets
+
+
+def find_rope_patterns(gm):
+    """Rotary embedding written the HF way,
+        x * cos + cat((-x[..., h:], x[..., :h]), -1) * sin,
+    is nine graph nodes; match it so that one kernel computes it.
+    -> ({add_node: (x_node, cos_node, sin_node)}, {interior nodes})"""
+    roots, skip = {}, set()
+    for add in gm.graph.nodes:
+        if not _is(add, operator.add, torch.add) or len(add.args) != 2:
+            continue
+        m1, m2 = add.args
+        if not (_is(m1, operator.mul, torch.mul) and _is(m2, operator.mul, torch.mul)):
+            continue
+        for a, b in ((m1, m2), (m2, m1)):
+            x, cos = a.args
+            cat, sin = b.args
+            if not _is(cat, torch.cat) or not isinstance(x, torch.fx.Node):
+                continue
+            parts = cat.args[0]
+            dim = cat.kwargs.get("dim", cat.args[1] if len(cat.args) > 1 else 0)
+            if dim != -1 or len(parts) != 2 or not _is(parts[0], operator.neg, torch.neg):
+                continue
+            hi, lo = parts[0].args[0], parts[1]
+            if not (_is(hi, operator.getitem) and _is(lo, operator.getitem)):
+                continue
+            if hi.args[0] is not x or lo.args[0] is not x:
+                continue
+            ih, il = hi.args[1], lo.args[1]
+            ok = (isinstance(ih, tuple) and isinstance(il, tuple) and len(ih) == 2 and len(il) == 2
+                  and ih[0] is Ellipsis and il[0] is Ellipsis and isinstance(ih[1], slice) and isinstance(il[1], slice)
+                  and ih[1].stop is None and il[1].start is None and ih[1].start == il[1].stop
+                  and ih[1].step is None and il[1].step is None)
+            interior = [a, b, cat, parts[0], hi, lo]
+            if not ok or any(len(n.users) != 1 for n in interior):
+                continue
+            roots[add] = (x, cos, sin, ih[1].start)
+            skip.update(interior)
+            break
+    return roots, skip
+
+
+def lower_rope(L, node, x_node, cos_node, sin_node, half):
+    x, cos, sin = L.arg(x_node), L.arg(cos_node), L.arg(sin_node)
+    if x.buf.dim() != 4 or x.shape[-1] != 2 * half or x.buf.stride(3) != 1:
+        raise Unsupported("rotary embedding on a tensor of shape %s" % (x.shape,))
+    Bn, H, T, D = x.shape                      # [B, H, T, D] view of a token-major projection
+    for t in (cos, sin):
+        if t.dtype != torch.float32 or t.buf.dim() != 2 or t.shape != (T, D) or t.buf.stride(1) != 1:
+            raise Unsupported("rotary tables must be fp32 [T, D], got %s %s" % (t.shape, t.dtype))
+        if t.req_grad:
+            raise Unsupported("trainable rotary tables")
+    out_dtype = L.cd if L.mixed else x.dtype
+    y = L.alloc((Bn, T, H, D), out_dtype)       # token-major like the projections
+    yv = y.permute(0, 2, 1, 3)
+    xs = (x.buf.stride(0), x.buf.stride(2), x.buf.stride(1))
+    ys = (yv.stride(0), yv.stride(2), yv.stride(1))
+    tab_ld = cos.buf.stride(0)
+    if sin.buf.stride(0) != tab_ld:
+        raise Unsupported("cos/sin tables with different row strides")
+    if x.dtype != out_dtype:
+        xin = L.alloc((Bn, T, H, D), out_dtype).permute(0, 2, 1, 3)
+        L.copy(x.buf, xin)
+        xs = (xin.stride(0), xin.stride(2), xin.stride(1))
+    else:
+        xin = x.buf
+    L.emit(L.kernels.rope(xin, yv, cos.buf, sin.buf, Bn, T, H, D, xs, ys, 0, tab_ld))
+    outv = Val(yv, req_grad=x.req_grad)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        if g.dtype != out_dtype or g.stride(3) != 1:
+            t = B.new_like(yv)
+            B.copy(g, t)
+            g = t
+        gs = (g.stride(0), g.stride(2), g.stride(1))
+        dst, prev = B.grad_target(x)
+        if prev is None and dst.dtype == out_dtype and dst.stride(3) == 1:
+            ds = (dst.stride(0), dst.stride(2), dst.stride(1))
+            B.emit(B.k.rope(g, dst, cos.buf, sin.buf, Bn, T, H, D, gs, ds, 1, tab_ld))
+        else:
+            tmp = B.new_like(yv)
+            B.emit(B.k.rope(g, tmp, cos.buf, sin.buf, Bn, T, H, D, gs, (tmp.stride(0), tmp.stride(2), tmp.stride(1)),
+                            1, tab_ld))
+            if prev is None:
+                B.copy(tmp, dst)
+            elif prev is dst:
+                B.copy(tmp, dst, accumulate=True)
+            else:
+                B.copy(prev, dst)
+                B.copy(tmp, dst, accumulate=True)
+        B.commit(x, dst)
+
+    if x.req_grad:
+        L.add_backward(bwd)
+    return outv
+
+
 FUNCTION_HANDLERS = {
     F.linear: lower_linear, torch._C._nn.linear: lower_linear,
     F.layer_norm: lower_layer_norm, torch.layer_norm: lower_layer_norm,
-    F.rms_norm: lower_rms_norm,
+    F.rms_norm: lower_rms_norm, torch.rms_norm: lower_rms_norm,
     F.scaled_dot_product_attention: lower_sdpa, torch._C._nn.scaled_dot_product_attention: lower_sdpa,
     F.conv2d: lower_conv2d, torch.conv2d: lower_conv2d,
     F.gelu: lower_act_maybe_gate, torch._C._nn.gelu: lower_act_maybe_gate,

@@ -88,7 +88,7 @@ _SIGNATURES = {
     "pf_cast": [_P, _I, _P, _I, _L, _P],
     "pf_fill": [_P, _I, _F, _L, _P],
     "pf_copy_strided": [_P, _I, POINTER(c_int64), _P, _I, POINTER(c_int64), POINTER(c_int64), _I, _I, _P],
-    "pf_rope": [_P, _P, _I, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P],
+    "pf_rope": [_P, _P, _I, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P],
     "pf_grad_accumulate_f32": [_P, _P, _I, _L, _P],
     "pf_split_gather": [_P, _P, _L, _L, _L, _P, _P],
     "pf_merge_scatter": [_P, _P, _L, _L, _L, _P, _P],
@@ -310,9 +310,10 @@ class HipKernels:
         args = (_ptr(src), _dt(src), ss, _ptr(dst), _dt(dst), ds, sz, nd, int(accumulate))
         return self._prep("pf_copy_strided", args, (src, dst, ss, ds, sz))
 
-    def rope(self, x, y, cos_t, sin_t, B, T, H, D, xs, ys, inverse):
-        args = (_ptr(x), _ptr(y), _dt(x), _ptr(cos_t), _ptr(sin_t), B, T, H, D, xs[0], xs[1], xs[2], ys[0], ys[1],
-                ys[2], int(inverse))
+    def rope(self, x, y, cos_t, sin_t, B, T, H, D, xs, ys, inverse, tab_ld=None):
+        tab_ld = D // 2 if tab_ld is None else tab_ld
+        args = (_ptr(x), _ptr(y), _dt(x), _ptr(cos_t), _ptr(sin_t), tab_ld, B, T, H, D, xs[0], xs[1], xs[2], ys[0],
+                ys[1], ys[2], int(inverse))
         return self._prep("pf_rope", args, (x, y, cos_t, sin_t))
 
     def grad_accumulate(self, acc, g, n):

@@ -151,3 +151,96 @@ def test_loss_wrappers_match_torch():
     s.backward()
     torch.testing.assert_close(s, x.detach().sum(), rtol=1e-5, atol=1e-4)
     assert torch.equal(x.grad, torch.ones_like(x))
+
+
+def _check_grads(model, ref, mixed):
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        gp, gq = p.grad.float().cpu(), q.grad.float()
+        assert torch.isfinite(gp).all(), n
+        if mixed is None:
+            assert (gp - gq).abs().max() <= 1e-4 * gq.abs().max() + 1e-9, (n, float((gp - gq).abs().max()))
+        else:
+            rel = (gp - gq).norm() / (gq.norm() + 1e-12)
+            assert rel <= 2.5e-2, (n, float(rel))
+
+
+@pytest.mark.parametrize("mixed", [None, "bf16"])
+def test_llama_style_four_stages_looped(mixed):
+    """BASELINE config 2 at reduced width: Llama-style decoder, 4 stages looped over 2
+    pipeline ranks, micro-batch 2 x 8, next-token CE inside the last stage."""
+    import torch.nn.functional as F
+
+    from oracle.stage_oracle import run_pipeline_step
+    from pfeife_amd.bench_models.llama import LlamaConfig, LlamaForCausalLM, split_stages
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = LlamaConfig(vocab=512, dim=256, layers=4, heads=4, ffn=688, max_seq=128)
+    torch.manual_seed(0)
+    model = LlamaForCausalLM(cfg)
+    ref = copy.deepcopy(model)
+    g = torch.Generator().manual_seed(42)
+    ids = torch.randint(0, cfg.vocab, (16, 128), generator=g)
+    option = PipeOption(device_cnt=2, batch_cnt=8, batch_size=2, split_points=["layers.1", "layers.2", "layers.3"],
+                        mixed_precision=mixed, optimizer=dict(type="sgd", lr=0.0))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(tok):
+        loss = cmodel(tok, tok)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    losses = runner.step(ids.cuda())
+    torch.cuda.synchronize()
+
+    def shifted_ce(logits, tok):
+        return F.cross_entropy(logits[:, :-1, :].reshape(-1, logits.shape[-1]).float(), tok[:, 1:].reshape(-1))
+
+    adt = {"bf16": torch.bfloat16}.get(mixed)
+    want = run_pipeline_step(split_stages(ref, [1, 2, 3]), shifted_ce, ids, ids, 8, device_cnt=2, autocast_dtype=adt)
+    ltol = 1e-5 if mixed is None else 2e-2
+    for a, b in zip(losses, want):
+        assert abs(float(a) - float(b)) <= ltol * abs(float(b)), (float(a), float(b))
+    _check_grads(model, ref, mixed)
+
+
+@pytest.mark.parametrize("mixed", [None, "bf16"])
+def test_vit_g_block_share_head_dim_88(mixed):
+    """BASELINE config 3 at reduced depth: ViT-g/14 blocks (dim 1408, 16 heads of 88,
+    MLP 6144, 257 tokens) fed with activations, sum loss on the output."""
+    from oracle.stage_oracle import run_pipeline_step
+    from pfeife_amd.bench_models.vit import BlockStack, ViTConfig
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=224, patch_size=14, dim=1408, depth=2, heads=16, mlp_dim=6144)
+    torch.manual_seed(0)
+    model = BlockStack(cfg)
+    ref = copy.deepcopy(model)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(4, 257, 1408, generator=g)
+    up = torch.randn(4, 257, 1408, generator=g) * 1e-2   # supplied upstream gradient
+    option = PipeOption(device_cnt=1, batch_cnt=2, batch_size=2, mixed_precision=mixed,
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(act, grad_out):
+        out = cmodel(act)
+        loss = (out.float() * grad_out).sum()
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    losses = runner.step(x.cuda(), up.cuda())
+    torch.cuda.synchronize()
+    adt = {"bf16": torch.bfloat16}.get(mixed)
+    want = run_pipeline_step([ref], lambda o, t: (o.float() * t).sum(), x, up, 2, device_cnt=1, autocast_dtype=adt)
+    ltol = 1e-4 if mixed is None else 2e-2
+    for a, b in zip(losses, want):
+        assert abs(float(a) - float(b)) <= ltol * abs(float(b)) + 1e-3, (float(a), float(b))
+    _check_grads(model, ref, mixed)
