@@ -106,11 +106,24 @@ __device__ __forceinline__ int gemm_tile_id(int tiles, int per_xcd) {
   return t < tiles ? t : -1;
 }
 
+// Tile id -> (tile row, tile column) in grouped order: ids walk down GROUP_M tile
+// rows before moving to the next tile column, so the ~32-64 workgroups an XCD runs
+// at the same time cover a compact patch of C and share their A rows and B columns
+// through that XCD's L2 instead of streaming whole operands from HBM.
+constexpr int GROUP_M = 8;
+__device__ __forceinline__ void gemm_tile_rc(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int per_group = GROUP_M * tiles_n;
+  const int group = t / per_group;
+  const int first_m = group * GROUP_M;
+  const int gm = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
+  const int r = t - group * per_group;
+  tm = first_m + r % gm;
+  tn = r / gm;
+}
+
 // ---------------------------------------------------------------------------
 // 16-bit MFMA kernel
 // ---------------------------------------------------------------------------
-constexpr int BK = 64;           // reduction elements per LDS tile
-constexpr int LDS_LD = BK + 8;   // padded LDS row (halves): 144 B keeps 16-byte reads conflict-free
 constexpr int EPI_LD = 40;       // floats per row of the 32x32 epilogue staging tile
 
 template <int N, class F>
@@ -135,71 +148,116 @@ template <> struct Mfma<PF_BF16> {
   }
 };
 
-// Global -> register staging of one operand tile (R rows of the output dimension x BK).
-//   TRANS = false: stored [row][k]  -> R/32 16-byte vectors per thread
-//   TRANS = true : stored [k][row]  -> one 8x8 block (8 vectors) per participating thread
-template <int R, bool TRANS> struct Stage;
+// Global -> register -> LDS staging of one operand tile: R rows of the output
+// dimension x BK reduction elements, LDS rows padded by 8 halves (16 bytes) so
+// that the 16-byte fragment reads are bank-conflict free.
+//   TRANS = false: stored [row][k]  -> R*BK/2048 16-byte vectors per thread
+//   TRANS = true : stored [k][row]  -> one 8(k) x 8(row) block (8 vectors) per participating
+//                                      thread, transposed in registers before the LDS store
+// Loads are raw buffer loads (buffer_load_dwordx4) on a descriptor whose extent
+// is the operand's valid byte range: rows past the end of the matrix come back
+// as zeros from the hardware range check, with no branch and a single 32-bit
+// offset register per vector, so a whole tile's loads are in flight together.
+// Only the reduction tail (K not a multiple of BK, last tile) is masked in
+// software, at LDS-store time.
+typedef int v4i_t __attribute__((ext_vector_type(4)));
 
-template <int R> struct Stage<R, false> {
-  static constexpr int NV = R / 32;  // R*8 vectors over 256 threads
-  static __device__ __forceinline__ void load(uint4 (&v)[8], const uint16_t* base, int64_t ld, int64_t r0,
-                                              int64_t R_total, int64_t k0, int64_t K, int tid, int /*first*/) {
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
+  const v4i_t x = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
+  return make_uint4((uint32_t)x.x, (uint32_t)x.y, (uint32_t)x.z, (uint32_t)x.w);
+}
+
+template <int R, int BK, int NT, bool TRANS> struct Stage;
+
+template <int R, int BK, int NT> struct Stage<R, BK, NT, false> {
+  static constexpr int LD = BK + 8;
+  static constexpr int VPR = BK / 8;              // vectors per row
+  static constexpr int NV = R * VPR / NT;         // vectors per thread
+  static constexpr int NBLK = 0;                  // (transposing path only)
+  static constexpr int NREG = NV;
+  static_assert(NV >= 1 && NV <= 8 && NV * NT == R * VPR, "tile does not divide over the workgroup");
+  // readable bytes of an R_total x K operand with row stride ld: whole 16-byte vectors (ld is a
+  // multiple of 8 and >= K, so the last row's vector tail is inside the row pitch; the hardware
+  // range check works on whole dwords, an extent cut inside a vector would zero valid elements)
+  static __device__ __forceinline__ uint32_t extent(int64_t R_total, int64_t K, int64_t ld) {
+    return (uint32_t)(((R_total - 1) * ld + (K + 7) / 8 * 8) * 2);
+  }
+  // byte offsets of this thread's vectors inside K-tile 0
+  static __device__ __forceinline__ void init(uint32_t (&off)[NV], int64_t ld, int64_t r0, int tid, int /*first*/) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int e = tid + i * 256;
-      const int row = e >> 3, kv = e & 7;
-      const int64_t gr = r0 + row, gk = k0 + kv * 8;
-      uint4 x = make_uint4(0, 0, 0, 0);
-      if (gr < R_total && gk < K) {
-        x = *(const uint4*)(base + gr * ld + gk);
-        if (gk + 8 > K) {  // K tail inside this vector: zero the elements >= K
-          uint32_t w[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            if (gk + 2 * q >= K) w[q] = 0;
-            else if (gk + 2 * q + 1 >= K) w[q] &= 0xffffu;
-          }
-          x = make_uint4(w[0], w[1], w[2], w[3]);
-        }
-      }
-      v[i] = x;
+      const int e = tid + i * NT;
+      off[i] = (uint32_t)(((r0 + e / VPR) * ld + (e % VPR) * 8) * 2);
     }
   }
-  static __device__ __forceinline__ void store(const uint4 (&v)[8], uint16_t* s, int tid, int /*first*/) {
+  static __device__ __forceinline__ uint32_t tile_step(int64_t /*ld*/) { return BK * 2; }
+  static __device__ __forceinline__ void load(uint4 (&v)[NV], __amdgpu_buffer_rsrc_t rs, const uint32_t (&off)[NV],
+                                              uint32_t adv, int /*tid*/, int /*first*/) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) v[i] = buf_load16(rs, off[i] + adv);
+  }
+  static __device__ __forceinline__ void store(const uint4 (&v)[NV], uint16_t* s, int64_t k0, int64_t K, int tid,
+                                               int /*first*/) {
+    const bool tail = k0 + BK > K;  // workgroup-uniform: only the last K-tile of a ragged K
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int e = tid + i * 256;
-      const int row = e >> 3, kv = e & 7;
-      *(uint4*)(s + row * LDS_LD + kv * 8) = v[i];
+      const int e = tid + i * NT;
+      const int row = e / VPR, kv = e % VPR;
+      uint4 x = v[i];
+      if (tail) {
+        const int64_t gk = k0 + kv * 8;
+        uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          if (gk + 2 * q >= K) w[q] = 0;
+          else if (gk + 2 * q + 1 >= K) w[q] &= 0xffffu;
+        }
+        x = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+      *(uint4*)(s + row * LD + kv * 8) = x;
     }
   }
 };
 
-template <int R> struct Stage<R, true> {
-  // R/8 x 8 blocks of 8(k) x 8(row) elements; one block per thread, R <= 256.
-  static constexpr int NBLK = R;  // (R/8) * (BK/8)
-  // `first` = id of the first participating thread (lets A and B use disjoint threads)
-  static __device__ __forceinline__ void load(uint4 (&v)[8], const uint16_t* base, int64_t ld, int64_t r0,
-                                              int64_t R_total, int64_t k0, int64_t K, int tid, int first) {
-    const int b = tid - first;
-    const bool mine = b >= 0 && b < NBLK;
-    const int rb = b % (R / 8), kb = b / (R / 8);
-    const int64_t gr = r0 + rb * 8;
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const int64_t gk = k0 + kb * 8 + r;
-      uint4 x = make_uint4(0, 0, 0, 0);
-      // rows of the output dimension beyond R_total only feed output rows that
-      // are never stored, but the read itself must stay inside the allocation:
-      // ld is a multiple of 8 and >= R_total, so gr + 8 <= ld whenever gr < R_total.
-      if (mine && gk < K && gr < R_total) x = *(const uint4*)(base + gk * ld + gr);
-      v[r] = x;
-    }
+template <int R, int BK, int NT> struct Stage<R, BK, NT, true> {
+  static constexpr int LD = BK + 8;
+  static constexpr int KB = BK / 8;                 // 8(k) x 8(row) blocks along k
+  static constexpr int NBLK = (R / 8) * KB;         // one block per participating thread
+  static constexpr int NREG = 8;
+  static_assert(NBLK <= NT, "tile too large for one transposing block per thread");
+  // readable bytes of a K x R_total operand with row stride ld (whole vectors): rows k >= K
+  // are out of range and come back as zeros
+  static __device__ __forceinline__ uint32_t extent(int64_t R_total, int64_t K, int64_t ld) {
+    return (uint32_t)(((K - 1) * ld + (R_total + 7) / 8 * 8) * 2);
   }
-  static __device__ __forceinline__ void store(const uint4 (&v)[8], uint16_t* s, int tid, int first) {
+  // `first` = id of the first participating thread (lets A and B use disjoint threads).
+  // Consecutive threads take consecutive k-blocks of the same 8 rows: their LDS stores
+  // then fall into one LDS row each (16 contiguous bytes per thread, no bank conflicts),
+  // and the 8 threads that share a k-row cover 128 contiguous bytes of it in global memory.
+  static __device__ __forceinline__ void init(uint32_t (&off)[8], int64_t ld, int64_t r0, int tid, int first) {
+    const int b = tid - first;
+    const int kb = b % KB, rb = b / KB;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) off[r] = (uint32_t)((((int64_t)kb * 8 + r) * ld + r0 + rb * 8) * 2);
+  }
+  static __device__ __forceinline__ uint32_t tile_step(int64_t ld) { return (uint32_t)(BK * ld * 2); }
+  static __device__ __forceinline__ void load(uint4 (&v)[8], __amdgpu_buffer_rsrc_t rs, const uint32_t (&off)[8],
+                                              uint32_t adv, int tid, int first) {
+    const int b = tid - first;
+    if (b < 0 || b >= NBLK) return;  // wavefront-uniform when NBLK is a multiple of 64
+    // columns beyond R_total inside a valid row read neighbouring data; they only feed
+    // output rows/columns that are never stored
+#pragma unroll
+    for (int r = 0; r < 8; ++r) v[r] = buf_load16(rs, off[r] + adv);
+  }
+  static __device__ __forceinline__ void store(const uint4 (&v)[8], uint16_t* s, int64_t /*k0*/, int64_t /*K*/,
+                                               int tid, int first) {
     const int b = tid - first;
     if (b < 0 || b >= NBLK) return;
-    const int rb = b % (R / 8), kb = b / (R / 8);
+    const int kb = b % KB, rb = b / KB;
     // 8x8 transpose of 16-bit values: 2x2 transposes inside 32-bit words, the
     // 4x4 transpose of the words is pure register renaming.
     const uint32_t in[8][4] = {{v[0].x, v[0].y, v[0].z, v[0].w}, {v[1].x, v[1].y, v[1].z, v[1].w},
@@ -215,21 +273,31 @@ template <int R> struct Stage<R, true> {
         lo[I] = (a & 0xffffu) | (c << 16);          // (k=2I, row 2J), (k=2I+1, row 2J)
         hi[I] = (a >> 16) | (c & 0xffff0000u);      // (k=2I, row 2J+1), (k=2I+1, row 2J+1)
       }
-      *(uint4*)(s + (rb * 8 + 2 * J) * LDS_LD + kb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-      *(uint4*)(s + (rb * 8 + 2 * J + 1) * LDS_LD + kb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+      *(uint4*)(s + (rb * 8 + 2 * J) * LD + kb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      *(uint4*)(s + (rb * 8 + 2 * J + 1) * LD + kb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
     }
   }
 };
 
-template <int DT, int BM, int BN, bool AT, bool BT>
-__global__ __launch_bounds__(256) void gemm16_kernel(const pf_gemm_desc p, const GemmGrid g) {
-  constexpr int WM = BM / 2, WN = BN / 2;  // per-wavefront sub-tile
+// Software pipeline: global loads run TWO K-tiles ahead of the MFMAs (two sets of
+// staging registers, two LDS buffers).  While tile kt is multiplied out of LDS,
+// tile kt+1 is already in registers (or landing) and tile kt+2 is being issued,
+// which covers the ~1 us L2/HBM latency at two workgroups per CU.
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, bool AT, bool BT>
+__global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)) ? 1 : 2)) void gemm16_kernel(const pf_gemm_desc p,
+                                                                                              const GemmGrid g) {
+  constexpr int NT = 64 * WGM * WGN;           // threads: WGM x WGN wavefronts
+  constexpr int WM = BM / WGM, WN = BN / WGN;  // per-wavefront sub-tile
   constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int LD = BK + 8;
+  using SA = Stage<BM, BK, NT, AT>;
+  using SB = Stage<BN, BK, NT, BT>;
   extern __shared__ __align__(16) uint16_t smem[];
 
   const int t = gemm_tile_id(g.tiles_m * g.tiles_n, g.per_xcd);
   if (t < 0) return;
-  const int tm = t % g.tiles_m, tn = t / g.tiles_m;
+  int tm, tn;
+  gemm_tile_rc(t, g.tiles_m, g.tiles_n, tm, tn);
   const int64_t M = p.M, N = p.N, K = p.K, lda = p.lda, ldb = p.ldb;
   const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
   const int64_t z = blockIdx.y, z1 = z / p.batch2, z2 = z % p.batch2;
@@ -240,10 +308,10 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const pf_gemm_desc p, const
   const int vec_epi = g.vec_epi;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm0 = (wave >> 1) * WM, wn0 = (wave & 1) * WN;
+  const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
   // disjoint loader threads when both operands take the transposing path
   constexpr int A_FIRST = 0;
-  constexpr int B_FIRST = (AT && BT && (BM + BN <= 256)) ? (256 - BN) : 0;
+  constexpr int B_FIRST = (AT && BT && (SA::NBLK + SB::NBLK <= NT)) ? (NT - SB::NBLK) : 0;
 
   float16_t acc[TM][TN];
 #pragma unroll
@@ -253,50 +321,77 @@ __global__ __launch_bounds__(256) void gemm16_kernel(const pf_gemm_desc p, const
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  uint4 ra[8], rb[8];
+  uint4 ra0[SA::NREG], rb0[SB::NREG], ra1[SA::NREG], rb1[SB::NREG];
+  uint32_t offa[SA::NREG], offb[SB::NREG];
   const int nk = (int)((K + BK - 1) / BK);
-  constexpr int BUF = (BM + BN) * LDS_LD;
+  constexpr int BUF = (BM + BN) * LD;
+  uint16_t* const buf0 = smem;
+  uint16_t* const buf1 = smem + BUF;
+  const int frag_off = (lane & 31) * LD + (lane >> 5) * 8;
+  const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(A, SA::extent(M, K, lda));
+  const __amdgpu_buffer_rsrc_t rs_b = make_rsrc(B, SB::extent(N, K, ldb));
+  SA::init(offa, lda, m0, tid, A_FIRST);
+  SB::init(offb, ldb, n0, tid, B_FIRST);
+  const uint32_t step_a = SA::tile_step(lda), step_b = SB::tile_step(ldb);
 
-  Stage<BM, AT>::load(ra, A, lda, m0, M, 0, K, tid, A_FIRST);
-  Stage<BN, BT>::load(rb, B, ldb, n0, N, 0, K, tid, B_FIRST);
-  Stage<BM, AT>::store(ra, smem, tid, A_FIRST);
-  Stage<BN, BT>::store(rb, smem + BM * LDS_LD, tid, B_FIRST);
-  __syncthreads();
-
-  const int frag_off = (lane & 31) * LDS_LD + (lane >> 5) * 8;
-  for (int kt = 0; kt < nk; ++kt) {
-    const bool more = kt + 1 < nk;
-    if (more) {
-      const int64_t k0 = (int64_t)(kt + 1) * BK;
-      Stage<BM, AT>::load(ra, A, lda, m0, M, k0, K, tid, A_FIRST);
-      Stage<BN, BT>::load(rb, B, ldb, n0, N, k0, K, tid, B_FIRST);
-    }
-    const uint16_t* s_a = smem + (kt & 1) * BUF;
-    const uint16_t* s_b = s_a + BM * LDS_LD;
+  auto compute = [&](const uint16_t* s_a) {
+    const uint16_t* s_b = s_a + BM * LD;
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       uint4 fa[TM], fb[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = *(const uint4*)(s_a + (wm0 + i * 32) * LDS_LD + frag_off + kk * 16);
+      for (int i = 0; i < TM; ++i) fa[i] = *(const uint4*)(s_a + (wm0 + i * 32) * LD + frag_off + kk * 16);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb[j] = *(const uint4*)(s_b + (wn0 + j * 32) * LDS_LD + frag_off + kk * 16);
+      for (int j = 0; j < TN; ++j) fb[j] = *(const uint4*)(s_b + (wn0 + j * 32) * LD + frag_off + kk * 16);
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = Mfma<DT>::run(fa[i], fb[j], acc[i][j]);
     }
-    if (more) {
-      uint16_t* s = smem + ((kt + 1) & 1) * BUF;
-      Stage<BM, AT>::store(ra, s, tid, A_FIRST);
-      Stage<BN, BT>::store(rb, s + BM * LDS_LD, tid, B_FIRST);
+  };
+
+  SA::load(ra0, rs_a, offa, 0, tid, A_FIRST);
+  SB::load(rb0, rs_b, offb, 0, tid, B_FIRST);
+  if (nk > 1) {
+    SA::load(ra1, rs_a, offa, step_a, tid, A_FIRST);
+    SB::load(rb1, rs_b, offb, step_b, tid, B_FIRST);
+  }
+  SA::store(ra0, buf0, 0, K, tid, A_FIRST);
+  SB::store(rb0, buf0 + BM * LD, 0, K, tid, B_FIRST);
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; kt += 2) {
+    // even phase: tile kt is in buf0, tile kt+1 is in (or landing in) set 1, set 0 is free
+    if (kt + 2 < nk) {
+      SA::load(ra0, rs_a, offa, (uint32_t)(kt + 2) * step_a, tid, A_FIRST);
+      SB::load(rb0, rs_b, offb, (uint32_t)(kt + 2) * step_b, tid, B_FIRST);
+    }
+    compute(buf0);
+    if (kt + 1 < nk) {
+      const int64_t k1 = (int64_t)(kt + 1) * BK;
+      SA::store(ra1, buf1, k1, K, tid, A_FIRST);
+      SB::store(rb1, buf1 + BM * LD, k1, K, tid, B_FIRST);
+    }
+    __syncthreads();
+    if (kt + 1 >= nk) break;
+    // odd phase: tile kt+1 is in buf1, tile kt+2 is landing in set 0, set 1 is free
+    if (kt + 3 < nk) {
+      SA::load(ra1, rs_a, offa, (uint32_t)(kt + 3) * step_a, tid, A_FIRST);
+      SB::load(rb1, rs_b, offb, (uint32_t)(kt + 3) * step_b, tid, B_FIRST);
+    }
+    compute(buf1);
+    if (kt + 2 < nk) {
+      const int64_t k2 = (int64_t)(kt + 2) * BK;
+      SA::store(ra0, buf0, k2, K, tid, A_FIRST);
+      SB::store(rb0, buf0 + BM * LD, k2, K, tid, B_FIRST);
     }
     __syncthreads();
   }
 
   // Epilogue.  D layout of v_mfma_f32_32x32x*: lane l holds column (l % 32) and
   // rows 8*(r/4) + 4*(l/32) + (r%4), r = 0..15.  Each wavefront re-lays one
-  // 32x32 tile at a time through its private LDS patch; afterwards lane l owns
-  // row l/2, columns 16*(l%2) .. +16 of the tile.
+  // row of TN 32x32 tiles at a time through its private LDS patch; afterwards
+  // lane l owns row l/2, columns 16*(l%2) .. +16 of each tile.
   float* stage = (float*)smem + wave * (TN * 32 * EPI_LD);
   const int wr_off = ((lane >> 5) * 4) * EPI_LD + (lane & 31);
   const int rd_row = lane >> 1, rd_col = (lane & 1) * 16;
@@ -345,7 +440,8 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const pf_gemm_desc p, const
 
   const int t = gemm_tile_id(g.tiles_m * g.tiles_n, g.per_xcd);
   if (t < 0) return;
-  const int tm = t % g.tiles_m, tn = t / g.tiles_m;
+  int tm, tn;
+  gemm_tile_rc(t, g.tiles_m, g.tiles_n, tm, tn);
   const int64_t M = p.M, N = p.N, K = p.K;
   const int a_trans = p.a_trans, b_trans = p.b_trans;
   const int64_t m0 = (int64_t)tm * TB, n0 = (int64_t)tn * TB;
@@ -407,8 +503,9 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const pf_gemm_desc p, const
 
 bool epi_ptr_ok(const void* p, int64_t ld) { return p == nullptr || (pf_aligned(p, 16) && ld % 8 == 0); }
 
-template <int DT, int BM, int BN>
+template <int DT, int BM, int BN, int BK, int WGM, int WGN>
 int launch16(const pf_gemm_desc& d, hipStream_t st) {
+  constexpr int NT = 64 * WGM * WGN;
   GemmGrid g;
   g.tiles_m = (int)((d.M + BM - 1) / BM);
   g.tiles_n = (int)((d.N + BN - 1) / BN);
@@ -418,18 +515,18 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
               (d.bias == nullptr || pf_aligned(d.bias, 16)) && epi_ptr_ok(d.aux_out, d.ld_aux_out) &&
               epi_ptr_ok(d.aux_in, d.ld_aux_in) && epi_ptr_ok(d.residual, d.ld_res);
   const dim3 grid((unsigned)(g.per_xcd * 8), (unsigned)(d.batch1 * d.batch2), 1);
-  size_t lds = 2 * (size_t)(BM + BN) * LDS_LD * sizeof(uint16_t);
-  const size_t lds_epi = 4 * (size_t)(BN / 64) * 32 * EPI_LD * sizeof(float);
+  size_t lds = 2 * (size_t)(BM + BN) * (BK + 8) * sizeof(uint16_t);
+  const size_t lds_epi = (size_t)(WGM * WGN) * (BN / WGN / 32) * 32 * EPI_LD * sizeof(float);
   if (lds < lds_epi) lds = lds_epi;
   if (lds > 64 * 1024) {  // opt in to the large LDS carve-out once per instantiation
     static bool raised[4] = {false, false, false, false};
     const int v = (d.a_trans ? 2 : 0) + (d.b_trans ? 1 : 0);
     if (!raised[v]) {
       hipError_t e = hipSuccess;
-      if (v == 0) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (v == 1) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (v == 2) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (v == 3) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (v == 0) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, BK, WGM, WGN, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (v == 1) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, BK, WGM, WGN, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (v == 2) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, BK, WGM, WGN, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (v == 3) e = hipFuncSetAttribute((const void*)gemm16_kernel<DT, BM, BN, BK, WGM, WGN, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) {
         pf_set_error("pf_gemm: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
         return PF_ERR_HIP;
@@ -438,7 +535,7 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
     }
   }
 #define PF_LAUNCH16(AT, BT)                                                                           \
-  hipLaunchKernelGGL((gemm16_kernel<DT, BM, BN, AT, BT>), grid, dim3(256), lds, st, d, g)
+  hipLaunchKernelGGL((gemm16_kernel<DT, BM, BN, BK, WGM, WGN, AT, BT>), grid, dim3(NT), lds, st, d, g)
   if (!d.a_trans && !d.b_trans) PF_LAUNCH16(false, false);
   else if (!d.a_trans && d.b_trans) PF_LAUNCH16(false, true);
   else if (d.a_trans && !d.b_trans) PF_LAUNCH16(true, false);
@@ -448,26 +545,27 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
   return PF_OK;
 }
 
-// Tile choice: the largest tile that still yields at least ~one workgroup per
-// CU (256 CUs); small problems (attention heads, narrow projections) take
-// smaller tiles so the launch fills the chip.  tile = 0: 256x128, 1: 128x128,
-// 2: 128x64, 3: 64x64.
+// Tile choice.  Measured on MI355X these kernels are bound by L2 -> CU operand
+// traffic, which per FLOP halves when the tile edge doubles; 128x128 with two
+// workgroups resident per CU is the largest configuration that keeps its
+// accumulators, two sets of staging registers and the fragment registers inside
+// the register file, so it is the ceiling here.  Smaller tiles are for problems
+// that would otherwise leave most of the 256 CUs without a workgroup.
+//   0: 128x128   1: 128x64   2: 64x64      (BK 64, 4 wavefronts)
 int choose_tile(const pf_gemm_desc& d) {
   const int64_t nb = (d.batch1 > 0 ? d.batch1 : 1) * (d.batch2 > 0 ? d.batch2 : 1);
   auto tiles = [&](int bm, int bn) { return ((d.M + bm - 1) / bm) * ((d.N + bn - 1) / bn) * nb; };
-  if (tiles(256, 128) >= 512 && d.M >= 256) return 0;
-  if (tiles(128, 128) >= 256 && d.M >= 128 && d.N >= 128) return 1;
-  if (tiles(128, 64) >= 256 && d.M >= 128) return 2;
-  return 3;
+  if (tiles(128, 128) >= 256 && d.M >= 128 && d.N >= 128) return 0;
+  if (tiles(128, 64) >= 256 && d.M >= 128) return 1;
+  return 2;
 }
 
 template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
   switch (choose_tile(d)) {
-    case 0: return launch16<DT, 256, 128>(d, st);
-    case 1: return launch16<DT, 128, 128>(d, st);
-    case 2: return launch16<DT, 128, 64>(d, st);
-    default: return launch16<DT, 64, 64>(d, st);
+    case 0: return launch16<DT, 128, 128, 64, 2, 2>(d, st);
+    case 1: return launch16<DT, 128, 64, 64, 2, 2>(d, st);
+    default: return launch16<DT, 64, 64, 64, 2, 2>(d, st);
   }
 }
 
@@ -515,13 +613,28 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
   PF_REQUIRE(d.lda % 8 == 0 && d.ldb % 8 == 0, "pf_gemm: lda/ldb must be multiples of 8 for 16-bit operands");
   PF_REQUIRE(d.a_stride1 % 8 == 0 && d.a_stride2 % 8 == 0 && d.b_stride1 % 8 == 0 && d.b_stride2 % 8 == 0,
              "pf_gemm: batch strides of 16-bit operands must be multiples of 8");
+  // operands are addressed with 32-bit byte offsets inside a buffer descriptor
+  const int64_t a_bytes = ((d.a_trans ? d.K : d.M) + 256) * d.lda * 2, b_bytes = ((d.b_trans ? d.K : d.N) + 256) * d.ldb * 2;
+  PF_REQUIRE(a_bytes < (1ll << 31) && b_bytes < (1ll << 31),
+             "pf_gemm: a 16-bit operand (per batch entry) must be smaller than 2 GiB");
+  if (d.K == 0) {  // nothing to reduce: the fp32 kernel's epilogue-only path handles it
+    GemmGrid g;
+    const int64_t tm = (d.M + 63) / 64, tn = (d.N + 63) / 64;
+    g.tiles_m = (int)tm;
+    g.tiles_n = (int)tn;
+    g.per_xcd = (int)((tm * tn + 7) / 8);
+    g.vec_epi = 0;
+    hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(g.per_xcd * 8), (unsigned)nb, 1), dim3(256), 0, st, d, g);
+    PF_CHECK_LAUNCH("pf_gemm(K=0)");
+    return PF_OK;
+  }
   if (d.in_dtype == PF_F16) return dispatch16<PF_F16>(d, st);
   return dispatch16<PF_BF16>(d, st);
 }
 
 extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   PF_REQUIRE(desc && out && cap > 0, "pf_gemm_variant: bad arguments");
-  static const char* tile_names[4] = {"256, 128", "128, 128", "128, 64", "64, 64"};
+  static const char* tile_names[3] = {"128, 128, 64, 2, 2", "128, 64, 64, 2, 2", "64, 64, 64, 2, 2"};
   if (desc->in_dtype == PF_F32) {
     snprintf(out, (size_t)cap, "gemm32_kernel");
   } else {
