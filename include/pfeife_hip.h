@@ -134,20 +134,41 @@ int pf_layernorm_fwd(const void* x, int x_dtype, const float* gamma, const float
 int pf_layernorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
                      const float* mean, const float* rstd, const void* dx_add, int add_dtype, void* dx,
                      int dx_dtype, float* dgamma_acc, float* dbeta_acc, float* workspace, int64_t rows,
-                     int64_t d, void* stream);
+                     int64_t d, int defer_reduce, void* stream);
 /* RMSNorm: y = x * rsqrt(mean(x^2) + eps) * gamma.  rstd fp32 [rows].
  * Replaces the pow/mean/rsqrt/mul chain (or aten::rms_norm) of Llama-style blocks. */
 int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, void* y, int y_dtype, float* rstd,
                    int64_t rows, int64_t d, float eps, void* stream);
 int pf_rmsnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
                    const float* rstd, const void* dx_add, int add_dtype, void* dx, int dx_dtype,
-                   float* dgamma_acc, float* workspace, int64_t rows, int64_t d, void* stream);
+                   float* dgamma_acc, float* workspace, int64_t rows, int64_t d, int defer_reduce, void* stream);
 /* Number of fp32 workspace elements the column reductions below need. */
 int64_t pf_colreduce_workspace(int64_t rows, int64_t cols);
 /* acc[c] += sum_r x[r*ld + c]  (bias gradient; deterministic two-stage reduce).
  * Replaces the sum-to-size of aten::addmm's bias gradient + AccumulateGrad. */
 int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
-                         float* workspace, void* stream);
+                         float* workspace, int defer_reduce, void* stream);
+/* Deferred column reductions.  With defer_reduce != 0 the three functions above only
+ * write their per-workgroup partial rows into `workspace` (layout: norm backward
+ * [pf_norm_bwd_partials(rows)][2][d] = dgamma then dbeta partials; column sum
+ * [pf_colsum_partials(rows)][cols]) and skip the accumulate; one
+ * pf_colreduce_finalize_batch launch then finishes any number of them:
+ *   acc[c] += sum_{p < n_partials} ws[p*stride + c]   for c < cols, per item.
+ * A backward pass of one stage has ~8 such reductions per transformer block; batching
+ * them replaces hundreds of few-microsecond launches by one.  `items_dev` is an array
+ * in DEVICE memory.  No counterpart in the reference (it is AccumulateGrad of the bias
+ * and normalisation parameters, pfeife/mp/worker.py:1585-1587). */
+typedef struct pf_reduce_item {
+  const float* ws;
+  float* acc;
+  int32_t n_partials;
+  int32_t reserved;
+  int64_t stride;
+  int64_t cols;
+} pf_reduce_item;
+int pf_norm_bwd_partials(int64_t rows);
+int pf_colsum_partials(int64_t rows);
+int pf_colreduce_finalize_batch(const pf_reduce_item* items_dev, int n_items, int64_t max_cols, void* stream);
 
 /* ---- softmax / attention probabilities ------------------------------------
  * Row softmax over [rows, cols] fp32 scores (row stride ld_s) producing
@@ -211,6 +232,11 @@ int pf_bias_add(const void* x, int x_dtype, const void* bias, int bias_dtype, vo
 /* dtype conversion / copy of n contiguous elements (autocast's weight casts,
  * done once per optimiser step instead of once per micro-batch). */
 int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream);
+/* dst[c*ld_dst + r] = src[r*ld_src + c] with dtype conversion: the transposed 16-bit
+ * shadow of a weight matrix, made once per optimiser step, lets the input-gradient
+ * product dx = dy W read W with its reduction dimension contiguous. */
+int pf_transpose_cast(const void* src, int src_dtype, int64_t ld_src, void* dst, int dst_dtype, int64_t ld_dst,
+                      int64_t rows, int64_t cols, void* stream);
 /* dst[i] = value for n elements of a 4-byte or 2-byte float dtype
  * (optimizer.zero_grad(set_to_none=False), pfeife/mp/worker.py:583-597). */
 int pf_fill(void* dst, int dtype, float value, int64_t n, void* stream);

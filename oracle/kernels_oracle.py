@@ -77,7 +77,7 @@ class OracleKernels:
         getattr(self, name)(*a, **kw)(None)
 
     def colreduce_workspace(self, rows, cols):
-        return 1
+        return 2 * max(1, cols)
 
     def reduce_workspace(self, n):
         return 1
@@ -129,7 +129,22 @@ class OracleKernels:
 
         return launch
 
-    def layernorm_bwd(self, dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws, rows, d, _rms=False):
+    def norm_bwd_partials(self, rows):
+        return 1
+
+    def colsum_partials(self, rows):
+        return 1
+
+    def colreduce_finalize_batch(self, items):
+        def launch(stream=None):
+            for ws, off, n, stride, cols, acc in items:
+                part = _strided(ws, (n, cols), (stride, 1)) if off == 0 else torch.as_strided(
+                    ws, (n, cols), (stride, 1), ws.storage_offset() + off)
+                _flat(acc, cols).add_(part.sum(dim=0))
+
+        return launch
+
+    def layernorm_bwd(self, dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws, rows, d, defer=0, _rms=False):
         def launch(stream=None):
             DY = _rows(dy, rows, d, d).float()
             X = _rows(x, rows, d, d).float()
@@ -143,6 +158,10 @@ class OracleKernels:
             if dx_add is not None:
                 out = out + _rows(dx_add, rows, d, d).float()
             _rows(dx, rows, d, d).copy_(out.to(dx.dtype))
+            if defer:
+                _flat(ws, 2 * d)[:d].copy_((DY * xh).sum(dim=0))
+                _flat(ws, 2 * d)[d:].copy_(DY.sum(dim=0))
+                return
             if dgamma is not None:
                 _flat(dgamma, d).add_((DY * xh).sum(dim=0))
             if dbeta is not None:
@@ -159,11 +178,15 @@ class OracleKernels:
 
         return launch
 
-    def rmsnorm_bwd(self, dy, x, gamma, rstd, dx_add, dx, dgamma, ws, rows, d):
-        return self.layernorm_bwd(dy, x, gamma, None, rstd, dx_add, dx, dgamma, None, ws, rows, d, _rms=True)
+    def rmsnorm_bwd(self, dy, x, gamma, rstd, dx_add, dx, dgamma, ws, rows, d, defer=0):
+        return self.layernorm_bwd(dy, x, gamma, None, rstd, dx_add, dx, dgamma, None, ws, rows, d, defer=defer,
+                                  _rms=True)
 
-    def colsum_accumulate(self, x, rows, cols, ld, acc, ws):
+    def colsum_accumulate(self, x, rows, cols, ld, acc, ws, defer=0):
         def launch(stream=None):
+            if defer:
+                _flat(ws, cols).copy_(_rows(x, rows, cols, ld).float().sum(dim=0))
+                return
             _flat(acc, cols).add_(_rows(x, rows, cols, ld).float().sum(dim=0))
 
         return launch
@@ -297,6 +320,12 @@ class OracleKernels:
     def cast(self, src, dst, n):
         def launch(stream=None):
             _flat(dst, n).copy_(_flat(src, n).to(dst.dtype))
+
+        return launch
+
+    def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
+        def launch(stream=None):
+            _rows(dst, cols, rows, ld_dst).copy_(_rows(src, rows, cols, ld_src).t().to(dst.dtype))
 
         return launch
 

@@ -202,6 +202,26 @@ __global__ __launch_bounds__(EW_BLOCK) void copy_strided_raw_kernel(const U* src
   }
 }
 
+// dst[c, r] = src[r, c] with dtype conversion, 64x64 tiles through LDS so that both
+// the reads and the writes are contiguous runs of 64 elements
+__global__ __launch_bounds__(256) void transpose_cast_kernel(const void* src, int sdt, int64_t ld_src, void* dst,
+                                                             int ddt, int64_t ld_dst, int64_t rows, int64_t cols) {
+  __shared__ float tile[64][65];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t r = r0 + ty + i * 4, c = c0 + tx;
+    tile[ty + i * 4][tx] = (r < rows && c < cols) ? pf_load_as_f32(src, r * ld_src + c, sdt) : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t c = c0 + ty + i * 4, r = r0 + tx;
+    if (c < cols && r < rows) pf_store_from_f32(dst, c * ld_dst + r, ddt, tile[tx][ty + i * 4]);
+  }
+}
+
 // ---- rotary embedding --------------------------------------------------------
 // one thread per (b, t, h, i) pair index i < D/2
 __global__ __launch_bounds__(EW_BLOCK) void rope_kernel(const void* x, void* y, int dt, const float* cos_t,
@@ -302,6 +322,20 @@ extern "C" int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype,
   PF_REQUIRE(src && dst, "pf_cast: null pointer");
   Cast f{src, dst, src_dtype, dst_dtype};
   return ew_launch(f, n, al16(src) && al16(dst), (hipStream_t)stream, "pf_cast");
+}
+
+extern "C" int pf_transpose_cast(const void* src, int src_dtype, int64_t ld_src, void* dst, int dst_dtype,
+                                 int64_t ld_dst, int64_t rows, int64_t cols, void* stream) {
+  PF_REQUIRE(rows >= 0 && cols >= 0 && pf_is_float_dtype(src_dtype) && pf_is_float_dtype(dst_dtype),
+             "pf_transpose_cast: bad arguments");
+  if (rows == 0 || cols == 0) return PF_OK;
+  PF_REQUIRE(src && dst && ld_src >= cols && ld_dst >= rows, "pf_transpose_cast: bad operands");
+  const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
+  PF_REQUIRE(grid.y <= 65535, "pf_transpose_cast: too many rows");
+  hipLaunchKernelGGL(transpose_cast_kernel, grid, dim3(256), 0, (hipStream_t)stream, src, src_dtype, ld_src, dst,
+                     dst_dtype, ld_dst, rows, cols);
+  PF_CHECK_LAUNCH("pf_transpose_cast");
+  return PF_OK;
 }
 
 extern "C" int pf_fill(void* dst, int dtype, float value, int64_t n, void* stream) {

@@ -556,6 +556,9 @@ int choose_tile(const pf_gemm_desc& d) {
   const int64_t nb = (d.batch1 > 0 ? d.batch1 : 1) * (d.batch2 > 0 ? d.batch2 : 1);
   auto tiles = [&](int bm, int bn) { return ((d.M + bm - 1) / bm) * ((d.N + bn - 1) / bn) * nb; };
   if (tiles(128, 128) >= 256 && d.M >= 128 && d.N >= 128) return 0;
+  // weight-gradient products (both operands transposed) reduce over thousands of tokens and
+  // have few output tiles: the larger tile's operand reuse beats filling every CU
+  if (d.a_trans && d.b_trans && d.K >= 1024 && tiles(128, 128) >= 96 && d.M >= 128 && d.N >= 128) return 0;
   if (tiles(128, 64) >= 256 && d.M >= 128) return 1;
   return 2;
 }

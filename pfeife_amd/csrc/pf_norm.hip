@@ -244,13 +244,13 @@ int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, voi
 
 int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* gamma, const float* mean,
              const float* rstd, const void* dx_add, int add_dt, void* dx, int dx_dt, float* dgamma, float* dbeta,
-             float* ws, int64_t rows, int64_t d, int rms, hipStream_t st, const char* name) {
+             float* ws, int64_t rows, int64_t d, int rms, int defer, hipStream_t st, const char* name) {
   PF_REQUIRE(rows >= 0 && d > 0, "%s: bad shape", name);
   if (rows == 0) return PF_OK;
   PF_REQUIRE(dy && x && gamma && rstd && dx, "%s: null pointer", name);
   PF_REQUIRE(rms || mean, "%s: mean required", name);
   PF_REQUIRE(pf_is_float_dtype(dy_dt) && pf_is_float_dtype(x_dt) && pf_is_float_dtype(dx_dt), "%s: bad dtype", name);
-  const int want = (dgamma || dbeta) ? 1 : 0;
+  const int want = (dgamma || dbeta || defer) ? 1 : 0;
   if (want) PF_REQUIRE(ws, "%s: workspace required for parameter gradients", name);
   const int blocks = norm_bwd_blocks(rows);
   const bool v = vec_ok(dy, dy_dt, d) && vec_ok(x, x_dt, d) && vec_ok(dx, dx_dt, d) && vec_ok(gamma, PF_F32, d) &&
@@ -271,7 +271,7 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
   }
 #undef PF_NB
   PF_CHECK_LAUNCH(name);
-  if (want) {
+  if (want && !defer) {
     const dim3 fg((unsigned)((d + 31) / 32));
     if (dgamma) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws, blocks, 2 * d, d, dgamma);
     if (dbeta) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws + d, blocks, 2 * d, d, dbeta);
@@ -285,6 +285,47 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
 // fp32 elements needed by the two-stage column reductions over a [rows, cols]
 // matrix: the norm backward writes 2 partial rows per workgroup, the column sum
 // one partial row per row chunk.
+// One launch finishing many deferred column reductions: block (x, y) handles 32 columns
+// of item y.  Items live in device memory.
+__global__ __launch_bounds__(256) void colreduce_finalize_batch_kernel(const pf_reduce_item* items) {
+  __shared__ float red[8][32];
+  const pf_reduce_item it = items[blockIdx.y];
+  const int cl = threadIdx.x & 31, part = threadIdx.x >> 5;
+  const int64_t c = (int64_t)blockIdx.x * 32 + cl;
+  if ((int64_t)blockIdx.x * 32 >= it.cols) return;  // uniform over the block
+  float s = 0.f;
+  if (c < it.cols)
+    for (int p = part; p < it.n_partials; p += 8) s += it.ws[(int64_t)p * it.stride + c];
+  red[part][cl] = s;
+  __syncthreads();
+  if (part == 0 && c < it.cols) {
+    float t = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) t += red[q][cl];
+    it.acc[c] += t;
+  }
+}
+
+extern "C" int pf_norm_bwd_partials(int64_t rows) { return norm_bwd_blocks(rows < 1 ? 1 : rows); }
+
+extern "C" int pf_colsum_partials(int64_t rows) {
+  if (rows < 1) rows = 1;
+  int64_t chunks = colsum_chunks(rows);
+  const int64_t rpc = (rows + chunks - 1) / chunks;
+  return (int)((rows + rpc - 1) / rpc);
+}
+
+extern "C" int pf_colreduce_finalize_batch(const pf_reduce_item* items_dev, int n_items, int64_t max_cols,
+                                           void* stream) {
+  PF_REQUIRE(n_items >= 0 && max_cols >= 0, "pf_colreduce_finalize_batch: bad arguments");
+  if (n_items == 0 || max_cols == 0) return PF_OK;
+  PF_REQUIRE(items_dev != nullptr && n_items <= 65535, "pf_colreduce_finalize_batch: bad item list");
+  hipLaunchKernelGGL(colreduce_finalize_batch_kernel, dim3((unsigned)((max_cols + 31) / 32), (unsigned)n_items),
+                     dim3(256), 0, (hipStream_t)stream, items_dev);
+  PF_CHECK_LAUNCH("pf_colreduce_finalize_batch");
+  return PF_OK;
+}
+
 extern "C" int64_t pf_colreduce_workspace(int64_t rows, int64_t cols) {
   if (cols < 1) cols = 1;
   if (rows < 1) rows = 1;
@@ -304,9 +345,9 @@ extern "C" int pf_layernorm_fwd(const void* x, int x_dtype, const float* gamma, 
 extern "C" int pf_layernorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
                                 const float* mean, const float* rstd, const void* dx_add, int add_dtype, void* dx,
                                 int dx_dtype, float* dgamma_acc, float* dbeta_acc, float* workspace, int64_t rows,
-                                int64_t d, void* stream) {
+                                int64_t d, int defer_reduce, void* stream) {
   return norm_bwd(dy, dy_dtype, x, x_dtype, gamma, mean, rstd, dx_add, add_dtype, dx, dx_dtype, dgamma_acc,
-                  dbeta_acc, workspace, rows, d, 0, (hipStream_t)stream, "pf_layernorm_bwd");
+                  dbeta_acc, workspace, rows, d, 0, defer_reduce, (hipStream_t)stream, "pf_layernorm_bwd");
 }
 
 extern "C" int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, void* y, int y_dtype, float* rstd,
@@ -317,17 +358,18 @@ extern "C" int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, vo
 
 extern "C" int pf_rmsnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
                               const float* rstd, const void* dx_add, int add_dtype, void* dx, int dx_dtype,
-                              float* dgamma_acc, float* workspace, int64_t rows, int64_t d, void* stream) {
+                              float* dgamma_acc, float* workspace, int64_t rows, int64_t d, int defer_reduce,
+                              void* stream) {
   return norm_bwd(dy, dy_dtype, x, x_dtype, gamma, nullptr, rstd, dx_add, add_dtype, dx, dx_dtype, dgamma_acc,
-                  nullptr, workspace, rows, d, 1, (hipStream_t)stream, "pf_rmsnorm_bwd");
+                  nullptr, workspace, rows, d, 1, defer_reduce, (hipStream_t)stream, "pf_rmsnorm_bwd");
 }
 
 extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
-                                    float* workspace, void* stream) {
+                                    float* workspace, int defer_reduce, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   PF_REQUIRE(rows >= 0 && cols >= 0 && ld >= cols, "pf_colsum_accumulate: bad shape");
   if (rows == 0 || cols == 0) return PF_OK;
-  PF_REQUIRE(x && acc && workspace, "pf_colsum_accumulate: null pointer");
+  PF_REQUIRE(x && (acc || defer_reduce) && workspace, "pf_colsum_accumulate: null pointer");
   PF_REQUIRE(pf_is_float_dtype(x_dtype), "pf_colsum_accumulate: bad dtype");
   int64_t chunks = colsum_chunks(rows);
   const int64_t rpc = (rows + chunks - 1) / chunks;
@@ -341,6 +383,7 @@ extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, in
     hipLaunchKernelGGL(colsum_kernel<1>, grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc);
   }
   PF_CHECK_LAUNCH("pf_colsum_accumulate");
+  if (defer_reduce) return PF_OK;
   hipLaunchKernelGGL(colreduce_finalize_kernel, dim3((unsigned)((cols + 31) / 32)), dim3(256), 0, st, workspace,
                      (int)chunks, cols, cols, acc);
   PF_CHECK_LAUNCH("pf_colsum_accumulate(finalize)");

@@ -4,7 +4,7 @@
 
 #include "pf_common.h"
 
-#define PF_ABI_VERSION 1
+#define PF_ABI_VERSION 2
 
 static thread_local char g_err[512] = "";
 

@@ -64,6 +64,21 @@ class ParamStore:
             self._keep.append(tensor)
         return sh
 
+    def shadow_t(self, tensor, dtype):
+        """Transposed copy [cols, rows] of a 2-d parameter in `dtype`, refreshed once per step."""
+        key = (tensor.data_ptr(), tuple(tensor.shape), tensor.dtype, dtype, "T")
+        sh = self._shadow.get(key)
+        if sh is None:
+            rows, cols = tensor.shape
+            sh = torch.empty((cols, rows), dtype=dtype, device=tensor.device)
+            src = tensor.detach()
+            if not src.is_contiguous():
+                raise Unsupported("non-contiguous parameter %s" % (tuple(tensor.shape),))
+            self.refresh.append(self.kernels.transpose_cast(src, cols, sh, rows, rows, cols))
+            self._shadow[key] = sh
+            self._keep.append(tensor)
+        return sh
+
     def grad(self, param):
         g = self._grads.get(id(param))
         if g is None:
@@ -158,9 +173,16 @@ class BwdCtx:
         self.out = program.bwd
         self._seq = 0
         self._pending = {}
+        self.reduces = []   # deferred column reductions, finished by one batched launch at the end
 
     def emit(self, launch):
         self.out.append(launch)
+
+    def colsum_into(self, x, rows, cols, ld, acc):
+        """acc[c] += sum_r x[r, c] (bias gradient), reduction finished at the end of the job."""
+        ws = self.temp((self.k.colreduce_workspace(rows, cols),), torch.float32)
+        self.emit(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
+        self.reduces.append((ws, 0, self.k.colsum_partials(rows), cols, cols, acc))
 
     def new_like(self, like, private=False):
         if private:
@@ -383,6 +405,8 @@ class Lowerer:
                 B.contribute(v, g)
         for fn in reversed(prog.backward_fns):
             fn(B)
+        if B.reduces:
+            prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
         prog.input_grads = []
         for v in prog.inputs:
             if isinstance(v, Val) and v.req_grad and v.param is None:
@@ -501,6 +525,9 @@ def lower_linear(L, node):
     if not w_cd.is_contiguous():
         raise Unsupported("linear with a non-contiguous weight")
     b_cd = None if b is None else L.params.shadow(b.buf, cd)
+    # dx = dy W reads W along its rows; a transposed shadow keeps the reduction dimension
+    # contiguous for that product too (the weight is static within a step, the copy is made once)
+    w_t = L.params.shadow_t(w.buf, cd) if (x.req_grad and w.param is not None and M >= 256) else None
 
     # fusions: linear -> activation, or linear -> (+ residual)
     act, res, out_node = ACT_NONE, None, node
@@ -558,11 +585,14 @@ def lower_linear(L, node):
             B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
                             b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
-            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(M, N)))
+            B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:
             dst, prev = B.grad_target(x)
             dm = as_matrix(dst)
-            kw2 = dict(M=M, N=K, K=N, lda=ld_dy, ldb=K, b_trans=1)
+            if w_t is not None:
+                wb, kw2 = w_t, dict(M=M, N=K, K=N, lda=ld_dy, ldb=N, b_trans=0)
+            else:
+                wb, kw2 = w_cd, dict(M=M, N=K, K=N, lda=ld_dy, ldb=K, b_trans=1)
             if x.preact is not None and x_users == 1 and prev is None:
                 kw2.update(dact=x.preact[0], aux_in=x.preact[1], ld_aux_in=K)
                 x.grad_is_preact = True
@@ -574,12 +604,12 @@ def lower_linear(L, node):
                     if pm is None:
                         raise Unsupported("accumulating into a non-matrix gradient")
                     kw2.update(residual=prev, ld_res=pm[2])
-                B.emit(B.k.gemm(dy, w_cd, dst, ldc=dm[2], **kw2))
+                B.emit(B.k.gemm(dy, wb, dst, ldc=dm[2], **kw2))
                 B.commit(x, dst)
             else:
                 # target is not a plain matrix (e.g. a permuted view): go through a temp
                 tmp = B.temp(tuple(x.shape), x.dtype)
-                B.emit(B.k.gemm(dy, w_cd, tmp, ldc=K, **kw2))
+                B.emit(B.k.gemm(dy, wb, tmp, ldc=K, **kw2))
                 if prev is None:
                     B.copy(tmp, dst)
                 elif prev is dst:
@@ -638,7 +668,8 @@ def lower_layer_norm(L, node, rms=False):
             g = t
         dgamma = L.params.grad(gamma.param) if gamma.req_grad and gamma.param is not None else None
         dbeta = L.params.grad(beta.param) if beta is not None and beta.req_grad and beta.param is not None else None
-        ws = L.workspace(rows, d) if (dgamma is not None or dbeta is not None) else None
+        want = dgamma is not None or dbeta is not None
+        ws = B.temp((B.k.colreduce_workspace(rows, d),), torch.float32) if want else None
         if x.req_grad:
             dst, prev = B.grad_target(x)
             if not dst.is_contiguous() or (prev is not None and not prev.is_contiguous()):
@@ -646,9 +677,16 @@ def lower_layer_norm(L, node, rms=False):
         else:
             dst, prev = B.temp(x.shape, x.dtype), None
         if rms:
-            B.emit(B.k.rmsnorm_bwd(g, x.buf, g32, rstd, prev, dst, dgamma, ws, rows, d))
+            B.emit(B.k.rmsnorm_bwd(g, x.buf, g32, rstd, prev, dst, None, ws, rows, d, defer=1 if want else 0))
         else:
-            B.emit(B.k.layernorm_bwd(g, x.buf, g32, mean, rstd, prev, dst, dgamma, dbeta, ws, rows, d))
+            B.emit(B.k.layernorm_bwd(g, x.buf, g32, mean, rstd, prev, dst, None, None, ws, rows, d,
+                                     defer=1 if want else 0))
+        if want:
+            nb = B.k.norm_bwd_partials(rows)
+            if dgamma is not None:
+                B.reduces.append((ws, 0, nb, 2 * d, d, dgamma))
+            if dbeta is not None:
+                B.reduces.append((ws, d, nb, 2 * d, d, dbeta))
         if x.req_grad:
             B.commit(x, dst)
 
@@ -803,7 +841,7 @@ def lower_conv2d(L, node):
             B.emit(B.k.gemm(dy, cols, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
                             b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
-            B.emit(B.k.colsum_accumulate(dy, M, N, ld_dy, L.params.grad(b.param), L.workspace(M, N)))
+            B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:
             dcols = B.temp((M, K), cd)
             B.emit(B.k.gemm(dy, w_cd, dcols, M=M, N=K, K=N, lda=ld_dy, ldb=K, ldc=K, b_trans=1))

@@ -16,7 +16,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpfeife_hip.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 PF_F32, PF_F16, PF_BF16, PF_I64, PF_I32, PF_U8 = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU = 0, 1, 2, 3, 4
@@ -68,10 +68,13 @@ _SIGNATURES = {
     "pf_gemm": [POINTER(GemmDesc), _P],
     "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
     "pf_layernorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _F, _P],
-    "pf_layernorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P],
+    "pf_layernorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _L, _I, _P],
     "pf_rmsnorm_fwd": [_P, _I, _P, _P, _I, _P, _L, _L, _F, _P],
-    "pf_rmsnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _L, _L, _P],
-    "pf_colsum_accumulate": [_P, _I, _L, _L, _L, _P, _P, _P],
+    "pf_rmsnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _L, _L, _I, _P],
+    "pf_colsum_accumulate": [_P, _I, _L, _L, _L, _P, _P, _I, _P],
+    "pf_colreduce_finalize_batch": [_P, _I, _L, _P],
+    "pf_norm_bwd_partials": None,
+    "pf_colsum_partials": None,
     "pf_softmax_fwd": [_P, _L, _P, _I, _L, _L, _L, _L, _I, _P],
     "pf_softmax_bwd": [_P, _L, _P, _I, _L, _P, _I, _L, _L, _L, _F, _P],
     "pf_cross_entropy_fwd": [_P, _I, _P, _P, _P, _P, _L, _L, _L, _P],
@@ -86,6 +89,7 @@ _SIGNATURES = {
     "pf_axpby": [_P, _I, _F, _P, _I, _F, _P, _I, _L, _P],
     "pf_bias_add": [_P, _I, _P, _I, _P, _I, _L, _L, _P],
     "pf_cast": [_P, _I, _P, _I, _L, _P],
+    "pf_transpose_cast": [_P, _I, _L, _P, _I, _L, _L, _L, _P],
     "pf_fill": [_P, _I, _F, _L, _P],
     "pf_copy_strided": [_P, _I, POINTER(c_int64), _P, _I, POINTER(c_int64), POINTER(c_int64), _I, _I, _P],
     "pf_rope": [_P, _P, _I, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P],
@@ -120,7 +124,7 @@ def load(path=None):
     for name, args in _SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = c_int
-        fn.argtypes = args
+        fn.argtypes = args if args is not None else [c_int64]
     for name, args in _RET_I64.items():
         fn = getattr(lib, name)
         fn.restype = c_int64
@@ -223,23 +227,41 @@ class HipKernels:
         args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(beta), _ptr(y), _dt(y), _ptr(mean), _ptr(rstd), rows, d, eps)
         return self._prep("pf_layernorm_fwd", args, (x, gamma, beta, y, mean, rstd))
 
-    def layernorm_bwd(self, dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws, rows, d):
+    def layernorm_bwd(self, dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws, rows, d, defer=0):
         args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx_add), _dt(dx_add),
-                _ptr(dx), _dt(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), rows, d)
+                _ptr(dx), _dt(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), rows, d, int(defer))
         return self._prep("pf_layernorm_bwd", args, (dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws))
 
     def rmsnorm_fwd(self, x, gamma, y, rstd, rows, d, eps):
         args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(y), _dt(y), _ptr(rstd), rows, d, eps)
         return self._prep("pf_rmsnorm_fwd", args, (x, gamma, y, rstd))
 
-    def rmsnorm_bwd(self, dy, x, gamma, rstd, dx_add, dx, dgamma, ws, rows, d):
+    def rmsnorm_bwd(self, dy, x, gamma, rstd, dx_add, dx, dgamma, ws, rows, d, defer=0):
         args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(rstd), _ptr(dx_add), _dt(dx_add), _ptr(dx),
-                _dt(dx), _ptr(dgamma), _ptr(ws), rows, d)
+                _dt(dx), _ptr(dgamma), _ptr(ws), rows, d, int(defer))
         return self._prep("pf_rmsnorm_bwd", args, (dy, x, gamma, rstd, dx_add, dx, dgamma, ws))
 
-    def colsum_accumulate(self, x, rows, cols, ld, acc, ws):
-        args = (_ptr(x), _dt(x), rows, cols, ld, _ptr(acc), _ptr(ws))
+    def colsum_accumulate(self, x, rows, cols, ld, acc, ws, defer=0):
+        args = (_ptr(x), _dt(x), rows, cols, ld, _ptr(acc), _ptr(ws), int(defer))
         return self._prep("pf_colsum_accumulate", args, (x, acc, ws))
+
+    def norm_bwd_partials(self, rows):
+        return int(self.lib.pf_norm_bwd_partials(rows))
+
+    def colsum_partials(self, rows):
+        return int(self.lib.pf_colsum_partials(rows))
+
+    def colreduce_finalize_batch(self, items):
+        """items: [(ws_tensor, ws_offset_elems, n_partials, stride, cols, acc_tensor)]"""
+        if not items:
+            return lambda stream: None
+        rows = []
+        for ws, off, n, stride, cols, acc in items:
+            rows.append([ws.data_ptr() + 4 * off, acc.data_ptr(), int(n), int(stride), int(cols)])
+        table = torch.tensor(rows, dtype=torch.int64).to(items[0][0].device)
+        max_cols = max(r[4] for r in rows)
+        keep = (table,) + tuple(i[0] for i in items) + tuple(i[5] for i in items)
+        return self._prep("pf_colreduce_finalize_batch", (table.data_ptr(), len(rows), max_cols), keep)
 
     # -- softmax / losses ----------------------------------------------------------
     def softmax_fwd(self, s, ld_s, p, ld_p, rows, cols, q_len, causal):
@@ -299,6 +321,10 @@ class HipKernels:
 
     def cast(self, src, dst, n):
         return self._prep("pf_cast", (_ptr(src), _dt(src), _ptr(dst), _dt(dst), n), (src, dst))
+
+    def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
+        args = (_ptr(src), _dt(src), ld_src, _ptr(dst), _dt(dst), ld_dst, rows, cols)
+        return self._prep("pf_transpose_cast", args, (src, dst))
 
     def fill(self, dst, value, n):
         return self._prep("pf_fill", (_ptr(dst), _dt(dst), float(value), n), (dst,))

@@ -383,3 +383,42 @@ def test_embedding(hip, oracle, dtype):
     r = both(hip, oracle, "embedding_bwd", dict(dout=dout, ids=ids, dtable=rnd((vocab, dim), F32, 4)), ["dtable"],
              n_ids=n, dim=dim, vocab=vocab)
     close(r["dtable"], 1e-5, 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16, F32])
+def test_transpose_cast(hip, oracle, dtype):
+    for rows, cols in [(1024, 4096), (1000, 1024), (37, 5), (64, 64)]:
+        src = rnd((rows, cols), F32, 1)
+        r = both(hip, oracle, "transpose_cast", dict(src=src, dst=torch.zeros(cols, rows, dtype=dtype)), ["dst"],
+                 ld_src=cols, ld_dst=rows, rows=rows, cols=cols)
+        assert torch.equal(r["dst"][0], r["dst"][1])
+        assert torch.equal(r["dst"][0], src.t().to(dtype))
+
+
+def test_deferred_reductions_match_immediate(hip):
+    """Partials written with defer=1 and finished by one batched launch give bit-identical
+    accumulators to the immediate two-kernel path (same partials, same summation order)."""
+    rows, d = 3152, 1024
+    x = rnd((rows, d), F32, 1).cuda()
+    dy = rnd((rows, d), F16, 2).cuda()
+    gamma = (rnd((d,), F32, 3) + 1).cuda()
+    mean, rstd = x.mean(1), 1 / torch.sqrt(x.var(1, unbiased=False) + 1e-5)
+    need = hip.colreduce_workspace(rows, d)
+    outs = {}
+    for defer in (0, 1):
+        dx = torch.zeros(rows, d, device="cuda")
+        dg, db, bias = rnd((d,), F32, 4).cuda(), rnd((d,), F32, 5).cuda(), rnd((d,), F32, 6).cuda()
+        ws1, ws2 = torch.zeros(need, device="cuda"), torch.zeros(need, device="cuda")
+        if defer:
+            hip.run("layernorm_bwd", dy, x, gamma, mean, rstd, None, dx, None, None, ws1, rows, d, defer=1)
+            hip.run("colsum_accumulate", dy, rows, d, d, None, ws2, defer=1)
+            nb = hip.norm_bwd_partials(rows)
+            hip.run("colreduce_finalize_batch", [(ws1, 0, nb, 2 * d, d, dg), (ws1, d, nb, 2 * d, d, db),
+                                                 (ws2, 0, hip.colsum_partials(rows), d, d, bias)])
+        else:
+            hip.run("layernorm_bwd", dy, x, gamma, mean, rstd, None, dx, dg, db, ws1, rows, d)
+            hip.run("colsum_accumulate", dy, rows, d, d, bias, ws2)
+        torch.cuda.synchronize()
+        outs[defer] = (dx.cpu(), dg.cpu(), db.cpu(), bias.cpu())
+    for a, b in zip(outs[0], outs[1]):
+        assert torch.equal(a, b)
