@@ -182,6 +182,32 @@ int pf_softmax_fwd(const float* s, int64_t ld_s, void* p, int p_dtype, int64_t l
 int pf_softmax_bwd(const float* dp, int64_t ld_dp, const void* p, int p_dtype, int64_t ld_p, void* ds,
                    int ds_dtype, int64_t ld_ds, int64_t rows, int64_t cols, float scale, void* stream);
 
+/* Fused attention: O = softmax(Q K^T * scale [causal]) V and its backward, without the
+ * [B,H,Tq,Tk] score matrices in memory.  q/k/v/o and the gradients are [B, H, T, hd]
+ * tensors (fp16 or bf16) addressed with ELEMENT strides (batch, head, token) and unit
+ * stride along hd, so that heads may sit inside a packed qkv projection.  lse: fp32
+ * [B,H,Tq] (written by forward, read by backward); delta: fp32 [B,H,Tq] scratch written
+ * and read by backward.  hd must be a multiple of 8 and <= 96 (PF_ERR_UNSUPPORTED
+ * otherwise: the caller then uses pf_gemm + pf_softmax).  causal: key j is visible to
+ * query i iff j <= i + (Tk - Tq).
+ * Replaces aten::scaled_dot_product_attention and its backward inside a stage
+ * (pfeife/mp/worker.py:1494, :1585-1587). */
+typedef struct pf_attn_desc {
+  int32_t dtype, B, H, Tq, Tk, hd, causal, reserved;
+  float scale;
+  float reserved2;
+  const void* q; const void* k; const void* v;
+  void* o;            /* forward: written; backward: read */
+  const void* d_o;
+  void* dq; void* dk; void* dv;
+  float* lse;
+  float* delta;
+  int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, o_st;
+  int64_t do_sb, do_sh, do_st, dq_sb, dq_sh, dq_st, dk_sb, dk_sh, dk_st, dv_sb, dv_sh, dv_st;
+} pf_attn_desc;
+int pf_attention_fwd(const pf_attn_desc* desc, void* stream);
+int pf_attention_bwd(const pf_attn_desc* desc, void* stream);
+
 /* ---- losses (pfeife/loss.py:53-70 CrossEntropyLoss / HFCrossEntropyLoss; the
  * mean-reduced nn.CrossEntropyLoss they wrap) -------------------------------
  * logits [rows, classes] (dtype l_dtype, contiguous), targets int64 [rows];

@@ -113,6 +113,45 @@ class OracleKernels:
 
         return launch
 
+    # -- fused attention -----------------------------------------------------------
+    MAX_FUSED_HEAD_DIM = 96
+
+    @staticmethod
+    def _attn_scores(q, k, scale, causal):
+        Tq, Tk = q.shape[2], k.shape[2]
+        s = torch.matmul(q.float(), k.float().transpose(-1, -2)) * scale
+        if causal:
+            i = torch.arange(Tq, device=s.device)[:, None]
+            j = torch.arange(Tk, device=s.device)[None, :]
+            s = s.masked_fill(j > i + (Tk - Tq), float("-inf"))
+        return s
+
+    def attention_fwd(self, q, k, v, o, lse, scale, causal):
+        def launch(stream=None):
+            s = self._attn_scores(q, k, scale, causal)
+            l = torch.logsumexp(s, dim=-1)
+            p = torch.exp(s - l[..., None]).to(q.dtype).float()   # probabilities enter the PV product in 16 bits
+            o.copy_(torch.matmul(p, v.float()).to(o.dtype))
+            lse.copy_(l)
+
+        return launch
+
+    def attention_bwd(self, q, k, v, o, d_o, lse, delta, dq, dk, dv, scale, causal):
+        def launch(stream=None):
+            s = self._attn_scores(q, k, scale, causal)
+            p = torch.exp(s - lse[..., None].float())
+            do = d_o.float()
+            dlt = (do * o.float()).sum(dim=-1)
+            delta.copy_(dlt)
+            dp = torch.matmul(do, v.float().transpose(-1, -2))
+            ds = (p * (dp - dlt[..., None]) * scale).to(q.dtype).float()
+            p16 = p.to(q.dtype).float()
+            dq.copy_(torch.matmul(ds, k.float()).to(dq.dtype))
+            dk.copy_(torch.matmul(ds.transpose(-1, -2), q.float()).to(dk.dtype))
+            dv.copy_(torch.matmul(p16.transpose(-1, -2), do).to(dv.dtype))
+
+        return launch
+
     # -- normalisation -----------------------------------------------------------
     def layernorm_fwd(self, x, gamma, beta, y, mean, rstd, rows, d, eps):
         def launch(stream=None):

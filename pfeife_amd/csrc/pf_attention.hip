@@ -1,0 +1,526 @@
+// Fused attention (forward, dQ, dK/dV) on gfx950 MFMA: softmax(Q K^T * scale [+ causal]) V
+// without materialising the [B,H,Tq,Tk] score / probability matrices.
+//
+// All three kernels work in the "transposed world": score tiles are computed so that a
+// lane owns ONE column of the tile (lane % 32) and 16 rows of it in registers.  The
+// softmax statistics of that column are then a per-lane loop plus one exchange with
+// lane ^ 32, and the probabilities can be fed straight back into the next MFMA as the
+// B operand (the MFMA reduction index may be permuted freely as long as A and B agree),
+// so P never goes through LDS.
+//
+//   forward / dQ kernel : tile = S^T[kv][q], column = query row   (workgroup = 128 queries)
+//   dK/dV kernel        : tile = S[q][kv],   column = key row     (workgroup = 128 keys)
+//
+// Operands whose MFMA reduction index is NOT their contiguous dimension (V in forward,
+// K in dQ, Q and dO in dK/dV) are transposed in registers (8x8 blocks) on their way
+// into LDS, like the GEMM's transposing loader.
+//
+// Q, K, V, O and their gradients are [B, H, T, hd] tensors addressed with element
+// strides (batch, head, token) and unit stride along hd, so heads can live inside a
+// packed qkv projection and the output can be token-major.
+#include "pf_common.h"
+
+namespace {
+
+constexpr int KT = 64;        // keys (forward/dQ) or queries (dK/dV) per LDS tile
+constexpr float LOG2E = 1.4426950408889634f;
+
+struct AttnArgs {
+  const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* o; const uint16_t* d_o;
+  uint16_t* out; uint16_t* dq; uint16_t* dk; uint16_t* dv;
+  float* lse; const float* delta;
+  int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, o_st;
+  int64_t do_sb, do_sh, do_st, dq_sb, dq_sh, dq_st, dk_sb, dk_sh, dk_st, dv_sb, dv_sh, dv_st;
+  int B, H, Tq, Tk, hd, causal;
+  float scale;
+};
+
+template <int DT> struct M32;
+template <> struct M32<PF_F16> {
+  static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0,
+                                                  0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    return (uint32_t)pf_f32_to_f16_bits(lo) | ((uint32_t)pf_f32_to_f16_bits(hi) << 16);
+  }
+};
+template <> struct M32<PF_BF16> {
+  static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
+                                                   0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    return (uint32_t)pf_f32_to_bf16_bits(lo) | ((uint32_t)pf_f32_to_bf16_bits(hi) << 16);
+  }
+};
+
+// registers r..r+7 of an accumulator tile -> one 16-byte MFMA operand (8 x 16-bit)
+template <int DT>
+__device__ __forceinline__ uint4 pack8(const float16_t& a, int r) {
+  return make_uint4(M32<DT>::pack(a[r], a[r + 1]), M32<DT>::pack(a[r + 2], a[r + 3]),
+                    M32<DT>::pack(a[r + 4], a[r + 5]), M32<DT>::pack(a[r + 6], a[r + 7]));
+}
+
+// row index inside a 32-row accumulator tile of register r for this lane
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+// 16-byte global load of 8 consecutive hd elements of one token row; zero when the
+// token or the hd chunk is out of range
+__device__ __forceinline__ uint4 load_row8(const uint16_t* base, int64_t st, int t, int T, int h0, int hd) {
+  if (t < T && h0 < hd) return *(const uint4*)(base + (int64_t)t * st + h0);
+  return make_uint4(0, 0, 0, 0);
+}
+
+// natural tile [ROWS tokens][HD + 8]: thread-strided 16-byte copies
+template <int ROWS, int HD>
+__device__ __forceinline__ void stage_natural(uint16_t* s, const uint16_t* base, int64_t st, int t0, int T, int hd,
+                                              int tid) {
+  constexpr int LD = HD + 8, VPR = HD / 8;
+  for (int e = tid; e < ROWS * VPR; e += 256) {
+    const int row = e / VPR, hv = e % VPR;
+    *(uint4*)(s + row * LD + hv * 8) = load_row8(base, st, t0 + row, T, hv * 8, hd);
+  }
+}
+
+// transposed tile [HD][ROWS + 8] (element (h, t)): 8x8 register transposes
+template <int ROWS, int HD>
+__device__ __forceinline__ void stage_transposed(uint16_t* s, const uint16_t* base, int64_t st, int t0, int T, int hd,
+                                                 int tid) {
+  constexpr int LD = ROWS + 8, TB = ROWS / 8, HB = HD / 8;
+  for (int b = tid; b < TB * HB; b += 256) {
+    const int tb = b % TB, hb = b / TB;  // consecutive threads: consecutive token blocks of the same 8 hd rows
+    uint32_t in[8][4];
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const uint4 x = load_row8(base, st, t0 + tb * 8 + r, T, hb * 8, hd);
+      in[r][0] = x.x; in[r][1] = x.y; in[r][2] = x.z; in[r][3] = x.w;
+    }
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+      uint32_t lo[4], hi[4];
+#pragma unroll
+      for (int I = 0; I < 4; ++I) {
+        const uint32_t a = in[2 * I][J], c = in[2 * I + 1][J];
+        lo[I] = (a & 0xffffu) | (c << 16);
+        hi[I] = (a >> 16) | (c & 0xffff0000u);
+      }
+      *(uint4*)(s + (hb * 8 + 2 * J) * LD + tb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      *(uint4*)(s + (hb * 8 + 2 * J + 1) * LD + tb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    }
+  }
+}
+
+// A operand read from a transposed tile for the reduction chunk [16*j, 16*j+16) of the
+// tile's token axis, with the index permutation that matches pack8(): element i of the
+// lane <-> token 16*j + 8*(i/4) + 4*(lane/32) + (i%4)
+template <int LD>
+__device__ __forceinline__ uint4 frag_transposed(const uint16_t* s, int row, int j, int lane) {
+  const uint16_t* p = s + row * LD + 16 * j + 4 * (lane >> 5);
+  const uint2 a = *(const uint2*)p, b = *(const uint2*)(p + 8);
+  return make_uint4(a.x, a.y, b.x, b.y);
+}
+
+// ---------------------------------------------------------------------------------
+// forward: one workgroup = 128 queries of one (batch, head); wavefront w owns 32 of them
+// ---------------------------------------------------------------------------------
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
+  constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8, VLD = KT + 8;
+  __shared__ __align__(16) uint16_t sK[KT * KLD];
+  __shared__ __align__(16) uint16_t sVt[HD * VLD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int q0 = blockIdx.x * 128 + wave * 32;
+  const int qi = q0 + (lane & 31);          // this lane's query row
+  const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;            // causal: key j visible to query i iff j <= i + shift
+
+  uint4 qf[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) qf[c] = load_row8(Q, a.q_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
+
+  float16_t oacc[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[o][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  int k_end = a.Tk;
+  if (a.causal) {
+    const int last_q = min(blockIdx.x * 128 + 127, a.Tq - 1);
+    k_end = min(a.Tk, last_q + shift + 1);
+  }
+  for (int k0 = 0; k0 < k_end; k0 += KT) {
+    __syncthreads();
+    stage_natural<KT, HD>(sK, K, a.k_st, k0, a.Tk, a.hd, tid);
+    stage_transposed<KT, HD>(sVt, V, a.v_st, k0, a.Tk, a.hd, tid);
+    __syncthreads();
+    float16_t s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const uint4 kf = *(const uint4*)(sK + (t * 32 + (lane & 31)) * KLD + c * 16 + (lane >> 5) * 8);
+        s[t] = M32<DT>::run(kf, qf[c], s[t]);
+      }
+    }
+    float mx = m;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kj = k0 + t * 32 + acc_row(r, lane);
+        const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
+        s[t][r] = ok ? s[t][r] * sc : -INFINITY;
+        mx = fmaxf(mx, s[t][r]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float alpha = (mx == -INFINITY) ? 1.f : exp2f(m - mx);
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = (mx == -INFINITY) ? 0.f : exp2f(s[t][r] - mx);
+        s[t][r] = p;
+        psum += p;
+      }
+    l = l * alpha + psum;
+    m = mx;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[o][r] *= alpha;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4 pf = pack8<DT>(s[j >> 1], 8 * (j & 1));
+#pragma unroll
+      for (int o = 0; o < NO; ++o) {
+        const uint4 vf = frag_transposed<VLD>(sVt, o * 32 + (lane & 31), j, lane);
+        oacc[o] = M32<DT>::run(vf, pf, oacc[o]);
+      }
+    }
+  }
+  l += __shfl_xor(l, 32, 64);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  if (qi < a.Tq) {
+    uint16_t* O = a.out + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd) {
+          const uint2 w = make_uint2(M32<DT>::pack(oacc[o][4 * g] * inv, oacc[o][4 * g + 1] * inv),
+                                     M32<DT>::pack(oacc[o][4 * g + 2] * inv, oacc[o][4 * g + 3] * inv));
+          *(uint2*)(O + h0) = w;
+        }
+      }
+    if ((lane >> 5) == 0) a.lse[((int64_t)bh) * a.Tq + qi] = (l > 0.f) ? (m + log2f(l)) / LOG2E : -INFINITY;
+  }
+}
+
+// delta[b,h,q] = sum_hd dO * O
+__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a, float* delta) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  const int64_t rows = (int64_t)a.B * a.H * a.Tq;
+  if (row >= rows) return;
+  const int q = (int)(row % a.Tq);
+  const int bh = (int)(row / a.Tq), b = bh / a.H, h = bh % a.H;
+  const uint16_t* O = a.o + b * a.o_sb + h * a.o_sh + (int64_t)q * a.o_st;
+  const uint16_t* D = a.d_o + b * a.do_sb + h * a.do_sh + (int64_t)q * a.do_st;
+  float s = 0.f;
+  for (int c = lane; c < a.hd; c += 64) {
+    const float x = (a.causal & 0x100) ? pf_bf16_bits_to_f32(O[c]) : pf_f16_bits_to_f32(O[c]);
+    const float y = (a.causal & 0x100) ? pf_bf16_bits_to_f32(D[c]) : pf_f16_bits_to_f32(D[c]);
+    s += x * y;
+  }
+  s = pf_wave_sum(s);
+  if (lane == 0) delta[row] = s;
+}
+
+// ---------------------------------------------------------------------------------
+// dQ: same tiling as forward (column = query); dQ^T[hd][q] += K^T[hd][kv] dS^T[kv][q]
+// ---------------------------------------------------------------------------------
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
+  constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8, TLD = KT + 8;
+  __shared__ __align__(16) uint16_t sK[KT * KLD];
+  __shared__ __align__(16) uint16_t sV[KT * KLD];
+  __shared__ __align__(16) uint16_t sKt[HD * TLD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int q0 = blockIdx.x * 128 + wave * 32;
+  const int qi = q0 + (lane & 31);
+  const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
+  const uint16_t* DO = a.d_o + b * a.do_sb + h * a.do_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;
+
+  uint4 qf[NC], dof[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    qf[c] = load_row8(Q, a.q_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
+    dof[c] = load_row8(DO, a.do_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
+  }
+  const bool qok = qi < a.Tq;
+  const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : 0.f;
+  const float dlt = qok ? a.delta[(int64_t)bh * a.Tq + qi] : 0.f;
+
+  float16_t acc[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[o][r] = 0.f;
+
+  int k_end = a.Tk;
+  if (a.causal) {
+    const int last_q = min(blockIdx.x * 128 + 127, a.Tq - 1);
+    k_end = min(a.Tk, last_q + shift + 1);
+  }
+  for (int k0 = 0; k0 < k_end; k0 += KT) {
+    __syncthreads();
+    stage_natural<KT, HD>(sK, K, a.k_st, k0, a.Tk, a.hd, tid);
+    stage_natural<KT, HD>(sV, V, a.v_st, k0, a.Tk, a.hd, tid);
+    stage_transposed<KT, HD>(sKt, K, a.k_st, k0, a.Tk, a.hd, tid);
+    __syncthreads();
+    float16_t s[2], dp[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = dp[t][r] = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int off = (t * 32 + (lane & 31)) * KLD + c * 16 + (lane >> 5) * 8;
+        s[t] = M32<DT>::run(*(const uint4*)(sK + off), qf[c], s[t]);
+        dp[t] = M32<DT>::run(*(const uint4*)(sV + off), dof[c], dp[t]);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kj = k0 + t * 32 + acc_row(r, lane);
+        const bool ok = qok && kj < a.Tk && (!a.causal || kj <= qi + shift);
+        const float p = ok ? exp2f(s[t][r] * sc - lse2) : 0.f;
+        s[t][r] = p * (dp[t][r] - dlt) * a.scale;   // dS^T
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4 dsf = pack8<DT>(s[j >> 1], 8 * (j & 1));
+#pragma unroll
+      for (int o = 0; o < NO; ++o) {
+        const uint4 kf = frag_transposed<TLD>(sKt, o * 32 + (lane & 31), j, lane);
+        acc[o] = M32<DT>::run(kf, dsf, acc[o]);
+      }
+    }
+  }
+  if (qok) {
+    uint16_t* DQ = a.dq + b * a.dq_sb + h * a.dq_sh + (int64_t)qi * a.dq_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd)
+          *(uint2*)(DQ + h0) = make_uint2(M32<DT>::pack(acc[o][4 * g], acc[o][4 * g + 1]),
+                                          M32<DT>::pack(acc[o][4 * g + 2], acc[o][4 * g + 3]));
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// dK/dV: column = key row; S[q][kv] = Q K^T, dV^T[hd][kv] += dO^T[hd][q] P[q][kv],
+//        dK^T[hd][kv] += Q^T[hd][q] dS[q][kv]
+// ---------------------------------------------------------------------------------
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
+  constexpr int NC = HD / 16, NO = HD / 32, QLD = HD + 8, TLD = KT + 8;
+  __shared__ __align__(16) uint16_t sQ[KT * QLD];
+  __shared__ __align__(16) uint16_t sDO[KT * QLD];
+  __shared__ __align__(16) uint16_t sQt[HD * TLD];
+  __shared__ __align__(16) uint16_t sDOt[HD * TLD];
+  __shared__ float sLse[KT], sDelta[KT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int kj = blockIdx.x * 128 + wave * 32 + (lane & 31);   // this lane's key row
+  const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
+  const uint16_t* DO = a.d_o + b * a.do_sb + h * a.do_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;
+  const bool kok = kj < a.Tk;
+
+  uint4 kf[NC], vf[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    kf[c] = load_row8(K, a.k_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
+    vf[c] = load_row8(V, a.v_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
+  }
+  float16_t dk[NO], dv[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[o][r] = dv[o][r] = 0.f;
+
+  int q_begin = 0;
+  if (a.causal) {  // queries i with i + shift >= first key of the block see it
+    q_begin = max(0, blockIdx.x * 128 - shift);
+    q_begin = q_begin / KT * KT;
+  }
+  for (int q0 = q_begin; q0 < a.Tq; q0 += KT) {
+    __syncthreads();
+    stage_natural<KT, HD>(sQ, Q, a.q_st, q0, a.Tq, a.hd, tid);
+    stage_natural<KT, HD>(sDO, DO, a.do_st, q0, a.Tq, a.hd, tid);
+    stage_transposed<KT, HD>(sQt, Q, a.q_st, q0, a.Tq, a.hd, tid);
+    stage_transposed<KT, HD>(sDOt, DO, a.do_st, q0, a.Tq, a.hd, tid);
+    if (tid < KT) {
+      const int qi = q0 + tid;
+      sLse[tid] = qi < a.Tq ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : 0.f;
+      sDelta[tid] = qi < a.Tq ? a.delta[(int64_t)bh * a.Tq + qi] : 0.f;
+    }
+    __syncthreads();
+    float16_t s[2], dp[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[t][r] = dp[t][r] = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int off = (t * 32 + (lane & 31)) * QLD + c * 16 + (lane >> 5) * 8;
+        s[t] = M32<DT>::run(*(const uint4*)(sQ + off), kf[c], s[t]);
+        dp[t] = M32<DT>::run(*(const uint4*)(sDO + off), vf[c], dp[t]);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ql = t * 32 + acc_row(r, lane), qi = q0 + ql;
+        const bool ok = kok && qi < a.Tq && (!a.causal || kj <= qi + shift);
+        const float p = ok ? exp2f(s[t][r] * sc - sLse[ql]) : 0.f;
+        s[t][r] = p;                                         // P
+        dp[t][r] = p * (dp[t][r] - sDelta[ql]) * a.scale;    // dS
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint4 pf = pack8<DT>(s[j >> 1], 8 * (j & 1));
+      const uint4 dsf = pack8<DT>(dp[j >> 1], 8 * (j & 1));
+#pragma unroll
+      for (int o = 0; o < NO; ++o) {
+        const int row = o * 32 + (lane & 31);
+        dv[o] = M32<DT>::run(frag_transposed<TLD>(sDOt, row, j, lane), pf, dv[o]);
+        dk[o] = M32<DT>::run(frag_transposed<TLD>(sQt, row, j, lane), dsf, dk[o]);
+      }
+    }
+  }
+  if (kok) {
+    uint16_t* DK = a.dk + b * a.dk_sb + h * a.dk_sh + (int64_t)kj * a.dk_st;
+    uint16_t* DV = a.dv + b * a.dv_sb + h * a.dv_sh + (int64_t)kj * a.dv_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd) {
+          *(uint2*)(DK + h0) = make_uint2(M32<DT>::pack(dk[o][4 * g], dk[o][4 * g + 1]),
+                                          M32<DT>::pack(dk[o][4 * g + 2], dk[o][4 * g + 3]));
+          *(uint2*)(DV + h0) = make_uint2(M32<DT>::pack(dv[o][4 * g], dv[o][4 * g + 1]),
+                                          M32<DT>::pack(dv[o][4 * g + 2], dv[o][4 * g + 3]));
+        }
+      }
+  }
+}
+
+bool strides_ok(const void* p, int64_t sb, int64_t sh, int64_t st) {
+  return pf_aligned(p, 16) && sb % 8 == 0 && sh % 8 == 0 && st % 8 == 0;
+}
+
+int check_common(const pf_attn_desc* d, const char* name) {
+  PF_REQUIRE(d != nullptr, "%s: null descriptor", name);
+  PF_REQUIRE(d->dtype == PF_F16 || d->dtype == PF_BF16, "%s: dtype must be fp16 or bf16", name);
+  PF_REQUIRE(d->B > 0 && d->H > 0 && d->Tq > 0 && d->Tk > 0 && d->hd > 0, "%s: bad shape", name);
+  if (d->hd % 8 != 0 || d->hd > 96) {
+    pf_set_error("%s: head dim %d is not supported by the fused kernels (multiple of 8, <= 96)", name, d->hd);
+    return PF_ERR_UNSUPPORTED;
+  }
+  PF_REQUIRE((int64_t)d->B * d->H <= 65535, "%s: B*H exceeds 65535", name);
+  PF_REQUIRE(d->q && d->k && d->v && d->lse, "%s: null operand", name);
+  PF_REQUIRE(strides_ok(d->q, d->q_sb, d->q_sh, d->q_st) && strides_ok(d->k, d->k_sb, d->k_sh, d->k_st) &&
+                 strides_ok(d->v, d->v_sb, d->v_sh, d->v_st),
+             "%s: q/k/v must be 16-byte aligned with strides that are multiples of 8", name);
+  if (d->causal) PF_REQUIRE(d->Tk >= d->Tq, "%s: causal attention needs Tk >= Tq", name);
+  return PF_OK;
+}
+
+AttnArgs make_args(const pf_attn_desc* d) {
+  AttnArgs a;
+  a.q = (const uint16_t*)d->q; a.k = (const uint16_t*)d->k; a.v = (const uint16_t*)d->v;
+  a.o = (const uint16_t*)d->o; a.d_o = (const uint16_t*)d->d_o; a.out = (uint16_t*)d->o;
+  a.dq = (uint16_t*)d->dq; a.dk = (uint16_t*)d->dk; a.dv = (uint16_t*)d->dv;
+  a.lse = d->lse; a.delta = d->delta;
+  a.q_sb = d->q_sb; a.q_sh = d->q_sh; a.q_st = d->q_st; a.k_sb = d->k_sb; a.k_sh = d->k_sh; a.k_st = d->k_st;
+  a.v_sb = d->v_sb; a.v_sh = d->v_sh; a.v_st = d->v_st; a.o_sb = d->o_sb; a.o_sh = d->o_sh; a.o_st = d->o_st;
+  a.do_sb = d->do_sb; a.do_sh = d->do_sh; a.do_st = d->do_st; a.dq_sb = d->dq_sb; a.dq_sh = d->dq_sh;
+  a.dq_st = d->dq_st; a.dk_sb = d->dk_sb; a.dk_sh = d->dk_sh; a.dk_st = d->dk_st; a.dv_sb = d->dv_sb;
+  a.dv_sh = d->dv_sh; a.dv_st = d->dv_st;
+  a.B = d->B; a.H = d->H; a.Tq = d->Tq; a.Tk = d->Tk; a.hd = d->hd; a.causal = d->causal ? 1 : 0;
+  a.scale = d->scale;
+  return a;
+}
+
+}  // namespace
+
+#define PF_ATTN_DISPATCH(KERNEL, grid, st, a, dt, hd)                                          \
+  do {                                                                                         \
+    if (dt == PF_F16) {                                                                        \
+      if (hd <= 64) hipLaunchKernelGGL((KERNEL<PF_F16, 64>), grid, dim3(256), 0, st, a);       \
+      else hipLaunchKernelGGL((KERNEL<PF_F16, 96>), grid, dim3(256), 0, st, a);                \
+    } else {                                                                                   \
+      if (hd <= 64) hipLaunchKernelGGL((KERNEL<PF_BF16, 64>), grid, dim3(256), 0, st, a);      \
+      else hipLaunchKernelGGL((KERNEL<PF_BF16, 96>), grid, dim3(256), 0, st, a);               \
+    }                                                                                          \
+  } while (0)
+
+extern "C" int pf_attention_fwd(const pf_attn_desc* d, void* stream) {
+  int rc = check_common(d, "pf_attention_fwd");
+  if (rc != PF_OK) return rc;
+  PF_REQUIRE(d->o && strides_ok(d->o, d->o_sb, d->o_sh, d->o_st) && d->o_st % 4 == 0,
+             "pf_attention_fwd: bad output operand");
+  AttnArgs a = make_args(d);
+  const dim3 grid((unsigned)((d->Tq + 127) / 128), (unsigned)(d->B * d->H));
+  PF_ATTN_DISPATCH(attn_fwd_kernel, grid, (hipStream_t)stream, a, d->dtype, d->hd);
+  PF_CHECK_LAUNCH("pf_attention_fwd");
+  return PF_OK;
+}
+
+extern "C" int pf_attention_bwd(const pf_attn_desc* d, void* stream) {
+  int rc = check_common(d, "pf_attention_bwd");
+  if (rc != PF_OK) return rc;
+  PF_REQUIRE(d->o && d->d_o && d->dq && d->dk && d->dv && d->delta, "pf_attention_bwd: null operand");
+  PF_REQUIRE(strides_ok(d->o, d->o_sb, d->o_sh, d->o_st) && strides_ok(d->d_o, d->do_sb, d->do_sh, d->do_st),
+             "pf_attention_bwd: o/dO must be 16-byte aligned with strides that are multiples of 8");
+  PF_REQUIRE(pf_aligned(d->dq, 8) && pf_aligned(d->dk, 8) && pf_aligned(d->dv, 8) && d->dq_sb % 4 == 0 &&
+                 d->dq_sh % 4 == 0 && d->dq_st % 4 == 0 && d->dk_sb % 4 == 0 && d->dk_sh % 4 == 0 &&
+                 d->dk_st % 4 == 0 && d->dv_sb % 4 == 0 && d->dv_sh % 4 == 0 && d->dv_st % 4 == 0,
+             "pf_attention_bwd: gradient operands must be 8-byte aligned with strides that are multiples of 4");
+  AttnArgs a = make_args(d);
+  hipStream_t st = (hipStream_t)stream;
+  AttnArgs ad = a;
+  if (d->dtype == PF_BF16) ad.causal |= 0x100;  // dtype flag for the delta kernel
+  const int64_t rows = (int64_t)d->B * d->H * d->Tq;
+  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, ad, d->delta);
+  const dim3 gq((unsigned)((d->Tq + 127) / 128), (unsigned)(d->B * d->H));
+  const dim3 gk((unsigned)((d->Tk + 127) / 128), (unsigned)(d->B * d->H));
+  PF_ATTN_DISPATCH(attn_dkv_kernel, gk, st, a, d->dtype, d->hd);
+  PF_ATTN_DISPATCH(attn_dq_kernel, gq, st, a, d->dtype, d->hd);
+  PF_CHECK_LAUNCH("pf_attention_bwd");
+  return PF_OK;
+}

@@ -296,6 +296,16 @@ class BwdCtx:
             raise Unsupported("strided copy over %d dimensions" % len(sizes))
         self.emit(self.k.copy_strided(src, ss, dst, ds, sizes, 1 if accumulate else 0))
 
+    def merge(self, tmp, dst, prev):
+        """dst = tmp (+ prev): finish a contribution that was computed into a temporary."""
+        if prev is None:
+            self.copy(tmp, dst)
+        elif prev is dst:
+            self.copy(tmp, dst, accumulate=True)
+        else:
+            self.copy(prev, dst)
+            self.copy(tmp, dst, accumulate=True)
+
     def contribute(self, val, t):
         """Add tensor t (val's shape, any strides/dtype) to val's gradient."""
         if not val.req_grad:
@@ -731,18 +741,20 @@ def lower_sdpa(L, node):
         return t
 
     qt, kt, vt = head_tensor(q), head_tensor(k), head_tensor(v)
+    req = q.req_grad or k.req_grad or v.req_grad
+    kern = L.kernels
+    if L.mixed and hv == hd and hd % 8 == 0 and hd <= getattr(kern, "MAX_FUSED_HEAD_DIM", 0):
+        return _lower_sdpa_fused(L, (q, k, v), (qt, kt, vt), (Bn, H, Tq, Tk, hd), scale, causal, req)
     S = L.pool.scratch("attn_s", (Bn, H, Tq, Tkp), torch.float32)
     P = L.alloc((Bn, H, Tq, Tkp), cd)
     O = L.alloc((Bn, Tq, H, hv), cd)           # token-major, so that transpose(1,2).reshape is a view
     Ov = O.permute(0, 2, 1, 3)
     bs = lambda t: (t.stride(0), t.stride(1))
-    kern = L.kernels
     L.emit(kern.gemm(qt, kt, S, M=Tq, N=Tk, K=hd, lda=qt.stride(2), ldb=kt.stride(2), ldc=Tkp, batch=(Bn, H),
                      sa=bs(qt), sb=bs(kt), sc=bs(S), alpha=scale))
     L.emit(kern.softmax_fwd(S, Tkp, P, Tkp, Bn * H * Tq, Tk, Tq, 1 if causal else 0))
     L.emit(kern.gemm(P, vt, Ov, M=Tq, N=hv, K=Tk, lda=Tkp, ldb=vt.stride(2), ldc=Ov.stride(2), b_trans=1,
                      batch=(Bn, H), sa=bs(P), sb=bs(vt), sc=bs(Ov)))
-    req = q.req_grad or k.req_grad or v.req_grad
     outv = Val(Ov, req_grad=req)
 
     def bwd(B):
@@ -760,7 +772,7 @@ def lower_sdpa(L, node):
                        sa=bs(g), sb=bs(vt), sc=bs(dP)))
         B.emit(kb.softmax_bwd(dP, Tkp, P, Tkp, dS, Tkp, Bn * H * Tq, Tk, scale))
 
-        def into(val, emit_fn, like_t):
+        def into(val, emit_fn):
             if not val.req_grad:
                 return
             dst, prev = B.grad_target(val)
@@ -771,25 +783,63 @@ def lower_sdpa(L, node):
             else:
                 tmp = B.temp(val.shape, cd)
                 emit_fn(tmp, 0)
-                if prev is None:
-                    B.copy(tmp, dst)
-                elif prev is dst:
-                    B.copy(tmp, dst, accumulate=True)
-                else:
-                    B.copy(prev, dst)
-                    B.copy(tmp, dst, accumulate=True)
+                B.merge(tmp, dst, prev)
                 B.commit(val, dst)
 
         # dQ = dS K ; dK = dS^T Q ; dV = P^T dO
         into(q, lambda dst, beta: B.emit(kb.gemm(dS, kt, dst, M=Tq, N=hd, K=Tk, lda=Tkp, ldb=kt.stride(2),
                                                   ldc=dst.stride(2), b_trans=1, batch=(Bn, H), sa=bs(dS), sb=bs(kt),
-                                                  sc=bs(dst), beta=beta)), qt)
+                                                  sc=bs(dst), beta=beta)))
         into(k, lambda dst, beta: B.emit(kb.gemm(dS, qt, dst, M=Tk, N=hd, K=Tq, lda=Tkp, ldb=qt.stride(2),
                                                   ldc=dst.stride(2), a_trans=1, b_trans=1, batch=(Bn, H), sa=bs(dS),
-                                                  sb=bs(qt), sc=bs(dst), beta=beta)), kt)
+                                                  sb=bs(qt), sc=bs(dst), beta=beta)))
         into(v, lambda dst, beta: B.emit(kb.gemm(P, g, dst, M=Tk, N=hv, K=Tq, lda=Tkp, ldb=g.stride(2),
                                                   ldc=dst.stride(2), a_trans=1, b_trans=1, batch=(Bn, H), sa=bs(P),
-                                                  sb=bs(g), sc=bs(dst), beta=beta)), vt)
+                                                  sb=bs(g), sc=bs(dst), beta=beta)))
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def _lower_sdpa_fused(L, vals, tensors, dims, scale, causal, req):
+    """softmax(QK^T)V as one kernel (no score matrix in memory) and a three-kernel backward."""
+    q, k, v = vals
+    qt, kt, vt = tensors
+    Bn, H, Tq, Tk, hd = dims
+    cd = L.cd
+    O = L.alloc((Bn, Tq, H, hd), cd)            # token-major, so that transpose(1,2).reshape is a view
+    Ov = O.permute(0, 2, 1, 3)
+    lse = L.alloc((Bn, H, Tq), torch.float32)
+    L.emit(L.kernels.attention_fwd(qt, kt, vt, Ov, lse, scale, causal))
+    outv = Val(Ov, req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        if g.dtype != cd or g.stride(3) != 1 or any(s % 8 for s in g.stride()[:3]):
+            t = B.new_like(Ov)
+            B.copy(g, t)
+            g = t
+        delta = L.pool.scratch("attn_delta", (Bn, H, Tq), torch.float32)
+        plan = []
+        outs = []
+        for val, like in ((q, qt), (k, kt), (v, vt)):
+            if val.req_grad:
+                dst, prev = B.grad_target(val)
+                direct = (prev is None and dst.dtype == cd and dst.stride(3) == 1
+                          and all(s % 4 == 0 for s in dst.stride()[:3]))
+                buf = dst if direct else B.temp(val.shape, cd)
+                plan.append((val, dst, prev, buf, direct))
+            else:
+                buf = B.temp(val.shape, cd)
+            outs.append(buf)
+        B.emit(B.k.attention_bwd(qt, kt, vt, Ov, g, lse, delta, outs[0], outs[1], outs[2], scale, causal))
+        for val, dst, prev, buf, direct in plan:
+            if not direct:
+                B.merge(buf, dst, prev)
+            B.commit(val, dst)
 
     if req:
         L.add_backward(bwd)

@@ -61,12 +61,25 @@ class GemmDesc(Structure):
     ]
 
 
+class AttnDesc(Structure):
+    """Mirror of `pf_attn_desc` in include/pfeife_hip.h."""
+
+    _fields_ = ([(n, c_int32) for n in ("dtype", "B", "H", "Tq", "Tk", "hd", "causal", "reserved")]
+                + [("scale", c_float), ("reserved2", c_float)]
+                + [(n, c_void_p) for n in ("q", "k", "v", "o", "d_o", "dq", "dk", "dv", "lse", "delta")]
+                + [(n, c_int64) for n in ("q_sb", "q_sh", "q_st", "k_sb", "k_sh", "k_st", "v_sb", "v_sh", "v_st",
+                                          "o_sb", "o_sh", "o_st", "do_sb", "do_sh", "do_st", "dq_sb", "dq_sh",
+                                          "dq_st", "dk_sb", "dk_sh", "dk_st", "dv_sb", "dv_sh", "dv_st")])
+
+
 # name -> argtypes (every function returns int unless listed in _RET_I64)
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
     "pf_init": [_I],
     "pf_gemm": [POINTER(GemmDesc), _P],
     "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
+    "pf_attention_fwd": [POINTER(AttnDesc), _P],
+    "pf_attention_bwd": [POINTER(AttnDesc), _P],
     "pf_layernorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _F, _P],
     "pf_layernorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _L, _I, _P],
     "pf_rmsnorm_fwd": [_P, _I, _P, _P, _I, _P, _L, _L, _F, _P],
@@ -221,6 +234,35 @@ class HipKernels:
         launch.variant = name.value.decode()
         launch.flops = 2.0 * M * N * K * batch[0] * batch[1]
         return launch
+
+    # -- fused attention -----------------------------------------------------------
+    MAX_FUSED_HEAD_DIM = 96
+
+    @staticmethod
+    def _attn_desc(q, k, v, o, lse, scale, causal, d_o=None, dq=None, dk=None, dv=None, delta=None):
+        d = AttnDesc()
+        Bn, H, Tq, hd = q.shape
+        d.dtype, d.B, d.H, d.Tq, d.Tk, d.hd, d.causal = dtype_code(q.dtype), Bn, H, Tq, k.shape[2], hd, int(causal)
+        d.scale = float(scale)
+        d.q, d.k, d.v, d.o, d.lse = _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse)
+        d.d_o, d.dq, d.dk, d.dv, d.delta = _ptr(d_o), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(delta)
+        for name, t in (("q", q), ("k", k), ("v", v), ("o", o), ("do", d_o), ("dq", dq), ("dk", dk), ("dv", dv)):
+            if t is None:
+                continue
+            if t.dim() != 4 or t.stride(3) != 1 or t.dtype != q.dtype:
+                raise RuntimeError("attention operand %s must be a [B,H,T,hd] tensor with unit hd stride" % name)
+            setattr(d, name + "_sb", t.stride(0))
+            setattr(d, name + "_sh", t.stride(1))
+            setattr(d, name + "_st", t.stride(2))
+        return d
+
+    def attention_fwd(self, q, k, v, o, lse, scale, causal):
+        d = self._attn_desc(q, k, v, o, lse, scale, causal)
+        return self._prep("pf_attention_fwd", (byref(d),), (d, q, k, v, o, lse))
+
+    def attention_bwd(self, q, k, v, o, d_o, lse, delta, dq, dk, dv, scale, causal):
+        d = self._attn_desc(q, k, v, o, lse, scale, causal, d_o, dq, dk, dv, delta)
+        return self._prep("pf_attention_bwd", (byref(d),), (d, q, k, v, o, d_o, lse, delta, dq, dk, dv))
 
     # -- normalisation -----------------------------------------------------------
     def layernorm_fwd(self, x, gamma, beta, y, mean, rstd, rows, d, eps):

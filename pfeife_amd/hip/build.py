@@ -19,6 +19,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 SOURCES = [
     "pf_runtime.cpp",
     "pf_gemm.hip",
+    "pf_attention.hip",
     "pf_norm.hip",
     "pf_elementwise.hip",
     "pf_softmax_loss.hip",

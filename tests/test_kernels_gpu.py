@@ -422,3 +422,59 @@ def test_deferred_reductions_match_immediate(hip):
         outs[defer] = (dx.cpu(), dg.cpu(), db.cpu(), bias.cpu())
     for a, b in zip(outs[0], outs[1]):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("case", [
+    dict(B=2, H=3, Tq=197, Tk=197, hd=64, causal=0, packed=True),    # ViT block
+    dict(B=1, H=2, Tq=257, Tk=257, hd=88, causal=0, packed=True),    # ViT-g head dim 88
+    dict(B=2, H=4, Tq=128, Tk=128, hd=64, causal=1, packed=False),   # decoder
+    dict(B=1, H=2, Tq=300, Tk=300, hd=64, causal=1, packed=False),   # ragged causal over several tiles
+    dict(B=2, H=2, Tq=64, Tk=77, hd=64, causal=0, packed=False),     # cross attention (77 context tokens)
+    dict(B=1, H=1, Tq=5, Tk=3, hd=8, causal=0, packed=False),        # tiny
+])
+def test_fused_attention(hip, oracle, dtype, case):
+    B, H, Tq, Tk, hd = case["B"], case["H"], case["Tq"], case["Tk"], case["hd"]
+    C = H * hd
+    if case["packed"]:
+        qkv = rnd((B, Tq, 3, H, hd), dtype, 1, 0.7)
+        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    else:
+        q = rnd((B, Tq, H, hd), dtype, 1, 0.7).permute(0, 2, 1, 3)
+        k = rnd((B, Tk, H, hd), dtype, 2, 0.7).permute(0, 2, 1, 3)
+        v = rnd((B, Tk, H, hd), dtype, 3, 0.7).permute(0, 2, 1, 3)
+    d_o = rnd((B, Tq, H, hd), dtype, 4).permute(0, 2, 1, 3)
+    scale = hd ** -0.5
+    res = {}
+    for name, tab, dev in (("hip", hip, "cuda"), ("oracle", oracle, "cpu")):
+        if case["packed"]:
+            base = qkv.to(dev)
+            qd, kd, vd = (base[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+            dbase = torch.zeros_like(base)
+            dq, dk, dv = (dbase[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+        else:
+            qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+            dq, dk, dv = torch.zeros_like(qd), torch.zeros_like(kd), torch.zeros_like(vd)
+        o = torch.zeros(B, Tq, H, hd, dtype=dtype, device=dev).permute(0, 2, 1, 3)
+        lse = torch.zeros(B, H, Tq, device=dev)
+        delta = torch.zeros(B, H, Tq, device=dev)
+        tab.run("attention_fwd", qd, kd, vd, o, lse, scale, case["causal"])
+        tab.run("attention_bwd", qd, kd, vd, o, d_o.to(dev), lse, delta, dq, dk, dv, scale, case["causal"])
+        if dev == "cuda":
+            torch.cuda.synchronize()
+        res[name] = [t.cpu().float() for t in (o, lse, dq, dk, dv)]
+    rt, at = TOL[dtype]
+    for i, nm in enumerate(["o", "lse", "dq", "dk", "dv"]):
+        a, b = res["hip"][i], res["oracle"][i]
+        tol = (1e-4, 1e-4) if nm == "lse" else (rt * 2, at * 2)
+        torch.testing.assert_close(a, b, rtol=tol[0], atol=tol[1], msg=lambda m, nm=nm: nm + ": " + m)
+    # the oracle itself against torch's attention and its autograd
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    mask = None
+    if case["causal"]:
+        mask = torch.ones(Tq, Tk, dtype=torch.bool).tril(Tk - Tq)
+    ref = torch.nn.functional.scaled_dot_product_attention(qf, kf, vf, attn_mask=mask)
+    ref.backward(d_o.float())
+    torch.testing.assert_close(res["oracle"][0], ref.detach(), rtol=3e-2, atol=3e-2)
+    for g, r in ((res["oracle"][2], qf.grad), (res["oracle"][3], kf.grad), (res["oracle"][4], vf.grad)):
+        torch.testing.assert_close(g, r, rtol=5e-2, atol=5e-2)
