@@ -234,12 +234,14 @@ template <int R, int BK, int NT> struct Stage<R, BK, NT, true> {
     return (uint32_t)(((K - 1) * ld + (R_total + 7) / 8 * 8) * 2);
   }
   // `first` = id of the first participating thread (lets A and B use disjoint threads).
-  // Consecutive threads take consecutive k-blocks of the same 8 rows: their LDS stores
-  // then fall into one LDS row each (16 contiguous bytes per thread, no bank conflicts),
-  // and the 8 threads that share a k-row cover 128 contiguous bytes of it in global memory.
+  // Consecutive threads take consecutive 8-column blocks of the same 8 k-rows, so that a
+  // wavefront's load covers long contiguous runs in global memory.  Their LDS stores then
+  // land 8 rows apart; the 16-byte chunk index inside the LDS row is XOR-swizzled with the
+  // row-block number so that those stores (and the fragment reads) spread over the banks.
+  static_assert(KB == 8, "the LDS swizzle assumes 8 chunks of 16 bytes per row");
   static __device__ __forceinline__ void init(uint32_t (&off)[8], int64_t ld, int64_t r0, int tid, int first) {
     const int b = tid - first;
-    const int kb = b % KB, rb = b / KB;
+    const int rb = b % (R / 8), kb = b / (R / 8);
 #pragma unroll
     for (int r = 0; r < 8; ++r) off[r] = (uint32_t)((((int64_t)kb * 8 + r) * ld + r0 + rb * 8) * 2);
   }
@@ -257,7 +259,8 @@ template <int R, int BK, int NT> struct Stage<R, BK, NT, true> {
                                                int tid, int first) {
     const int b = tid - first;
     if (b < 0 || b >= NBLK) return;
-    const int kb = b % KB, rb = b / KB;
+    const int rb = b % (R / 8), kb = b / (R / 8);
+    const int chunk = kb ^ (rb & 7);
     // 8x8 transpose of 16-bit values: 2x2 transposes inside 32-bit words, the
     // 4x4 transpose of the words is pure register renaming.
     const uint32_t in[8][4] = {{v[0].x, v[0].y, v[0].z, v[0].w}, {v[1].x, v[1].y, v[1].z, v[1].w},
@@ -273,8 +276,8 @@ template <int R, int BK, int NT> struct Stage<R, BK, NT, true> {
         lo[I] = (a & 0xffffu) | (c << 16);          // (k=2I, row 2J), (k=2I+1, row 2J)
         hi[I] = (a >> 16) | (c & 0xffff0000u);      // (k=2I, row 2J+1), (k=2I+1, row 2J+1)
       }
-      *(uint4*)(s + (rb * 8 + 2 * J) * LD + kb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-      *(uint4*)(s + (rb * 8 + 2 * J + 1) * LD + kb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+      *(uint4*)(s + (rb * 8 + 2 * J) * LD + chunk * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      *(uint4*)(s + (rb * 8 + 2 * J + 1) * LD + chunk * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
     }
   }
 };
@@ -327,7 +330,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)
   constexpr int BUF = (BM + BN) * LD;
   uint16_t* const buf0 = smem;
   uint16_t* const buf1 = smem + BUF;
-  const int frag_off = (lane & 31) * LD + (lane >> 5) * 8;
+  const int l31 = lane & 31, half = lane >> 5;
   const __amdgpu_buffer_rsrc_t rs_a = make_rsrc(A, SA::extent(M, K, lda));
   const __amdgpu_buffer_rsrc_t rs_b = make_rsrc(B, SB::extent(N, K, ldb));
   SA::init(offa, lda, m0, tid, A_FIRST);
@@ -339,10 +342,20 @@ __global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       uint4 fa[TM], fb[TN];
+      // 16-byte chunk (kk*2 + half) of the row; tiles written by the transposing loader
+      // keep it XOR-swizzled with the row's 8-row block number
 #pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = *(const uint4*)(s_a + (wm0 + i * 32) * LD + frag_off + kk * 16);
+      for (int i = 0; i < TM; ++i) {
+        const int row = wm0 + i * 32 + l31;
+        const int chunk = AT ? ((kk * 2 + half) ^ ((row >> 3) & 7)) : (kk * 2 + half);
+        fa[i] = *(const uint4*)(s_a + row * LD + chunk * 8);
+      }
 #pragma unroll
-      for (int j = 0; j < TN; ++j) fb[j] = *(const uint4*)(s_b + (wn0 + j * 32) * LD + frag_off + kk * 16);
+      for (int j = 0; j < TN; ++j) {
+        const int row = wn0 + j * 32 + l31;
+        const int chunk = BT ? ((kk * 2 + half) ^ ((row >> 3) & 7)) : (kk * 2 + half);
+        fb[j] = *(const uint4*)(s_b + row * LD + chunk * 8);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
