@@ -89,6 +89,19 @@ def build_workload(name, device):
     return runner, tuple(t.to(device) for t in inputs), info
 
 
+# Fabric-side bytes per launch (FETCH_SIZE + WRITE_SIZE, calibrated against a copy kernel) of the
+# GEMM instantiations of the vit_l16_fp16 workload, from the two rocprofv3 --pmc runs summarised
+# in profiles/vit_l16_fp16_pmc_traffic.md.
+MEASURED_TRAFFIC = {
+    "vit_l16_fp16": {
+        "gemm16_kernel<1, 128, 64, 64, 2, 2, false, false>": 9.04e7,
+        "gemm16_kernel<1, 128, 128, 64, 2, 2, true, true>": 1.105e8,
+        "gemm16_kernel<1, 128, 128, 64, 2, 2, false, false>": 1.240e8,
+        "gemm16_kernel<1, 64, 64, 64, 2, 2, true, true>": 4.56e7,
+    },
+}
+
+
 def gemm_roofline(runner, mixed, reps=3):
     """Replays every matrix-product launch of one step, grouped by kernel
     instantiation, between HIP events on the launch stream; returns the roofline
@@ -225,6 +238,9 @@ def main():
     ap.add_argument("--workload", default="vit_l16_fp16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain copy kernel (ew_kernel<Scale>, 256 MiB read + 256 MiB written) three "
+                         "times, as the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs every pipeline stage on ONE GPU; --gpus %d is not supported "
@@ -257,7 +273,25 @@ def main():
     value = samples * args.steps / dt
     log("[bench] %.2f ms/step, %.1f samples/s, last losses %s" % (ms, value, [round(float(l), 4) for l in losses]))
 
+    # host-side cost of a step: time to ENQUEUE it (no synchronisation inside step())
+    t0 = time.perf_counter()
+    for _ in range(3):
+        runner.step(*batch)
+    host_ms = 1e3 * (time.perf_counter() - t0) / 3
+    torch.cuda.synchronize()
+    log("[bench] host enqueue time %.2f ms/step" % host_ms)
+    if args.calibrate_copy:
+        n = 64 * 1024 * 1024
+        src = torch.ones(n, device=device)
+        dst = torch.empty(n, device=device)
+        launch = runner.worker.kernels.axpby(src, 1.0, None, 0.0, dst, n)
+        for _ in range(3):
+            launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+
     roof, per_variant = (None, {}) if args.no_roofline else gemm_roofline(runner, info["mixed"])
+    if roof is not None:
+        roof["traffic"] = MEASURED_TRAFFIC.get(args.workload, {}).get(roof["kernel"])
     for k, v in sorted(per_variant.items(), key=lambda kv: -kv[1]["ms_per_step"]):
         log("[bench] %-46s %4d launches/step %8.3f ms/step %8.1f us/launch %7.1f TFLOP/s"
             % (k, v["launches_per_step"], v["ms_per_step"], v["avg_launch_us"], v["tflops"]))
@@ -305,6 +339,7 @@ def main():
         "hbm_kernel": hbm,
         "cpu_baseline": cpu,
         "model_tflops": None if flops_step is None else round(flops_step / (ms * 1e-3) / 1e12, 2),
+        "host_enqueue_ms_per_step": round(host_ms, 3),
     }
     print(json.dumps(rec), flush=True)
 

@@ -407,10 +407,12 @@ __global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)
   // lane l owns row l/2, columns 16*(l%2) .. +16 of each tile.
   float* stage = (float*)smem + wave * (TN * 32 * EPI_LD);
   const int wr_off = ((lane >> 5) * 4) * EPI_LD + (lane & 31);
-  const int rd_row = lane >> 1, rd_col = (lane & 1) * 16;
+  const int rd_row = lane >> 2, rd_col = (lane & 3) * 8;
   // The accumulators are only ever indexed with compile-time constants (a dynamic
   // index would push them out of the register file): one row of TN tiles is
   // dumped with static indices, then a rolled loop runs the arithmetic on it.
+  // Read-back: 4 adjacent lanes cover the 32 columns of one tile row, so every store
+  // instruction writes whole 64-byte (16-bit C) or 128-byte (fp32 C) runs per row.
   static_for<TM>([&](auto ic) {
     constexpr int i = decltype(ic)::value;
     __syncthreads();  // previous tiles fully read (and, first time, main-loop tiles no longer needed)
@@ -421,23 +423,21 @@ __global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)
         stage[j * (32 * EPI_LD) + wr_off + (8 * (r >> 2) + (r & 3)) * EPI_LD] = acc[i][j][r];
     });
     __syncthreads();
-    const int64_t row = m0 + wm0 + i * 32 + rd_row;
-    if (row < M) {
 #pragma nounroll
-      for (int jh = 0; jh < 2 * TN; ++jh) {
-        const int j = jh >> 1, h = jh & 1;
-        const int64_t c8 = n0 + wn0 + j * 32 + rd_col + h * 8;
-        if (c8 >= N) continue;
-        const float4* src = (const float4*)(stage + j * (32 * EPI_LD) + rd_row * EPI_LD + rd_col + h * 8);
-        const float4 x = src[0], y = src[1];
-        float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
-        if (vec_epi && c8 + 8 <= N) {
-          epilogue_vec8(epi, c_base, row, c8, v);
-        } else {
+    for (int jp = 0; jp < 2 * TN; ++jp) {
+      const int j = jp >> 1, rr = rd_row + 16 * (jp & 1);
+      const int64_t row = m0 + wm0 + i * 32 + rr;
+      const int64_t c8 = n0 + wn0 + j * 32 + rd_col;
+      if (row >= M || c8 >= N) continue;
+      const float4* src = (const float4*)(stage + j * (32 * EPI_LD) + rr * EPI_LD + rd_col);
+      const float4 x = src[0], y = src[1];
+      float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+      if (vec_epi && c8 + 8 <= N) {
+        epilogue_vec8(epi, c_base, row, c8, v);
+      } else {
 #pragma nounroll
-          for (int k = 0; k < 8; ++k)
-            if (c8 + k < N) epilogue_scalar(epi, c_base, row, c8 + k, v[k]);
-        }
+        for (int k = 0; k < 8; ++k)
+          if (c8 + k < N) epilogue_scalar(epi, c_base, row, c8 + k, v[k]);
       }
     }
   });
