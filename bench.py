@@ -31,13 +31,14 @@ WORKLOADS = {
     "vit_s16_fp32": ("vit", "VIT_S16", 16, 4, ["blocks.6"], 2, None),
     "llama_1b_bf16": ("llama", "LLAMA_1B", 16, 8, ["layers.4", "layers.8", "layers.12"], 2, "bf16"),
     "vit_g14_share_bf16": ("vit_share", "VIT_G14_SHARE", 96, 4, [], 1, "bf16"),
+    "sdxl_stage_fp16": ("unet", "SDXL_STAGE", 4, 1, [], 1, "fp16"),
 }
 
 
 def build_workload(name, device):
     import torch
 
-    from pfeife_amd.bench_models import llama, vit
+    from pfeife_amd.bench_models import llama, unet_stage, vit
     from pfeife_amd.loss import CrossEntropyLoss
     from pfeife_amd.mp import PartialRunner, initialize_pfeife, partial_compiler
     from pfeife_amd.option import PipeOption
@@ -55,6 +56,13 @@ def build_workload(name, device):
         model = vit.BlockStack(cfg)
         inputs = (torch.randn(batch, cfg.tokens, cfg.dim, generator=g),
                   torch.randn(batch, cfg.tokens, cfg.dim, generator=g) * 1e-2)
+    elif family == "unet":
+        cfg = getattr(unet_stage, cfg_name)
+        model = unet_stage.UNetStage(cfg)
+        inputs = (torch.randn(batch, cfg.in_channels, 32, 32, generator=g),
+                  torch.randn(batch, cfg.temb_dim, generator=g),
+                  torch.randn(batch, 77, cfg.context_dim, generator=g),
+                  torch.randn(batch, cfg.channels, 32, 32, generator=g))
     else:
         cfg = getattr(llama, cfg_name)
         model = llama.LlamaForCausalLM(cfg)
@@ -77,6 +85,12 @@ def build_workload(name, device):
             out = cmodel(act)
             out.backward(grad_out.to(out.dtype))   # supplied upstream gradient of this GPU's block share
             return out.detach()[0, 0, 0]
+    elif family == "unet":
+        def exec_fn(hidden, temb, ctx, target):
+            out = cmodel(hidden, temb, ctx)
+            loss = torch.nn.functional.mse_loss(out.float(), target.float())   # as train_sdxl.py:1422-1424
+            loss.backward()
+            return loss.detach()
     else:
         def exec_fn(ids):
             loss = cmodel(ids, ids)                # next-token CE is inside the last stage
@@ -208,6 +222,8 @@ def cpu_baseline(name):
         y = torch.randn(mb * cnt, cfg.tokens, cfg.dim, generator=g) * 1e-2
         loss_fn = lambda o, t: (o * t).sum()
         unit, per_sample = "samples/s", 1
+    elif family == "unet":
+        raise RuntimeError("no CPU baseline leg for the UNet stage workload (run with --no-cpu-baseline)")
     else:
         cfg = getattr(llama, cfg_name)
         model = llama.LlamaForCausalLM(cfg)
@@ -313,6 +329,8 @@ def main():
         if info["family"] == "vit":
             extra = 2 * (T - 1) * (cfg.channels * cfg.patch_size ** 2) * d + 2 * d * cfg.num_classes
         flops_step = 3.0 * samples * (L * per_block + extra)
+    elif info["family"] == "unet":
+        flops_step = None
     else:
         T, d, ff, L, V = cfg.max_seq, cfg.dim, cfg.ffn, cfg.layers, cfg.vocab
         per_tok = L * (8 * d * d + 6 * d * ff + 4 * T * d) + 2 * d * V

@@ -142,6 +142,20 @@ int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, void* y, int 
 int pf_rmsnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
                    const float* rstd, const void* dx_add, int add_dtype, void* dx, int dx_dtype,
                    float* dgamma_acc, float* workspace, int64_t rows, int64_t d, int defer_reduce, void* stream);
+/* GroupNorm over channels-last [B, HW, C] tensors (the memory layout this library keeps
+ * convolutional feature maps in), `groups` groups of C/groups adjacent channels.
+ * mean/rstd: fp32 [B*groups].  Backward: dx, and dgamma/dbeta ACCUMULATED (or, with
+ * defer_reduce, left as per-sample partial rows [B][2][C] at the start of `workspace` for
+ * pf_colreduce_finalize_batch: n_partials = B, stride = 2*C).  workspace holds
+ * pf_groupnorm_workspace(B, C, groups) floats; C/groups <= 64 for the backward.
+ * Replaces aten::native_group_norm(+backward) of the UNet stage
+ * (bench_models/models/train_sdxl.py, diffusers ResnetBlock2D / Transformer2DModel). */
+int pf_groupnorm_fwd(const void* x, int x_dtype, const float* gamma, const float* beta, void* y, int y_dtype,
+                     float* mean, float* rstd, int64_t B, int64_t HW, int64_t C, int groups, float eps, void* stream);
+int pf_groupnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma, const float* mean,
+                     const float* rstd, void* dx, int dx_dtype, float* dgamma_acc, float* dbeta_acc, float* workspace,
+                     int64_t B, int64_t HW, int64_t C, int groups, int defer_reduce, void* stream);
+int64_t pf_groupnorm_workspace(int64_t B, int64_t C, int groups);
 /* Number of fp32 workspace elements the column reductions below need. */
 int64_t pf_colreduce_workspace(int64_t rows, int64_t cols);
 /* acc[c] += sum_r x[r*ld + c]  (bias gradient; deterministic two-stage reduce).
@@ -251,10 +265,12 @@ int pf_glu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64_t ld_gate,
  * fan-out gradient sum `g.add_(lg)` of pfeife/mp/worker.py:1543). n elements. */
 int pf_axpby(const void* a, int a_dtype, float alpha, const void* b, int b_dtype, float beta, void* out,
              int out_dtype, int64_t n, void* stream);
-/* y[r, c] = x[r, c] + bias[c % bias_len] (broadcast add of a bias / positional
- * embedding over the leading dimension). */
+/* y[r, c] = x[r, c] + bias[row_of_bias(r), c] over n = rows*bias_len elements.
+ * rows_per_bias == 0: one bias row broadcast over every row (bias / positional embedding);
+ * rows_per_bias  > 0: row r uses bias row r / rows_per_bias (a per-sample vector, e.g. the
+ * time-embedding projection added to every pixel of that sample). */
 int pf_bias_add(const void* x, int x_dtype, const void* bias, int bias_dtype, void* y, int y_dtype, int64_t n,
-                int64_t bias_len, void* stream);
+                int64_t bias_len, int64_t rows_per_bias, void* stream);
 /* dtype conversion / copy of n contiguous elements (autocast's weight casts,
  * done once per optimiser step instead of once per micro-batch). */
 int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream);

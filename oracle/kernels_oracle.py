@@ -208,6 +208,50 @@ class OracleKernels:
 
         return launch
 
+    def groupnorm_workspace(self, B, C, groups):
+        return B * 2 * C + B * groups * 2
+
+    def groupnorm_fwd(self, x, gamma, beta, y, mean, rstd, B, HW, C, groups, eps):
+        def launch(stream=None):
+            X = _strided(x, (B, HW, groups, C // groups), (HW * C, C, C // groups, 1)).float()
+            mu = X.mean(dim=(1, 3), keepdim=True)
+            var = ((X - mu) ** 2).mean(dim=(1, 3), keepdim=True)
+            rs = 1.0 / torch.sqrt(var + eps)
+            out = ((X - mu) * rs).reshape(B, HW, C) * _flat(gamma, C).float() + _flat(beta, C).float()
+            _strided(y, (B, HW, C), (HW * C, C, 1)).copy_(out.to(y.dtype))
+            _flat(mean, B * groups).copy_(mu.reshape(-1))
+            _flat(rstd, B * groups).copy_(rs.reshape(-1))
+
+        return launch
+
+    def groupnorm_bwd(self, dy, x, gamma, mean, rstd, dx, dgamma, dbeta, ws, B, HW, C, groups, defer=0):
+        def launch(stream=None):
+            Cg = C // groups
+            X = _strided(x, (B, HW, groups, Cg), (HW * C, C, Cg, 1)).float()
+            DY = _strided(dy, (B, HW, groups, Cg), (HW * C, C, Cg, 1)).float()
+            mu = _flat(mean, B * groups).float().view(B, 1, groups, 1)
+            rs = _flat(rstd, B * groups).float().view(B, 1, groups, 1)
+            gm = _flat(gamma, C).float().view(1, 1, groups, Cg)
+            xh = (X - mu) * rs
+            g = DY * gm
+            c1 = g.mean(dim=(1, 3), keepdim=True)
+            c2 = (g * xh).mean(dim=(1, 3), keepdim=True)
+            out = rs * (g - c1 - xh * c2)
+            _strided(dx, (B, HW, C), (HW * C, C, 1)).copy_(out.reshape(B, HW, C).to(dx.dtype))
+            pg = (DY * xh).sum(dim=1).reshape(B, C)
+            pb = DY.sum(dim=1).reshape(B, C)
+            if defer:
+                w = _strided(ws, (B, 2, C), (2 * C, C, 1))
+                w[:, 0].copy_(pg)
+                w[:, 1].copy_(pb)
+                return
+            if dgamma is not None:
+                _flat(dgamma, C).add_(pg.sum(0))
+            if dbeta is not None:
+                _flat(dbeta, C).add_(pb.sum(0))
+
+        return launch
+
     def rmsnorm_fwd(self, x, gamma, y, rstd, rows, d, eps):
         def launch(stream=None):
             X = _rows(x, rows, d, d).float()
@@ -349,10 +393,16 @@ class OracleKernels:
 
         return launch
 
-    def bias_add(self, x, bias, y, n, bias_len):
+    def bias_add(self, x, bias, y, n, bias_len, rows_per_bias=0):
         def launch(stream=None):
-            v = _flat(x, n).float().view(-1, bias_len) + _flat(bias, bias_len).float()
-            _flat(y, n).copy_(v.reshape(-1).to(y.dtype))
+            rows = n // bias_len
+            X = _flat(x, n).float().view(rows, bias_len)
+            if rows_per_bias:
+                nb = rows // rows_per_bias
+                bb = _strided(bias, (nb, bias_len), (bias_len, 1)).float().repeat_interleave(rows_per_bias, dim=0)
+            else:
+                bb = _flat(bias, bias_len).float()
+            _flat(y, n).copy_((X + bb).reshape(-1).to(y.dtype))
 
         return launch
 

@@ -107,11 +107,12 @@ struct GradAcc {
   }
 };
 struct BiasAdd {  // bias_len is a multiple of 8 on the vector path
-  const void* x; const void* bias; void* y; int xdt, bdt, ydt; int64_t bias_len;
+  const void* x; const void* bias; void* y; int xdt, bdt, ydt; int64_t bias_len, span;
   template <int W> __device__ void run(int64_t i) const {
     float v[W], b[W];
     ld_vec<W>(x, i, xdt, v);
-    ld_vec<W>(bias, i % bias_len, bdt, b);
+    // span = elements of x that share one bias row (0: every row uses bias row 0)
+    ld_vec<W>(bias, (span ? (i / span) * bias_len : 0) + i % bias_len, bdt, b);
 #pragma unroll
     for (int k = 0; k < W; ++k) v[k] += b[k];
     st_vec<W>(y, i, ydt, v);
@@ -305,14 +306,15 @@ extern "C" int pf_axpby(const void* a, int a_dtype, float alpha, const void* b, 
 }
 
 extern "C" int pf_bias_add(const void* x, int x_dtype, const void* bias, int bias_dtype, void* y, int y_dtype,
-                           int64_t n, int64_t bias_len, void* stream) {
+                           int64_t n, int64_t bias_len, int64_t rows_per_bias, void* stream) {
   PF_REQUIRE(n >= 0 && bias_len > 0 && pf_is_float_dtype(x_dtype) && pf_is_float_dtype(bias_dtype) &&
                  pf_is_float_dtype(y_dtype),
              "pf_bias_add: bad arguments");
   if (n == 0) return PF_OK;
   PF_REQUIRE(x && bias && y, "pf_bias_add: null pointer");
   PF_REQUIRE(n % bias_len == 0, "pf_bias_add: n must be a multiple of bias_len");
-  BiasAdd f{x, bias, y, x_dtype, bias_dtype, y_dtype, bias_len};
+  PF_REQUIRE(rows_per_bias >= 0, "pf_bias_add: negative rows_per_bias");
+  BiasAdd f{x, bias, y, x_dtype, bias_dtype, y_dtype, bias_len, rows_per_bias * bias_len};
   return ew_launch(f, n, al16(x) && al16(bias) && al16(y) && bias_len % 8 == 0, (hipStream_t)stream, "pf_bias_add");
 }
 

@@ -208,6 +208,118 @@ __global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, in
   }
 }
 
+
+// ---- GroupNorm on channels-last [B, HW, C] tensors ---------------------------------
+// statistics: one workgroup per (batch, group); two passes over the group's HW x Cg
+// elements (the second one hits L2)
+__global__ __launch_bounds__(256) void groupnorm_stats_kernel(const void* x, int x_dt, float* mean, float* rstd,
+                                                              int64_t HW, int64_t C, int G, float eps) {
+  __shared__ float sm[4];
+  const int64_t b = blockIdx.x / G, g = blockIdx.x % G;
+  const int64_t Cg = C / G, n = HW * Cg;
+  const int64_t base = b * HW * C + g * Cg;
+  float s = 0.f;
+  for (int64_t e = threadIdx.x; e < n; e += 256) s += pf_load_as_f32(x, base + (e / Cg) * C + e % Cg, x_dt);
+  const float mu = pf_block_sum<4>(s, sm) / (float)n;
+  float q = 0.f;
+  for (int64_t e = threadIdx.x; e < n; e += 256) {
+    const float t = pf_load_as_f32(x, base + (e / Cg) * C + e % Cg, x_dt) - mu;
+    q += t * t;
+  }
+  const float var = pf_block_sum<4>(q, sm) / (float)n;
+  if (threadIdx.x == 0) {
+    mean[blockIdx.x] = mu;
+    rstd[blockIdx.x] = 1.0f / sqrtf(var + eps);
+  }
+}
+
+// y = (x - mean[b,g]) * rstd[b,g] * gamma[c] + beta[c], 8 channels per thread (Cg % 8 == 0) or 1
+template <int W>
+__global__ __launch_bounds__(256) void groupnorm_apply_kernel(const void* x, int x_dt, const float* gamma,
+                                                              const float* beta, const float* mean,
+                                                              const float* rstd, void* y, int y_dt, int64_t total,
+                                                              int64_t HW, int64_t C, int G) {
+  const int64_t Cg = C / G;
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * W; i < total; i += gsz * W) {
+    const int64_t c = i % C, b = i / (HW * C);
+    const int64_t sg = b * G + c / Cg;
+    const float mu = mean[sg], rs = rstd[sg];
+    float v[W], gm[W], bt[W];
+    ld_vec<W>(x, i, x_dt, v);
+    ld_vec<W>(gamma, c, PF_F32, gm);
+    ld_vec<W>(beta, c, PF_F32, bt);
+#pragma unroll
+    for (int k = 0; k < W; ++k) v[k] = (v[k] - mu) * rs * gm[k] + bt[k];
+    st_vec<W>(y, i, y_dt, v);
+  }
+}
+
+// backward statistics: workgroup per (batch, group); lane = channel inside the group
+// (Cg <= 64), the 4 wavefronts split the pixels.  Writes c1 = mean(dy*gamma),
+// c2 = mean(dy*gamma*xhat) per (b, g) and the per-batch channel sums of dy*xhat and dy.
+__global__ __launch_bounds__(256) void groupnorm_bwd_stats_kernel(const void* dy, int dy_dt, const void* x, int x_dt,
+                                                                  const float* gamma, const float* mean,
+                                                                  const float* rstd, float* c12, float* ws,
+                                                                  int64_t HW, int64_t C, int G) {
+  __shared__ float sm[4];
+  __shared__ float red[2][4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t b = blockIdx.x / G, g = blockIdx.x % G;
+  const int64_t Cg = C / G;
+  const float mu = mean[blockIdx.x], rs = rstd[blockIdx.x];
+  float s1 = 0.f, s2 = 0.f, pg = 0.f, pb = 0.f;
+  if (lane < Cg) {
+    const int64_t c = g * Cg + lane;
+    const float gm = gamma[c];
+    for (int64_t p = wave; p < HW; p += 4) {
+      const int64_t i = (b * HW + p) * C + c;
+      const float d = pf_load_as_f32(dy, i, dy_dt);
+      const float xh = (pf_load_as_f32(x, i, x_dt) - mu) * rs;
+      s1 += d * gm;
+      s2 += d * gm * xh;
+      pg += d * xh;
+      pb += d;
+    }
+  }
+  red[0][wave][lane] = pg;
+  red[1][wave][lane] = pb;
+  const float n = (float)(HW * Cg);
+  s1 = pf_block_sum<4>(s1, sm);
+  s2 = pf_block_sum<4>(s2, sm);   // (the block sums synchronise, so `red` is complete below)
+  if (threadIdx.x == 0) {
+    c12[2 * blockIdx.x] = s1 / n;
+    c12[2 * blockIdx.x + 1] = s2 / n;
+  }
+  if (wave == 0 && lane < Cg) {
+    const int64_t c = g * Cg + lane;
+    ws[(b * 2) * C + c] = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
+    ws[(b * 2 + 1) * C + c] = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
+  }
+}
+
+template <int W>
+__global__ __launch_bounds__(256) void groupnorm_bwd_apply_kernel(const void* dy, int dy_dt, const void* x, int x_dt,
+                                                                  const float* gamma, const float* mean,
+                                                                  const float* rstd, const float* c12, void* dx,
+                                                                  int dx_dt, int64_t total, int64_t HW, int64_t C,
+                                                                  int G) {
+  const int64_t Cg = C / G;
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * W; i < total; i += gsz * W) {
+    const int64_t c = i % C, b = i / (HW * C);
+    const int64_t sg = b * G + c / Cg;
+    const float mu = mean[sg], rs = rstd[sg], c1 = c12[2 * sg], c2 = c12[2 * sg + 1];
+    float d[W], v[W], gm[W];
+    ld_vec<W>(dy, i, dy_dt, d);
+    ld_vec<W>(x, i, x_dt, v);
+    ld_vec<W>(gamma, c, PF_F32, gm);
+#pragma unroll
+    for (int k = 0; k < W; ++k) d[k] = rs * (d[k] * gm[k] - c1 - (v[k] - mu) * rs * c2);
+    st_vec<W>(dx, i, dx_dt, d);
+  }
+}
+
 inline int64_t colsum_chunks(int64_t rows) {
   int64_t chunks = (rows + 31) / 32;
   if (chunks > 256) chunks = 256;
@@ -363,6 +475,65 @@ extern "C" int pf_rmsnorm_bwd(const void* dy, int dy_dtype, const void* x, int x
   return norm_bwd(dy, dy_dtype, x, x_dtype, gamma, nullptr, rstd, dx_add, add_dtype, dx, dx_dtype, dgamma_acc,
                   nullptr, workspace, rows, d, 1, defer_reduce, (hipStream_t)stream, "pf_rmsnorm_bwd");
 }
+
+
+extern "C" int pf_groupnorm_fwd(const void* x, int x_dtype, const float* gamma, const float* beta, void* y,
+                                int y_dtype, float* mean, float* rstd, int64_t B, int64_t HW, int64_t C, int groups,
+                                float eps, void* stream) {
+  PF_REQUIRE(B >= 0 && HW > 0 && C > 0 && groups > 0 && C % groups == 0, "pf_groupnorm_fwd: bad shape");
+  if (B == 0) return PF_OK;
+  PF_REQUIRE(x && gamma && beta && y && mean && rstd, "pf_groupnorm_fwd: null pointer");
+  PF_REQUIRE(pf_is_float_dtype(x_dtype) && pf_is_float_dtype(y_dtype), "pf_groupnorm_fwd: bad dtype");
+  PF_REQUIRE(B * groups < (1ll << 31), "pf_groupnorm_fwd: too many groups");
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(groupnorm_stats_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, x, x_dtype, mean, rstd, HW,
+                     C, groups, eps);
+  const int64_t total = B * HW * C;
+  const bool v = (C / groups) % 8 == 0 && vec_ok(x, x_dtype, C) && vec_ok(y, y_dtype, C) && vec_ok(gamma, PF_F32, C) &&
+                 vec_ok(beta, PF_F32, C);
+  int64_t blocks = (total / (v ? 8 : 1) + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  if (blocks < 1) blocks = 1;
+  if (v) hipLaunchKernelGGL(groupnorm_apply_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, st, x, x_dtype, gamma, beta, mean, rstd, y, y_dtype, total, HW, C, groups);
+  else hipLaunchKernelGGL(groupnorm_apply_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, x, x_dtype, gamma, beta, mean, rstd, y, y_dtype, total, HW, C, groups);
+  PF_CHECK_LAUNCH("pf_groupnorm_fwd");
+  return PF_OK;
+}
+
+extern "C" int pf_groupnorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, const float* gamma,
+                                const float* mean, const float* rstd, void* dx, int dx_dtype, float* dgamma_acc,
+                                float* dbeta_acc, float* workspace, int64_t B, int64_t HW, int64_t C, int groups,
+                                int defer_reduce, void* stream) {
+  PF_REQUIRE(B >= 0 && HW > 0 && C > 0 && groups > 0 && C % groups == 0, "pf_groupnorm_bwd: bad shape");
+  if (B == 0) return PF_OK;
+  PF_REQUIRE(C / groups <= 64, "pf_groupnorm_bwd: more than 64 channels per group");
+  PF_REQUIRE(dy && x && gamma && mean && rstd && dx && workspace, "pf_groupnorm_bwd: null pointer");
+  PF_REQUIRE(pf_is_float_dtype(dy_dtype) && pf_is_float_dtype(x_dtype) && pf_is_float_dtype(dx_dtype),
+             "pf_groupnorm_bwd: bad dtype");
+  hipStream_t st = (hipStream_t)stream;
+  float* ws = workspace;                 // [B][2][C] channel partials
+  float* c12 = workspace + B * 2 * C;    // [B*G][2]
+  hipLaunchKernelGGL(groupnorm_bwd_stats_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, dy, dy_dtype, x,
+                     x_dtype, gamma, mean, rstd, c12, ws, HW, C, groups);
+  const int64_t total = B * HW * C;
+  const bool v = (C / groups) % 8 == 0 && vec_ok(dy, dy_dtype, C) && vec_ok(x, x_dtype, C) && vec_ok(dx, dx_dtype, C) &&
+                 vec_ok(gamma, PF_F32, C);
+  int64_t blocks = (total / (v ? 8 : 1) + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  if (blocks < 1) blocks = 1;
+  if (v) hipLaunchKernelGGL(groupnorm_bwd_apply_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, st, dy, dy_dtype, x, x_dtype, gamma, mean, rstd, c12, dx, dx_dtype, total, HW, C, groups);
+  else hipLaunchKernelGGL(groupnorm_bwd_apply_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, st, dy, dy_dtype, x, x_dtype, gamma, mean, rstd, c12, dx, dx_dtype, total, HW, C, groups);
+  PF_CHECK_LAUNCH("pf_groupnorm_bwd");
+  if (!defer_reduce) {
+    const dim3 fg((unsigned)((C + 31) / 32));
+    if (dgamma_acc) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws, (int)B, 2 * C, C, dgamma_acc);
+    if (dbeta_acc) hipLaunchKernelGGL(colreduce_finalize_kernel, fg, dim3(256), 0, st, ws + C, (int)B, 2 * C, C, dbeta_acc);
+    PF_CHECK_LAUNCH("pf_groupnorm_bwd(finalize)");
+  }
+  return PF_OK;
+}
+
+extern "C" int64_t pf_groupnorm_workspace(int64_t B, int64_t C, int groups) { return B * 2 * C + B * groups * 2; }
 
 extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
                                     float* workspace, int defer_reduce, void* stream) {

@@ -79,6 +79,20 @@ class ParamStore:
             self._keep.append(tensor)
         return sh
 
+    def shadow_perm(self, tensor, dtype, perm):
+        """Contiguous copy of tensor.permute(perm) in `dtype` (e.g. conv weights as [O, kh, kw, C]),
+        refreshed once per step."""
+        key = (tensor.data_ptr(), tuple(tensor.shape), tensor.dtype, dtype, tuple(perm))
+        sh = self._shadow.get(key)
+        if sh is None:
+            src = tensor.detach().permute(*perm)
+            sh = torch.empty(src.shape, dtype=dtype, device=tensor.device)
+            sizes, ss, ds = collapse_for_copy(src.shape, src.stride(), sh.stride())
+            self.refresh.append(self.kernels.copy_strided(src, ss, sh, ds, sizes, 0))
+            self._shadow[key] = sh
+            self._keep.append(tensor)
+        return sh
+
     def grad(self, param):
         g = self._grads.get(id(param))
         if g is None:
@@ -857,8 +871,12 @@ def lower_conv2d(L, node):
     pair = lambda v: (v, v) if isinstance(v, int) else tuple(v)
     stride, padding, dilation = pair(stride), pair(padding), pair(dilation)
     O, C, kh, kw_ = w.shape
+    if (groups == 1 and dilation == (1, 1) and stride == (1, 1) and kh == kw_ and kh in (1, 3)
+            and padding == (kh // 2, kh // 2)):
+        return _lower_conv_same(L, x, w, b, kh)
     if groups != 1 or dilation != (1, 1) or padding != (0, 0) or stride != (kh, kw_):
-        raise Unsupported("conv2d other than a non-overlapping patch projection (kernel == stride, no padding)")
+        raise Unsupported("conv2d other than a patch projection (kernel == stride, no padding) or a 1x1 / 3x3 "
+                          "stride-1 'same' convolution")
     Bn, Cx, H, W = x.shape
     if Cx != C or H % kh or W % kw_:
         raise Unsupported("conv2d patch projection with ragged image size")
@@ -902,6 +920,151 @@ def lower_conv2d(L, node):
             if prev is not None and prev is not dst:
                 B.copy(prev, dst)
             B.copy(dcols.view(sizes), dview, accumulate=prev is not None)
+            B.commit(x, dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+
+def as_nhwc(L, t, dtype=None):
+    """Channels-last contiguous [B, H, W, C] tensor holding the logical NCHW tensor t (a view when
+    t already lives in channels-last memory with the wanted dtype, a copy kernel otherwise)."""
+    dtype = dtype or t.dtype
+    p = t.permute(0, 2, 3, 1)
+    if p.is_contiguous() and t.dtype == dtype:
+        return p
+    out = L.alloc(p.shape, dtype)
+    L.copy(p, out)
+    return out
+
+
+def _grad_nhwc(B, g, dtype):
+    """Gradient of a logical-NCHW value as a contiguous channels-last matrix source."""
+    p = g.permute(0, 2, 3, 1)
+    if p.is_contiguous() and g.dtype == dtype:
+        return p
+    t = B.temp(p.shape, dtype)
+    B.copy(p, t)
+    return t
+
+
+def _lower_conv_same(L, x, w, b, k):
+    """1x1 or 3x3 stride-1 'same' convolution as one GEMM over channels-last rows
+    (3x3: the nine shifted windows of a zero-bordered copy are laid side by side first)."""
+    cd = L.cd
+    Bn, C, H, W = x.shape
+    O = w.shape[0]
+    M = Bn * H * W
+    xn = as_nhwc(L, x.buf, cd)
+    if k == 1:
+        cols, Kc = xn.reshape(M, C), C
+        w_cd = L.params.shadow(w.buf, cd).reshape(O, C)
+    else:
+        Kc = 9 * C
+        padded = torch.zeros((Bn, H + 2, W + 2, C), dtype=cd, device=L.device)  # border stays zero for good
+        L.cur.fwd_bytes += padded.numel() * padded.element_size()
+        L.copy(xn, padded[:, 1:H + 1, 1:W + 1, :])
+        cols = L.alloc((M, Kc), cd)
+        ps = padded.stride()
+        win = torch.as_strided(padded, (Bn, H, W, 3, 3, C), (ps[0], ps[1], ps[2], ps[1], ps[2], 1))
+        L.copy(win, cols.view(Bn, H, W, 3, 3, C))
+        w_cd = L.params.shadow_perm(w.buf, cd, (0, 2, 3, 1)).reshape(O, Kc)
+    b_cd = None if b is None else L.params.shadow(b.buf, cd)
+    out = L.alloc((Bn, H, W, O), cd)
+    L.emit(L.kernels.gemm(cols, w_cd, out, M=M, N=O, K=Kc, lda=Kc, ldb=Kc, ldc=O, bias=b_cd,
+                          round_mid=1 if L.mixed else 0))
+    req = x.req_grad or w.req_grad or (b is not None and b.req_grad)
+    outv = Val(out.permute(0, 3, 1, 2), req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        dy = _grad_nhwc(B, g, cd).reshape(M, O)
+        if w.req_grad and w.param is not None:
+            wg = L.params.grad(w.param)
+            if k == 1:
+                B.emit(B.k.gemm(dy, cols, wg, M=O, N=Kc, K=M, lda=O, ldb=Kc, ldc=Kc, a_trans=1, b_trans=1, beta=1))
+            else:
+                tmp = B.temp((O, 3, 3, C), torch.float32)
+                B.emit(B.k.gemm(dy, cols, tmp, M=O, N=Kc, K=M, lda=O, ldb=Kc, ldc=Kc, a_trans=1, b_trans=1))
+                B.copy(tmp, wg.permute(0, 2, 3, 1), accumulate=True)
+        if b is not None and b.req_grad and b.param is not None:
+            B.colsum_into(dy, M, O, O, L.params.grad(b.param))
+        if x.req_grad:
+            dst, prev = B.grad_target(x)
+            dstn = dst.permute(0, 2, 3, 1)
+            if k == 1:
+                direct = prev is None and dstn.is_contiguous()
+                t = dstn if direct else B.temp((Bn, H, W, C), x.dtype)
+                B.emit(B.k.gemm(dy, w_cd, t, M=M, N=C, K=O, lda=O, ldb=C, ldc=C, b_trans=1))
+                if not direct:
+                    B.merge(t, dstn, None if prev is None else prev.permute(0, 2, 3, 1))
+            else:
+                dcols = B.temp((M, Kc), cd)
+                B.emit(B.k.gemm(dy, w_cd, dcols, M=M, N=Kc, K=O, lda=O, ldb=Kc, ldc=Kc, b_trans=1))
+                dpad = B.temp((Bn, H + 2, W + 2, C), torch.float32)
+                B.emit(B.k.fill(dpad, 0.0, dpad.numel()))
+                dc = dcols.view(Bn, H, W, 3, 3, C)
+                for i in range(3):
+                    for j in range(3):   # nine bijective shifted adds, one after the other on the stream
+                        B.copy(dc[:, :, :, i, j, :], dpad[:, i:i + H, j:j + W, :], accumulate=True)
+                B.merge(dpad[:, 1:H + 1, 1:W + 1, :], dstn, None if prev is None else prev.permute(0, 2, 3, 1))
+            B.commit(x, dst)
+
+    if req:
+        L.add_backward(bwd)
+    return outv
+
+
+def lower_group_norm(L, node):
+    x = L.arg(node.args[0])
+    groups = int(_kw(node, 1, "num_groups"))
+    gamma = L.arg(_kw(node, 2, "weight"))
+    beta = L.arg(_kw(node, 3, "bias"))
+    eps = float(_kw(node, 4, "eps", 1e-5))
+    if x.buf.dim() != 4 or gamma is None or beta is None:
+        raise Unsupported("group_norm other than affine on [B, C, H, W]")
+    Bn, C, H, W = x.shape
+    xn = as_nhwc(L, x.buf)
+    # fp32 result under autocast; written in the compute dtype when it only feeds matrix products,
+    # directly or through one activation
+    users = list(node.users)
+    to_cd = L.consumers_cast_to_cd(node) or (
+        L.mixed and len(users) == 1 and _act_of_node(users[0]) is not None and L.consumers_cast_to_cd(users[0]))
+    y_dtype = L.cd if to_cd else (torch.float32 if L.mixed else x.dtype)
+    y = L.alloc((Bn, H, W, C), y_dtype)
+    mean = L.alloc((Bn * groups,), torch.float32)
+    rstd = L.alloc((Bn * groups,), torch.float32)
+    g32 = gamma.buf if gamma.dtype == torch.float32 else L.params.shadow(gamma.buf, torch.float32)
+    b32 = beta.buf if beta.dtype == torch.float32 else L.params.shadow(beta.buf, torch.float32)
+    L.emit(L.kernels.groupnorm_fwd(xn, g32, b32, y, mean, rstd, Bn, H * W, C, groups, eps))
+    req = x.req_grad or gamma.req_grad or beta.req_grad
+    outv = Val(y.permute(0, 3, 1, 2), req_grad=req)
+
+    def bwd(B):
+        g = B.grad_of(outv)
+        if g is None:
+            return
+        gn = _grad_nhwc(B, g, g.dtype)
+        ws = B.temp((B.k.groupnorm_workspace(Bn, C, groups),), torch.float32)
+        if x.req_grad:
+            dst, prev = B.grad_target(x)
+            dstn = dst.permute(0, 2, 3, 1)
+            direct = prev is None and dstn.is_contiguous()
+            t = dstn if direct else B.temp((Bn, H, W, C), x.dtype)
+        else:
+            t = B.temp((Bn, H, W, C), x.dtype)
+        B.emit(B.k.groupnorm_bwd(gn, xn, g32, mean, rstd, t, None, None, ws, Bn, H * W, C, groups, defer=1))
+        if gamma.req_grad and gamma.param is not None:
+            B.reduces.append((ws, 0, Bn, 2 * C, C, L.params.grad(gamma.param)))
+        if beta.req_grad and beta.param is not None:
+            B.reduces.append((ws, C, Bn, 2 * C, C, L.params.grad(beta.param)))
+        if x.req_grad:
+            if not direct:
+                B.merge(t, dstn, None if prev is None else prev.permute(0, 2, 3, 1))
             B.commit(x, dst)
 
     if req:
@@ -1162,6 +1325,32 @@ def lower_add(L, node):
         if req:
             L.add_backward(bwd)
         return outv
+    # per-sample, per-channel vector added to every pixel: [B, C, H, W] + [B, C, 1, 1]
+    if (a.buf.dim() == 4 and b.buf.dim() == 4 and b.shape == (a.shape[0], a.shape[1], 1, 1)
+            and a.buf.permute(0, 2, 3, 1).is_contiguous() and b.buf.reshape(-1).is_contiguous()
+            and b.buf.stride(1) == 1):
+        Bn, C, H, W = a.shape
+        out = L.alloc((Bn, H, W, C), out_dtype)
+        L.emit(L.kernels.bias_add(a.buf, b.buf, out, Bn * H * W * C, C, H * W))
+        outv = Val(out.permute(0, 3, 1, 2), req_grad=req)
+
+        def bwd_chan(B):
+            g = B.grad_of(outv)
+            if g is None:
+                return
+            B.contribute(a, g)
+            if b.req_grad:
+                gn = _grad_nhwc(B, g, g.dtype).reshape(Bn, H * W, C)
+                acc = B.temp((Bn, C), torch.float32)
+                B.emit(B.k.fill(acc, 0.0, acc.numel()))
+                ws = B.temp((B.k.colreduce_workspace(H * W, C),), torch.float32)
+                for i in range(Bn):
+                    B.emit(B.k.colsum_accumulate(gn[i], H * W, C, C, acc[i], ws))
+                B.contribute(b, acc.view(Bn, C, 1, 1))
+
+        if req:
+            L.add_backward(bwd_chan)
+        return outv
     # broadcast of b over the leading dimensions of a
     bshape = tuple(b.shape)
     while bshape and bshape[0] == 1:
@@ -1198,9 +1387,10 @@ def lower_add(L, node):
 def lower_unary_act(L, node):
     act = _act_of_node(node)
     x = L.arg(node.args[0])
-    if not x.buf.is_contiguous():
-        raise Unsupported("activation on a non-contiguous tensor")
-    y = L.alloc(x.shape, x.dtype)
+    if not is_dense(x.buf):
+        raise Unsupported("activation on a non-dense tensor")
+    y = torch.empty_like(x.buf)   # same (possibly permuted) dense layout: the kernel walks flat memory
+    L.cur.fwd_bytes += y.numel() * y.element_size()
     L.emit(L.kernels.act_fwd(x.buf, y, act, y.numel()))
     outv = Val(y, req_grad=x.req_grad)
 
@@ -1208,20 +1398,17 @@ def lower_unary_act(L, node):
         g = B.grad_of(outv)
         if g is None:
             return
-        gc = g if (g.is_contiguous() and g.dtype == x.dtype) else _compact(B, g)
+        if not (g.dtype == x.dtype and g.stride() == x.buf.stride()):
+            t = B.new_like(y)
+            B.copy(g, t)
+            g = t
         dst, prev = B.grad_target(x)
-        if prev is None and dst.is_contiguous():
-            B.emit(B.k.act_bwd(gc, x.buf, dst, act, y.numel()))
+        if prev is None and dst.stride() == x.buf.stride() and dst.dtype == x.dtype:
+            B.emit(B.k.act_bwd(g, x.buf, dst, act, y.numel()))
         else:
-            tmp = B.temp(x.shape, x.dtype)
-            B.emit(B.k.act_bwd(gc, x.buf, tmp, act, y.numel()))
-            if prev is None:
-                B.copy(tmp, dst)
-            elif prev is dst:
-                B.copy(tmp, dst, accumulate=True)
-            else:
-                B.copy(prev, dst)
-                B.copy(tmp, dst, accumulate=True)
+            tmp = B.new_like(y)
+            B.emit(B.k.act_bwd(g, x.buf, tmp, act, y.numel()))
+            B.merge(tmp, dst, prev)
         B.commit(x, dst)
 
     if x.req_grad:
@@ -1523,6 +1710,7 @@ FUNCTION_HANDLERS = {
     F.linear: lower_linear, torch._C._nn.linear: lower_linear,
     F.layer_norm: lower_layer_norm, torch.layer_norm: lower_layer_norm,
     F.rms_norm: lower_rms_norm, torch.rms_norm: lower_rms_norm,
+    F.group_norm: lower_group_norm, torch.group_norm: lower_group_norm,
     F.scaled_dot_product_attention: lower_sdpa, torch._C._nn.scaled_dot_product_attention: lower_sdpa,
     F.conv2d: lower_conv2d, torch.conv2d: lower_conv2d,
     F.gelu: lower_act_maybe_gate, torch._C._nn.gelu: lower_act_maybe_gate,

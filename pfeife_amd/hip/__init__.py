@@ -100,7 +100,9 @@ _SIGNATURES = {
     "pf_glu_fwd": [_P, _L, _P, _L, _P, _L, _I, _I, _L, _L, _P],
     "pf_glu_bwd": [_P, _L, _P, _L, _P, _L, _P, _L, _P, _L, _I, _I, _L, _L, _P],
     "pf_axpby": [_P, _I, _F, _P, _I, _F, _P, _I, _L, _P],
-    "pf_bias_add": [_P, _I, _P, _I, _P, _I, _L, _L, _P],
+    "pf_bias_add": [_P, _I, _P, _I, _P, _I, _L, _L, _L, _P],
+    "pf_groupnorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _L, _I, _F, _P],
+    "pf_groupnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P],
     "pf_cast": [_P, _I, _P, _I, _L, _P],
     "pf_transpose_cast": [_P, _I, _L, _P, _I, _L, _L, _L, _P],
     "pf_fill": [_P, _I, _F, _L, _P],
@@ -112,7 +114,7 @@ _SIGNATURES = {
     "pf_embedding_fwd": [_P, _I, _P, _P, _I, _L, _L, _L, _P],
     "pf_embedding_bwd": [_P, _I, _P, _P, _L, _L, _L, _P],
 }
-_RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L]}
+_RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L], "pf_groupnorm_workspace": [_L, _L, _I]}
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_RET_I64) + ["pf_version", "pf_last_error"])
 
 _lib = None
@@ -274,6 +276,19 @@ class HipKernels:
                 _ptr(dx), _dt(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), rows, d, int(defer))
         return self._prep("pf_layernorm_bwd", args, (dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws))
 
+    def groupnorm_workspace(self, B, C, groups):
+        return int(self.lib.pf_groupnorm_workspace(B, C, groups))
+
+    def groupnorm_fwd(self, x, gamma, beta, y, mean, rstd, B, HW, C, groups, eps):
+        args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(beta), _ptr(y), _dt(y), _ptr(mean), _ptr(rstd), B, HW, C, groups,
+                eps)
+        return self._prep("pf_groupnorm_fwd", args, (x, gamma, beta, y, mean, rstd))
+
+    def groupnorm_bwd(self, dy, x, gamma, mean, rstd, dx, dgamma, dbeta, ws, B, HW, C, groups, defer=0):
+        args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx), _dt(dx),
+                _ptr(dgamma), _ptr(dbeta), _ptr(ws), B, HW, C, groups, int(defer))
+        return self._prep("pf_groupnorm_bwd", args, (dy, x, gamma, mean, rstd, dx, dgamma, dbeta, ws))
+
     def rmsnorm_fwd(self, x, gamma, y, rstd, rows, d, eps):
         args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(y), _dt(y), _ptr(rstd), rows, d, eps)
         return self._prep("pf_rmsnorm_fwd", args, (x, gamma, y, rstd))
@@ -357,8 +372,8 @@ class HipKernels:
         args = (_ptr(a), _dt(a), alpha, _ptr(b), _dt(b), beta, _ptr(out), _dt(out), n)
         return self._prep("pf_axpby", args, (a, b, out))
 
-    def bias_add(self, x, bias, y, n, bias_len):
-        args = (_ptr(x), _dt(x), _ptr(bias), _dt(bias), _ptr(y), _dt(y), n, bias_len)
+    def bias_add(self, x, bias, y, n, bias_len, rows_per_bias=0):
+        args = (_ptr(x), _dt(x), _ptr(bias), _dt(bias), _ptr(y), _dt(y), n, bias_len, rows_per_bias)
         return self._prep("pf_bias_add", args, (x, bias, y))
 
     def cast(self, src, dst, n):

@@ -478,3 +478,33 @@ def test_fused_attention(hip, oracle, dtype, case):
     torch.testing.assert_close(res["oracle"][0], ref.detach(), rtol=3e-2, atol=3e-2)
     for g, r in ((res["oracle"][2], qf.grad), (res["oracle"][3], kf.grad), (res["oracle"][4], vf.grad)):
         torch.testing.assert_close(g, r, rtol=5e-2, atol=5e-2)
+
+
+@pytest.mark.parametrize("xdt,ydt", [(F32, F32), (F16, F16), (F32, BF16)])
+def test_groupnorm_and_channel_bias(hip, oracle, xdt, ydt):
+    for B, HW, C, G in [(4, 1024, 1280, 32), (2, 64, 64, 8), (3, 49, 96, 32)]:
+        x = rnd((B, HW, C), xdt, 1) * 2 + 0.3
+        gamma, beta = rnd((C,), F32, 2) + 1, rnd((C,), F32, 3)
+        t = dict(x=x, gamma=gamma, beta=beta, y=torch.zeros(B, HW, C, dtype=ydt), mean=torch.zeros(B * G),
+                 rstd=torch.zeros(B * G))
+        r = both(hip, oracle, "groupnorm_fwd", t, ["y", "mean", "rstd"], B=B, HW=HW, C=C, groups=G, eps=1e-5)
+        close(r["y"], *TOL[ydt])
+        close(r["mean"], 1e-5, 1e-5)
+        close(r["rstd"], 1e-4, 1e-5)
+        ref = torch.nn.functional.group_norm(x.float().permute(0, 2, 1), G, gamma, beta, 1e-5).permute(0, 2, 1)
+        torch.testing.assert_close(r["y"][1].float(), ref.to(ydt).float(), rtol=TOL[ydt][0], atol=TOL[ydt][1])
+        dy = rnd((B, HW, C), ydt, 4)
+        need = hip.groupnorm_workspace(B, C, G)
+        t = dict(dy=dy, x=x, gamma=gamma, mean=r["mean"][1], rstd=r["rstd"][1], dx=torch.zeros(B, HW, C, dtype=xdt),
+                 dgamma=rnd((C,), F32, 5), dbeta=rnd((C,), F32, 6), ws=torch.zeros(need))
+        r = both(hip, oracle, "groupnorm_bwd", t, ["dx", "dgamma", "dbeta"], B=B, HW=HW, C=C, groups=G)
+        close(r["dx"], TOL[xdt][0] * 2, TOL[xdt][1] * 2)
+        close(r["dgamma"], 1e-3, 1e-3 * (B * HW) ** 0.5)
+        close(r["dbeta"], 1e-3, 1e-3 * (B * HW) ** 0.5)
+    # per-sample vector added to every row of that sample
+    B, HW, C = 3, 50, 64
+    x, bias = rnd((B * HW, C), xdt, 7), rnd((B, C), xdt, 8)
+    r = both(hip, oracle, "bias_add", dict(x=x, bias=bias, y=torch.zeros(B * HW, C, dtype=F32)), ["y"],
+             n=B * HW * C, bias_len=C, rows_per_bias=HW)
+    close(r["y"], 1e-6, 1e-6)
+    torch.testing.assert_close(r["y"][1], (x.float().view(B, HW, C) + bias.float()[:, None, :]).view(B * HW, C))

@@ -244,3 +244,59 @@ def test_vit_g_block_share_head_dim_88(mixed):
     for a, b in zip(losses, want):
         assert abs(float(a) - float(b)) <= ltol * abs(float(b)) + 1e-3, (float(a), float(b))
     _check_grads(model, ref, mixed)
+
+
+@pytest.mark.parametrize("mixed", [None, "fp16"])
+def test_unet_stage_sdxl_style(mixed):
+    """BASELINE config 4 at reduced width: ResNet blocks (GroupNorm 32, 3x3 convs, time
+    embedding), spatial transformers with self- and cross-attention to 77 context tokens,
+    GEGLU; MSE loss against an N(0,1) target computed in user code."""
+    import torch.nn.functional as F
+
+    from pfeife_amd.bench_models.unet_stage import UNetStage, UNetStageConfig
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = UNetStageConfig(in_channels=128, channels=256, temb_dim=256, context_dim=512, heads=4, layers=2, groups=32)
+    torch.manual_seed(0)
+    model = UNetStage(cfg)
+    ref = copy.deepcopy(model)
+    g = torch.Generator().manual_seed(42)
+    B, hw = 4, 16
+    hidden = torch.randn(B, cfg.in_channels, hw, hw, generator=g)
+    temb = torch.randn(B, cfg.temb_dim, generator=g)
+    ctx = torch.randn(B, 77, cfg.context_dim, generator=g)
+    target = torch.randn(B, cfg.channels, hw, hw, generator=g)
+    option = PipeOption(device_cnt=1, batch_cnt=2, batch_size=2, mixed_precision=mixed,
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(h, t, c, y):
+        out = cmodel(h, t, c)
+        loss = F.mse_loss(out.float(), y.float())
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    losses = runner.step(hidden.cuda(), temb.cuda(), ctx.cuda(), target.cuda())
+    torch.cuda.synchronize()
+    adt = {"fp16": torch.float16}.get(mixed)
+    for p in ref.parameters():
+        p.grad = torch.zeros_like(p)
+    want = []
+    for i in range(2):
+        sl = slice(2 * i, 2 * i + 2)
+        if adt is None:
+            out = ref(hidden[sl], temb[sl], ctx[sl])
+        else:
+            with torch.autocast("cpu", dtype=adt):
+                out = ref(hidden[sl], temb[sl], ctx[sl])
+        loss = F.mse_loss(out.float(), target[sl].float())
+        loss.backward()
+        want.append(loss.detach())
+    ltol = 1e-5 if mixed is None else 2e-2
+    for a, b in zip(losses, want):
+        assert abs(float(a) - float(b)) <= ltol * abs(float(b)), (float(a), float(b))
+    _check_grads(model, ref, mixed)
