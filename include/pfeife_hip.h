@@ -46,6 +46,18 @@ const char* pf_last_error(void);
  * (pfeife/mp/net_states.py:131-132). */
 int pf_init(int device);
 
+/* ---- launch-list replay -------------------------------------------------------------
+ * The job loop of a step (pfeife/mp/worker.py:912-1006) issues the same kernels on the same
+ * buffers every step.  Bracket one job's launches (ordinary calls of the entry points
+ * below, on `stream`) with capture_begin / capture_end to obtain a hipGraphExec handle;
+ * pf_graph_launch replays it with one host call.  `stream` must be a created stream (not
+ * the legacy default stream).  No hipMemset nodes are ever recorded: every clear in this
+ * library is a fill kernel. */
+int pf_graph_capture_begin(void* stream);
+int pf_graph_capture_end(void* stream, void** graph_exec_out);
+int pf_graph_launch(void* graph_exec, void* stream);
+int pf_graph_destroy(void* graph_exec);
+
 /* ---- dense contractions (MFMA) -------------------------------------------
  * One descriptor covers every matrix product a stage executes:
  *   C[z] = epilogue( alpha * op(A[z]) . op(B[z]) )        for z in [0, batch1*batch2)

@@ -69,6 +69,7 @@ def _rows(t, rows, cols, ld):
 
 class OracleKernels:
     name = "oracle"
+    supports_graphs = False
 
     def __init__(self, device="cpu"):
         self.device = torch.device(device)

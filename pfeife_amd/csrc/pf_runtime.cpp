@@ -44,3 +44,50 @@ extern "C" int pf_init(int device) {
   }
   return PF_OK;
 }
+
+// ---- hipGraph capture of launch lists ---------------------------------------------
+// A stage job is a fixed list of kernel launches on fixed buffers, so it is captured once
+// (stream capture around the ordinary entry points) and replayed with one call per job.
+extern "C" int pf_graph_capture_begin(void* stream) {
+  PF_REQUIRE(stream != nullptr, "pf_graph_capture_begin: the legacy default stream cannot be captured");
+  hipError_t e = hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) {
+    pf_set_error("pf_graph_capture_begin: %s", hipGetErrorString(e));
+    return PF_ERR_HIP;
+  }
+  return PF_OK;
+}
+
+extern "C" int pf_graph_capture_end(void* stream, void** graph_exec_out) {
+  PF_REQUIRE(stream != nullptr && graph_exec_out != nullptr, "pf_graph_capture_end: bad arguments");
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture((hipStream_t)stream, &graph);
+  if (e != hipSuccess || graph == nullptr) {
+    pf_set_error("pf_graph_capture_end: %s", hipGetErrorString(e));
+    return PF_ERR_HIP;
+  }
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  hipGraphDestroy(graph);
+  if (e != hipSuccess) {
+    pf_set_error("pf_graph_capture_end: instantiate: %s", hipGetErrorString(e));
+    return PF_ERR_HIP;
+  }
+  *graph_exec_out = (void*)exec;
+  return PF_OK;
+}
+
+extern "C" int pf_graph_launch(void* graph_exec, void* stream) {
+  PF_REQUIRE(graph_exec != nullptr, "pf_graph_launch: null graph");
+  hipError_t e = hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream);
+  if (e != hipSuccess) {
+    pf_set_error("pf_graph_launch: %s", hipGetErrorString(e));
+    return PF_ERR_HIP;
+  }
+  return PF_OK;
+}
+
+extern "C" int pf_graph_destroy(void* graph_exec) {
+  if (graph_exec) hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+  return PF_OK;
+}

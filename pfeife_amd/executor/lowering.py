@@ -162,12 +162,20 @@ class StageProgram:
         self.input_grads = []   # filled by lower_backward: gradient tensor (or None) per input
         self.fwd_bytes = 0
         self.tile_groups = []   # sibling regions that must all be written for the zero-fill to be skipped
+        self.fwd_graph = None   # replay callables once the launch lists have been captured
+        self.bwd_graph = None
 
     def run_forward(self, stream):
+        if self.fwd_graph is not None:
+            self.fwd_graph(stream)
+            return
         for launch in self.fwd:
             launch(stream)
 
     def run_backward(self, stream):
+        if self.bwd_graph is not None:
+            self.bwd_graph(stream)
+            return
         for launch in self.bwd:
             launch(stream)
 

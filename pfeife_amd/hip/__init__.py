@@ -76,6 +76,10 @@ class AttnDesc(Structure):
 _P, _I, _L, _F = c_void_p, c_int, c_int64, c_float
 _SIGNATURES = {
     "pf_init": [_I],
+    "pf_graph_capture_begin": [_P],
+    "pf_graph_capture_end": [_P, POINTER(c_void_p)],
+    "pf_graph_launch": [_P, _P],
+    "pf_graph_destroy": [_P],
     "pf_gemm": [POINTER(GemmDesc), _P],
     "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
     "pf_attention_fwd": [POINTER(AttnDesc), _P],
@@ -174,6 +178,7 @@ class HipKernels:
     """
 
     name = "hip"
+    supports_graphs = True
 
     def __init__(self, device=None):
         self.lib = load()
@@ -199,6 +204,31 @@ class HipKernels:
 
     def run(self, name, *a, **kw):
         getattr(self, name)(*a, **kw)(current_stream_ptr())
+
+    def capture(self, launches, stream):
+        """Record `launches` (prepared launches) into a hipGraph on `stream`; returns a replay
+        callable `fn(stream)` that issues the whole list with one host call."""
+        lib = self.lib
+        rc = lib.pf_graph_capture_begin(stream)
+        if rc != 0:
+            raise RuntimeError("graph capture: %s" % lib.pf_last_error().decode())
+        try:
+            for launch in launches:
+                launch(stream)
+        finally:
+            handle = c_void_p()
+            rc = lib.pf_graph_capture_end(stream, byref(handle))
+        if rc != 0:
+            raise RuntimeError("graph capture: %s" % lib.pf_last_error().decode())
+        h = handle.value
+
+        def replay(s, _h=h, _fn=lib.pf_graph_launch, _keep=launches):
+            if _fn(_h, s) != 0:
+                raise RuntimeError("graph launch: %s" % lib.pf_last_error().decode())
+
+        replay.kernel = "pf_graph_launch"
+        replay.handle = h
+        return replay
 
     def colreduce_workspace(self, rows, cols):
         return int(self.lib.pf_colreduce_workspace(rows, cols))

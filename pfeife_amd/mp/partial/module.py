@@ -73,6 +73,19 @@ class PartialRunner:
 
     # -- one optimisation step ---------------------------------------------------
     def step(self, *args, **kwargs):
+        """One optimisation step.  All device work of the step is issued on the worker's own
+        stream, ordered after the caller's current stream on entry and before it on exit."""
+        so = self.worker.stream_obj
+        if so is None:
+            return self._step(*args, **kwargs)
+        outer = torch.cuda.current_stream(so.device)
+        so.wait_stream(outer)
+        with torch.cuda.stream(so):
+            out = self._step(*args, **kwargs)
+        outer.wait_stream(so)
+        return out
+
+    def _step(self, *args, **kwargs):
         if self.exec_fn is None:
             raise RuntimeError("call set_exec_fn() before step()")
         option = self.option
@@ -110,6 +123,7 @@ class PartialRunner:
             if is_fwd and worker.last_forward.get(i) == mb:
                 self.finalize_output(mb)
         worker.optimizer_step()
+        worker.steps_done += 1
         return self._take_results()
 
     def _take_results(self):
@@ -153,9 +167,12 @@ class PartialRunner:
         while True:
             args, kwargs = q.get()
             try:
-                if self.net_state.device.type == "cuda":
+                if self.worker.stream_obj is not None:
                     torch.cuda.set_device(self.net_state.device)
-                ret = self.exec_fn(*args, **kwargs)
+                    with torch.cuda.stream(self.worker.stream_obj):   # user code shares the step's stream
+                        ret = self.exec_fn(*args, **kwargs)
+                else:
+                    ret = self.exec_fn(*args, **kwargs)
             except BaseException as e:  # surfaced on the thread that called step()
                 ret = _ExecError(e)
             self._return_queues[batch_idx].put(ret)

@@ -13,6 +13,8 @@ every stage:
     producer's output buffer and writes the gradient buffer its producer reads;
   * `_init_optimizer` / `optimizer_step` (worker.py:583-597, 1432-1436).
 """
+import os
+
 import torch
 
 from ..executor.lowering import BufferPool, Lowerer, ParamStore
@@ -55,6 +57,14 @@ class StageWorker:
         self.order = []
         self.optimizer = None
         self.mem_usage_info = {}
+        # every launch of a step goes to one created stream (default priority): a created
+        # stream can be captured into hipGraphs, the legacy default stream cannot
+        self.stream_obj = torch.cuda.Stream(self.device) if self.device.type == "cuda" else None
+        self.use_graphs = (bool(getattr(kernels, "supports_graphs", False)) and self.stream_obj is not None
+                           and os.environ.get("PFEIFE_NO_GRAPH", "0") != "1")
+        self.graphs_ready = False
+        self.steps_done = 0
+        self.begin_graph = None
 
     # -- graph ---------------------------------------------------------------------
     def set_partition_graph(self, part_graph, example_inputs):
@@ -182,13 +192,29 @@ class StageWorker:
                     out_grads[ref[1]].append(slot.loss_grads[oi])
             L.lower_backward(prog, out_grads)
         self.mbs[mb] = slot
+        self.graphs_ready = False   # new programs (and possibly new parameters): capture again
+        self.begin_graph = None
         return slot
 
     # -- per step --------------------------------------------------------------------
     def stream(self):
-        if self.device.type == "cuda":
-            return torch.cuda.current_stream(self.device).cuda_stream
-        return None
+        return self.stream_obj.cuda_stream if self.stream_obj is not None else None
+
+    def capture_graphs(self):
+        """Record every job's launch list (and the per-step zero/refresh list) into hipGraphs.
+        Called after one complete eager step, when every program exists and every kernel has
+        run once (so one-time function attributes are set)."""
+        s = self.stream()
+        for slot in self.mbs.values():
+            for prog in slot.stage_programs.values():
+                if prog.fwd_graph is None and prog.fwd:
+                    prog.fwd_graph = self.kernels.capture(prog.fwd, s)
+                if prog.bwd_graph is None and prog.bwd:
+                    prog.bwd_graph = self.kernels.capture(prog.bwd, s)
+        pre = list(self.params.zero) + list(self.params.refresh)
+        self.begin_graph = self.kernels.capture(pre, s) if pre else None
+        self._begin_len = (len(self.params.zero), len(self.params.refresh))
+        self.graphs_ready = True
 
     def distribute_input(self, mb, placeholder_idx, value):
         """Copy one micro-batch slab into the stage input buffer it was built for."""
@@ -206,10 +232,15 @@ class StageWorker:
     def begin_step(self):
         s = self.stream()
         self.params.rebind_grads()
-        for launch in self.params.zero:      # optimizer.zero_grad(set_to_none=False)
-            launch(s)
-        for launch in self.params.refresh:   # one master -> 16-bit cast per step, not per micro-batch
-            launch(s)
+        if self.use_graphs and not self.graphs_ready and self.steps_done >= 1 and len(self.mbs) == self.option.batch_cnt:
+            self.capture_graphs()
+        if self.graphs_ready and self.begin_graph is not None:
+            self.begin_graph(s)
+        else:
+            for launch in self.params.zero:      # optimizer.zero_grad(set_to_none=False)
+                launch(s)
+            for launch in self.params.refresh:   # one master -> 16-bit cast per step, not per micro-batch
+                launch(s)
         for slot in self.mbs.values():
             slot.grad_seen.clear()
 
