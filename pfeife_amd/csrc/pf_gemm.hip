@@ -565,6 +565,7 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
 // the register file, so it is the ceiling here.  Smaller tiles are for problems
 // that would otherwise leave most of the 256 CUs without a workgroup.
 //   0: 128x128   1: 128x64   2: 64x64      (BK 64, 4 wavefronts)
+// (A 256x128 tile run by 8 wavefronts was measured too: same throughput as 128x128, so it is not built.)
 int choose_tile(const pf_gemm_desc& d) {
   const int64_t nb = (d.batch1 > 0 ? d.batch1 : 1) * (d.batch2 > 0 ? d.batch2 : 1);
   auto tiles = [&](int bm, int bn) { return ((d.M + bm - 1) / bm) * ((d.N + bn - 1) / bn) * nb; };
