@@ -41,18 +41,14 @@ template <> struct M32<PF_F16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0,
                                                   0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    return (uint32_t)pf_f32_to_f16_bits(lo) | ((uint32_t)pf_f32_to_f16_bits(hi) << 16);
-  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return pf_pack2_f16(lo, hi); }
 };
 template <> struct M32<PF_BF16> {
   static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
                                                    0, 0, 0);
   }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    return (uint32_t)pf_f32_to_bf16_bits(lo) | ((uint32_t)pf_f32_to_bf16_bits(hi) << 16);
-  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return pf_pack2_bf16(lo, hi); }
 };
 
 // registers r..r+7 of an accumulator tile -> one 16-byte MFMA operand (8 x 16-bit)
@@ -72,28 +68,38 @@ __device__ __forceinline__ uint4 load_row8(const uint16_t* base, int64_t st, int
   return make_uint4(0, 0, 0, 0);
 }
 
-// natural tile [ROWS tokens][HD + 8]: thread-strided 16-byte copies
-template <int ROWS, int HD>
-__device__ __forceinline__ void stage_natural(uint16_t* s, const uint16_t* base, int64_t st, int t0, int T, int hd,
-                                              int tid) {
-  constexpr int LD = HD + 8, VPR = HD / 8;
-  for (int e = tid; e < ROWS * VPR; e += 256) {
-    const int row = e / VPR, hv = e % VPR;
-    *(uint4*)(s + row * LD + hv * 8) = load_row8(base, st, t0 + row, T, hv * 8, hd);
+// One [KT tokens][HD] tile in flight: NV 16-byte vectors per thread, loaded from global into
+// registers while the previous tile is being multiplied, stored to LDS ([KT][HD + 8]) afterwards.
+template <int HD> struct Tile {
+  static constexpr int LD = HD + 8, VPR = HD / 8, NV = (KT * VPR + 255) / 256;
+  uint4 v[NV];
+  __device__ __forceinline__ void load(const uint16_t* base, int64_t st, int t0, int T, int hd, int tid) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = tid + i * 256;
+      v[i] = (e < KT * VPR) ? load_row8(base, st, t0 + e / VPR, T, (e % VPR) * 8, hd) : make_uint4(0, 0, 0, 0);
+    }
   }
-}
+  __device__ __forceinline__ void store(uint16_t* s, int tid) const {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int e = tid + i * 256;
+      if (e < KT * VPR) *(uint4*)(s + (e / VPR) * LD + (e % VPR) * 8) = v[i];
+    }
+  }
+};
 
-// transposed tile [HD][ROWS + 8] (element (h, t)): 8x8 register transposes
-template <int ROWS, int HD>
-__device__ __forceinline__ void stage_transposed(uint16_t* s, const uint16_t* base, int64_t st, int t0, int T, int hd,
-                                                 int tid) {
-  constexpr int LD = ROWS + 8, TB = ROWS / 8, HB = HD / 8;
+// LDS natural tile [KT][HD + 8] -> LDS transposed tile [HD][KT + 8] (element (h, t)):
+// 8x8 blocks transposed in registers, no global traffic
+template <int HD>
+__device__ __forceinline__ void transpose_tile(const uint16_t* nat, uint16_t* tr, int tid) {
+  constexpr int NLD = HD + 8, TLD = KT + 8, TB = KT / 8, HB = HD / 8;
   for (int b = tid; b < TB * HB; b += 256) {
-    const int tb = b % TB, hb = b / TB;  // consecutive threads: consecutive token blocks of the same 8 hd rows
+    const int hb = b % HB, tb = b / HB;   // consecutive threads: adjacent 16-byte chunks of the same 8 token rows
     uint32_t in[8][4];
 #pragma unroll
     for (int r = 0; r < 8; ++r) {
-      const uint4 x = load_row8(base, st, t0 + tb * 8 + r, T, hb * 8, hd);
+      const uint4 x = *(const uint4*)(nat + (tb * 8 + r) * NLD + hb * 8);
       in[r][0] = x.x; in[r][1] = x.y; in[r][2] = x.z; in[r][3] = x.w;
     }
 #pragma unroll
@@ -105,8 +111,8 @@ __device__ __forceinline__ void stage_transposed(uint16_t* s, const uint16_t* ba
         lo[I] = (a & 0xffffu) | (c << 16);
         hi[I] = (a >> 16) | (c & 0xffff0000u);
       }
-      *(uint4*)(s + (hb * 8 + 2 * J) * LD + tb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-      *(uint4*)(s + (hb * 8 + 2 * J + 1) * LD + tb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+      *(uint4*)(tr + (hb * 8 + 2 * J) * TLD + tb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+      *(uint4*)(tr + (hb * 8 + 2 * J + 1) * TLD + tb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
     }
   }
 }
@@ -128,6 +134,7 @@ template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
   constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8, VLD = KT + 8;
   __shared__ __align__(16) uint16_t sK[KT * KLD];
+  __shared__ __align__(16) uint16_t sV[KT * KLD];
   __shared__ __align__(16) uint16_t sVt[HD * VLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
@@ -155,10 +162,19 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     const int last_q = min(blockIdx.x * 128 + 127, a.Tq - 1);
     k_end = min(a.Tk, last_q + shift + 1);
   }
+  Tile<HD> tk, tv;
+  tk.load(K, a.k_st, 0, a.Tk, a.hd, tid);
+  tv.load(V, a.v_st, 0, a.Tk, a.hd, tid);
   for (int k0 = 0; k0 < k_end; k0 += KT) {
+    __syncthreads();                     // previous tile's LDS reads are done
+    tk.store(sK, tid);
+    tv.store(sV, tid);
     __syncthreads();
-    stage_natural<KT, HD>(sK, K, a.k_st, k0, a.Tk, a.hd, tid);
-    stage_transposed<KT, HD>(sVt, V, a.v_st, k0, a.Tk, a.hd, tid);
+    transpose_tile<HD>(sV, sVt, tid);
+    if (k0 + KT < k_end) {               // next tile's global loads fly during this tile's math
+      tk.load(K, a.k_st, k0 + KT, a.Tk, a.hd, tid);
+      tv.load(V, a.v_st, k0 + KT, a.Tk, a.hd, tid);
+    }
     __syncthreads();
     float16_t s[2];
 #pragma unroll
@@ -171,24 +187,38 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
         s[t] = M32<DT>::run(kf, qf[c], s[t]);
       }
     }
+    // only the tile on the causal diagonal and the ragged last tile need per-element masks
+    const bool masked = (k0 + KT > a.Tk) || (a.causal && k0 + KT - 1 > q0 + shift);
     float mx = m;
+    if (masked) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int kj = k0 + t * 32 + acc_row(r, lane);
-        const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
-        s[t][r] = ok ? s[t][r] * sc : -INFINITY;
-        mx = fmaxf(mx, s[t][r]);
-      }
+        for (int r = 0; r < 16; ++r) {
+          const int kj = k0 + t * 32 + acc_row(r, lane);
+          const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
+          s[t][r] = ok ? s[t][r] * sc : -INFINITY;
+          mx = fmaxf(mx, s[t][r]);
+        }
+    } else {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          s[t][r] *= sc;
+          mx = fmaxf(mx, s[t][r]);
+        }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = (mx == -INFINITY) ? 1.f : exp2f(m - mx);
+    const bool dead = (mx == -INFINITY);
+    const float mref = dead ? 0.f : mx;
+    const float alpha = dead ? 1.f : exp2f(m - mx);
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = (mx == -INFINITY) ? 0.f : exp2f(s[t][r] - mx);
+        const float p = exp2f(s[t][r] - mref);   // masked entries: exp2(-inf) = 0
         s[t][r] = p;
         psum += p;
       }
@@ -280,7 +310,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
     dof[c] = load_row8(DO, a.do_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
   }
   const bool qok = qi < a.Tq;
-  const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : 0.f;
+  // a query row past the end keeps lse = +inf so that its probabilities are exactly zero
+  const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
   const float dlt = qok ? a.delta[(int64_t)bh * a.Tq + qi] : 0.f;
 
   float16_t acc[NO];
@@ -294,12 +325,21 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
     const int last_q = min(blockIdx.x * 128 + 127, a.Tq - 1);
     k_end = min(a.Tk, last_q + shift + 1);
   }
+  Tile<HD> tk, tv;
+  tk.load(K, a.k_st, 0, a.Tk, a.hd, tid);
+  tv.load(V, a.v_st, 0, a.Tk, a.hd, tid);
   for (int k0 = 0; k0 < k_end; k0 += KT) {
     __syncthreads();
-    stage_natural<KT, HD>(sK, K, a.k_st, k0, a.Tk, a.hd, tid);
-    stage_natural<KT, HD>(sV, V, a.v_st, k0, a.Tk, a.hd, tid);
-    stage_transposed<KT, HD>(sKt, K, a.k_st, k0, a.Tk, a.hd, tid);
+    tk.store(sK, tid);
+    tv.store(sV, tid);
     __syncthreads();
+    transpose_tile<HD>(sK, sKt, tid);
+    if (k0 + KT < k_end) {
+      tk.load(K, a.k_st, k0 + KT, a.Tk, a.hd, tid);
+      tv.load(V, a.v_st, k0 + KT, a.Tk, a.hd, tid);
+    }
+    __syncthreads();
+    const bool masked = (k0 + KT > a.Tk) || (a.causal && k0 + KT - 1 > q0 + shift);
     float16_t s[2], dp[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -311,12 +351,17 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
         s[t] = M32<DT>::run(*(const uint4*)(sK + off), qf[c], s[t]);
         dp[t] = M32<DT>::run(*(const uint4*)(sV + off), dof[c], dp[t]);
       }
+      if (masked) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int kj = k0 + t * 32 + acc_row(r, lane);
-        const bool ok = qok && kj < a.Tk && (!a.causal || kj <= qi + shift);
-        const float p = ok ? exp2f(s[t][r] * sc - lse2) : 0.f;
-        s[t][r] = p * (dp[t][r] - dlt) * a.scale;   // dS^T
+        for (int r = 0; r < 16; ++r) {
+          const int kj = k0 + t * 32 + acc_row(r, lane);
+          const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
+          const float p = ok ? exp2f(s[t][r] * sc - lse2) : 0.f;
+          s[t][r] = p * (dp[t][r] - dlt) * a.scale;   // dS^T
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[t][r] = exp2f(s[t][r] * sc - lse2) * (dp[t][r] - dlt) * a.scale;
       }
     }
 #pragma unroll
@@ -357,7 +402,8 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
   __shared__ float sLse[KT], sDelta[KT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int kj = blockIdx.x * 128 + wave * 32 + (lane & 31);   // this lane's key row
+  const int kw0 = blockIdx.x * 128 + wave * 32;                // this wavefront's first key row
+  const int kj = kw0 + (lane & 31);                            // this lane's key row
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
@@ -383,18 +429,34 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
     q_begin = max(0, blockIdx.x * 128 - shift);
     q_begin = q_begin / KT * KT;
   }
-  for (int q0 = q_begin; q0 < a.Tq; q0 += KT) {
-    __syncthreads();
-    stage_natural<KT, HD>(sQ, Q, a.q_st, q0, a.Tq, a.hd, tid);
-    stage_natural<KT, HD>(sDO, DO, a.do_st, q0, a.Tq, a.hd, tid);
-    stage_transposed<KT, HD>(sQt, Q, a.q_st, q0, a.Tq, a.hd, tid);
-    stage_transposed<KT, HD>(sDOt, DO, a.do_st, q0, a.Tq, a.hd, tid);
+  Tile<HD> tq, tdo;
+  float r_lse = 0.f, r_dlt = 0.f;
+  auto prefetch = [&](int q0) {
+    tq.load(Q, a.q_st, q0, a.Tq, a.hd, tid);
+    tdo.load(DO, a.do_st, q0, a.Tq, a.hd, tid);
     if (tid < KT) {
       const int qi = q0 + tid;
-      sLse[tid] = qi < a.Tq ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : 0.f;
-      sDelta[tid] = qi < a.Tq ? a.delta[(int64_t)bh * a.Tq + qi] : 0.f;
+      // rows past the end: Q and dO rows are zero, lse = +inf makes their P exactly zero
+      r_lse = qi < a.Tq ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
+      r_dlt = qi < a.Tq ? a.delta[(int64_t)bh * a.Tq + qi] : 0.f;
+    }
+  };
+  if (q_begin < a.Tq) prefetch(q_begin);
+  for (int q0 = q_begin; q0 < a.Tq; q0 += KT) {
+    __syncthreads();
+    tq.store(sQ, tid);
+    tdo.store(sDO, tid);
+    if (tid < KT) {
+      sLse[tid] = r_lse;
+      sDelta[tid] = r_dlt;
     }
     __syncthreads();
+    transpose_tile<HD>(sQ, sQt, tid);
+    transpose_tile<HD>(sDO, sDOt, tid);
+    if (q0 + KT < a.Tq) prefetch(q0 + KT);
+    __syncthreads();
+    // causal: the tile needs element masks only where it crosses the diagonal
+    const bool masked = a.causal && (kw0 + 31 > q0 + shift);
     float16_t s[2], dp[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
@@ -408,9 +470,9 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int ql = t * 32 + acc_row(r, lane), qi = q0 + ql;
-        const bool ok = kok && qi < a.Tq && (!a.causal || kj <= qi + shift);
-        const float p = ok ? exp2f(s[t][r] * sc - sLse[ql]) : 0.f;
+        const int ql = t * 32 + acc_row(r, lane);
+        float p = exp2f(s[t][r] * sc - sLse[ql]);
+        if (masked && kj > q0 + ql + shift) p = 0.f;
         s[t][r] = p;                                         // P
         dp[t][r] = p * (dp[t][r] - sDelta[ql]) * a.scale;    // dS
       }

@@ -83,6 +83,20 @@ __device__ __forceinline__ uint16_t pf_f32_to_f16_bits(float f) {
   return c.u;
 }
 
+// two fp32 -> one packed pair of 16-bit values (low half = first argument), round to nearest
+// even: single v_cvt_pk_{bf16,f16}_f32 instructions on gfx950
+typedef __bf16 pf_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 pf_f16x2_t __attribute__((ext_vector_type(2)));
+typedef float pf_f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pf_pack2_bf16(float lo, float hi) {
+  const pf_f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_bf16x2_t));
+}
+__device__ __forceinline__ uint32_t pf_pack2_f16(float lo, float hi) {
+  const pf_f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, pf_f16x2_t));
+}
+
 // Element codecs: T is float, pf_half tag or pf_bf16 tag. Storage of the 16-bit
 // kinds is always handled as uint16_t so that no implicit arithmetic sneaks in.
 template <int DT> struct Codec;
@@ -151,8 +165,7 @@ template <> struct Vec8<PF_F16> {
   static __device__ __forceinline__ void store(void* p, int64_t i, const float (&v)[8]) {
     uint32_t w[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      w[k] = (uint32_t)pf_f32_to_f16_bits(v[2 * k]) | ((uint32_t)pf_f32_to_f16_bits(v[2 * k + 1]) << 16);
+    for (int k = 0; k < 4; ++k) w[k] = pf_pack2_f16(v[2 * k], v[2 * k + 1]);
     *(uint4*)((uint16_t*)p + i) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 };
@@ -169,8 +182,7 @@ template <> struct Vec8<PF_BF16> {
   static __device__ __forceinline__ void store(void* p, int64_t i, const float (&v)[8]) {
     uint32_t w[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k)
-      w[k] = (uint32_t)pf_f32_to_bf16_bits(v[2 * k]) | ((uint32_t)pf_f32_to_bf16_bits(v[2 * k + 1]) << 16);
+    for (int k = 0; k < 4; ++k) w[k] = pf_pack2_bf16(v[2 * k], v[2 * k + 1]);
     *(uint4*)((uint16_t*)p + i) = make_uint4(w[0], w[1], w[2], w[3]);
   }
 };
