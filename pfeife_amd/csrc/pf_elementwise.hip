@@ -223,6 +223,36 @@ __global__ __launch_bounds__(256) void transpose_cast_kernel(const void* src, in
   }
 }
 
+// 16-bit -> 16-bit transpose without LDS: a wavefront owns a 64x64 tile, lane (lr, lc) the
+// 8x8 block (lr, lc); eight 16-byte loads, an in-register 8x8 transpose, eight 16-byte stores.
+// Eight lanes cover 128 contiguous bytes on both the read and the write side.
+__global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* src, int64_t ld_src, uint16_t* dst,
+                                                          int64_t ld_dst, int64_t rows, int64_t cols) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lr = lane >> 3, lc = lane & 7;
+  const int64_t r0 = ((int64_t)blockIdx.y * 4 + wave) * 64 + lr * 8, c0 = (int64_t)blockIdx.x * 64 + lc * 8;
+  if (r0 >= rows || c0 >= cols) return;
+  uint32_t in[8][4];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    uint4 x = make_uint4(0, 0, 0, 0);
+    if (r0 + r < rows) x = *(const uint4*)(src + (r0 + r) * ld_src + c0);
+    in[r][0] = x.x; in[r][1] = x.y; in[r][2] = x.z; in[r][3] = x.w;
+  }
+#pragma unroll
+  for (int J = 0; J < 4; ++J) {
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int I = 0; I < 4; ++I) {
+      const uint32_t a = in[2 * I][J], c = in[2 * I + 1][J];
+      lo[I] = (a & 0xffffu) | (c << 16);
+      hi[I] = (a >> 16) | (c & 0xffff0000u);
+    }
+    if (c0 + 2 * J < cols) *(uint4*)(dst + (c0 + 2 * J) * ld_dst + r0) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    if (c0 + 2 * J + 1 < cols) *(uint4*)(dst + (c0 + 2 * J + 1) * ld_dst + r0) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+  }
+}
+
 // ---- rotary embedding --------------------------------------------------------
 // one thread per (b, t, h, i) pair index i < D/2
 __global__ __launch_bounds__(EW_BLOCK) void rope_kernel(const void* x, void* y, int dt, const float* cos_t,
@@ -332,6 +362,17 @@ extern "C" int pf_transpose_cast(const void* src, int src_dtype, int64_t ld_src,
              "pf_transpose_cast: bad arguments");
   if (rows == 0 || cols == 0) return PF_OK;
   PF_REQUIRE(src && dst && ld_src >= cols && ld_dst >= rows, "pf_transpose_cast: bad operands");
+  // same 16-bit dtype, everything 16-byte granular (the destination rows are `rows` long and
+  // written 8 at a time: ld_dst >= ceil8(rows)): register-transpose path
+  if (src_dtype == dst_dtype && src_dtype != PF_F32 && cols % 8 == 0 && ld_src % 8 == 0 && ld_dst % 8 == 0 &&
+      ld_dst >= (rows + 7) / 8 * 8 && pf_aligned(src, 16) && pf_aligned(dst, 16)) {
+    const dim3 g16((unsigned)((cols + 63) / 64), (unsigned)((rows + 255) / 256));
+    PF_REQUIRE(g16.y <= 65535, "pf_transpose_cast: too many rows");
+    hipLaunchKernelGGL(transpose16_kernel, g16, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, ld_src,
+                       (uint16_t*)dst, ld_dst, rows, cols);
+    PF_CHECK_LAUNCH("pf_transpose_cast");
+    return PF_OK;
+  }
   const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)((rows + 63) / 64));
   PF_REQUIRE(grid.y <= 65535, "pf_transpose_cast: too many rows");
   hipLaunchKernelGGL(transpose_cast_kernel, grid, dim3(256), 0, (hipStream_t)stream, src, src_dtype, ld_src, dst,

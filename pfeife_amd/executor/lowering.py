@@ -196,9 +196,21 @@ class BwdCtx:
         self._seq = 0
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
+        self._transposed = {}  # (data_ptr, rows, cols, ld) -> transposed copy made earlier in this job
 
     def emit(self, launch):
         self.out.append(launch)
+
+    def transposed(self, t, rows, cols, ld):
+        """[cols, rows] copy of the 16-bit matrix t (made once per job and matrix: several products
+        that reduce over the same token rows share it)."""
+        key = (t.data_ptr(), rows, cols, ld)
+        tt = self._transposed.get(key)
+        if tt is None:
+            tt = self.temp((cols, rows), t.dtype)
+            self.emit(self.k.transpose_cast(t, ld, tt, rows, rows, cols))
+            self._transposed[key] = tt
+        return tt
 
     def colsum_into(self, x, rows, cols, ld, acc):
         """acc[c] += sum_r x[r, c] (bias gradient), reduction finished at the end of the job."""
@@ -614,8 +626,16 @@ def lower_linear(L, node):
             dy = B.matrix_in(g, cd)
         _, _, ld_dy = as_matrix(dy)
         if w.req_grad and w.param is not None:
-            B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
-                            b_trans=1, beta=1))
+            if L.mixed and M % 8 == 0 and M >= 1024:
+                # dW = dY^T X reduces over the token rows: with both operands copied transposed
+                # (cheap, HBM-bound) it runs on the row-row MFMA path, ~2x the rate of the
+                # transposing loaders
+                dy_t = B.transposed(dy, M, N, ld_dy)
+                x_t = B.transposed(xm, M, K, lda)
+                B.emit(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1))
+            else:
+                B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
+                                b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:

@@ -508,3 +508,14 @@ def test_groupnorm_and_channel_bias(hip, oracle, xdt, ydt):
              n=B * HW * C, bias_len=C, rows_per_bias=HW)
     close(r["y"], 1e-6, 1e-6)
     torch.testing.assert_close(r["y"][1], (x.float().view(B, HW, C) + bias.float()[:, None, :]).view(B * HW, C))
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_transpose_16bit_register_path(hip, oracle, dtype):
+    for rows, cols, lds, ldd in [(3152, 4096, 4096, 3152), (1000, 264, 272, 1000), (8, 8, 8, 8), (77, 64, 64, 80)]:
+        src = rnd((rows, lds), dtype, 1)
+        dst = torch.zeros(cols, ldd, dtype=dtype)
+        r = both(hip, oracle, "transpose_cast", dict(src=src, dst=dst), ["dst"], ld_src=lds, ld_dst=ldd, rows=rows,
+                 cols=cols)
+        assert torch.equal(r["dst"][0][:, :rows], src[:, :cols].t())
+        assert torch.equal(r["dst"][1][:, :rows], src[:, :cols].t())

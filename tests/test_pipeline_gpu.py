@@ -317,3 +317,16 @@ def test_unet_stage_sdxl_style(mixed):
     for a, b in zip(losses, want):
         assert abs(float(a) - float(b)) <= ltol * abs(float(b)), (float(a), float(b))
     _check_grads(model, ref, mixed)
+
+
+@pytest.mark.parametrize("mixed", ["fp16", "bf16"])
+def test_many_token_rows_take_the_transposed_weight_gradient_path(mixed):
+    """With >= 1024 token rows per micro-batch the weight gradients are computed from transposed
+    copies of dY and X (row-row MFMA path); same parity bar as every other configuration."""
+    from pfeife_amd.bench_models.vit import ViTConfig
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=128, depth=2, heads=2, mlp_dim=256, num_classes=16)
+    m, r, l, rl, runner = _run_vit(cfg, 512, 2, "blocks.1", mixed)   # 256 images x 5 tokens = 1280 rows
+    _check(m, r, l, rl, mixed)
+    kernels = [getattr(x, "kernel", "") for p in runner.worker.mbs[0].stage_programs.values() for x in p.bwd]
+    assert "pf_transpose_cast" in kernels
