@@ -311,6 +311,23 @@ int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* 
             int64_t T, int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh, int64_t y_sb, int64_t y_st,
             int64_t y_sh, int inverse, void* stream);
 
+/* ---- optimizer step ----------------------------------------------------------------
+ * Multi-tensor Adam (adamw = 0: torch.optim.Adam, L2 weight decay added to the gradient;
+ * adamw = 1: torch.optim.AdamW, decoupled decay) on fp32 parameters with fp32 gradients
+ * and moments, `step` = 1-based step count, one launch per parameter group.  Tensors must be
+ * 16-byte aligned; `items_dev` lives in DEVICE memory.  Replaces the foreach kernels of
+ * `scaler.step(self.optimizer)` in ProcessWorker.optimizer_step (pfeife/mp/worker.py:1432-1436)
+ * for the optimizers `get_optimizer_cls` maps "adam" / "adamw" to (pfeife/option.py:9-29). */
+typedef struct pf_adam_item {
+  float* param;
+  const float* grad;
+  float* exp_avg;
+  float* exp_avg_sq;
+  int64_t n;
+} pf_adam_item;
+int pf_adam_step(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1, double beta2,
+                 double eps, double weight_decay, int64_t step, int adamw, void* stream);
+
 /* ---- gradient accumulation --------------------------------------------------
  * acc[i] += g[i] for i < n, acc fp32, g of dtype g_dtype: autograd's
  * AccumulateGrad `param.grad.add_(new_grad)` executed once per parameter per

@@ -2,6 +2,8 @@
 // fills, strided copies, rotary embedding and the fp32 gradient accumulation.
 // All of them move 16 bytes (8 x 16-bit) or 32 bytes (8 x fp32) per lane per
 // step in a grid-stride loop sized to keep every CU busy.
+#include <math.h>
+
 #include "pf_common.h"
 
 namespace {
@@ -253,6 +255,51 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* src, i
   }
 }
 
+// ---- multi-tensor Adam / AdamW ---------------------------------------------------------
+// One launch updates every parameter of a param group.  Items live in device memory;
+// block y walks item y in a grid-stride loop.  The arithmetic follows torch.optim.Adam's
+// single-tensor formulation operation by operation (lerp for the first moment, mul + addcmul
+// for the second, sqrt / bias_correction2_sqrt + eps, addcdiv).
+__global__ __launch_bounds__(256) void adam_kernel(const pf_adam_item* items, float lr, float omb1, float beta2,
+                                                   float omb2, float eps, float weight_decay, float step_size,
+                                                   float bias_c2_sqrt, int adamw) {
+  // omb1 = 1 - beta1, omb2 = 1 - beta2, step_size = lr / (1 - beta1^t): formed in double on the
+  // host like torch does, then rounded once
+  const pf_adam_item it = items[blockIdx.y];
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x * 4;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < it.n; i += gsz) {
+    if (i + 4 <= it.n) {
+      float4 p = *(float4*)(it.param + i), g = *(const float4*)(it.grad + i);
+      float4 m = *(float4*)(it.exp_avg + i), v = *(float4*)(it.exp_avg_sq + i);
+      float pp[4] = {p.x, p.y, p.z, p.w}, gg[4] = {g.x, g.y, g.z, g.w};
+      float mm[4] = {m.x, m.y, m.z, m.w}, vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (adamw) pp[k] *= 1.f - lr * weight_decay;
+        else if (weight_decay != 0.f) gg[k] += weight_decay * pp[k];
+        mm[k] = mm[k] + omb1 * (gg[k] - mm[k]);
+        vv[k] = vv[k] * beta2 + omb2 * gg[k] * gg[k];
+        const float denom = sqrtf(vv[k]) / bias_c2_sqrt + eps;
+        pp[k] = pp[k] - step_size * (mm[k] / denom);
+      }
+      *(float4*)(it.param + i) = make_float4(pp[0], pp[1], pp[2], pp[3]);
+      *(float4*)(it.exp_avg + i) = make_float4(mm[0], mm[1], mm[2], mm[3]);
+      *(float4*)(it.exp_avg_sq + i) = make_float4(vv[0], vv[1], vv[2], vv[3]);
+    } else {
+      for (int64_t j = i; j < it.n; ++j) {
+        float pv = it.param[j], gv = it.grad[j], mv = it.exp_avg[j], vv = it.exp_avg_sq[j];
+        if (adamw) pv *= 1.f - lr * weight_decay;
+        else if (weight_decay != 0.f) gv += weight_decay * pv;
+        mv = mv + omb1 * (gv - mv);
+        vv = vv * beta2 + omb2 * gv * gv;
+        const float denom = sqrtf(vv) / bias_c2_sqrt + eps;
+        pv = pv - step_size * (mv / denom);
+        it.param[j] = pv; it.exp_avg[j] = mv; it.exp_avg_sq[j] = vv;
+      }
+    }
+  }
+}
+
 // ---- rotary embedding --------------------------------------------------------
 // one thread per (b, t, h, i) pair index i < D/2
 __global__ __launch_bounds__(EW_BLOCK) void rope_kernel(const void* x, void* y, int dt, const float* cos_t,
@@ -455,5 +502,22 @@ extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, co
   hipLaunchKernelGGL(rope_kernel, ew_grid(total), dim3(EW_BLOCK), 0, (hipStream_t)stream, x, y, dtype, cos_t, sin_t,
                      tab_ld, B, T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
   PF_CHECK_LAUNCH("pf_rope");
+  return PF_OK;
+}
+
+extern "C" int pf_adam_step(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1,
+                            double beta2, double eps, double weight_decay, int64_t step, int adamw, void* stream) {
+  PF_REQUIRE(n_items >= 0 && max_n >= 0 && step >= 1, "pf_adam_step: bad arguments");
+  if (n_items == 0 || max_n == 0) return PF_OK;
+  PF_REQUIRE(items_dev != nullptr && n_items <= 65535, "pf_adam_step: bad item list");
+  const double bc1 = 1.0 - pow(beta1, (double)step);
+  const double bc2 = 1.0 - pow(beta2, (double)step);
+  int64_t bx = (max_n / 4 + 255) / 256;
+  if (bx > 64) bx = 64;   // enough blocks per tensor; small tensors leave most of them idle at once
+  if (bx < 1) bx = 1;
+  hipLaunchKernelGGL(adam_kernel, dim3((unsigned)bx, (unsigned)n_items), dim3(256), 0, (hipStream_t)stream, items_dev,
+                     (float)lr, (float)(1.0 - beta1), (float)beta2, (float)(1.0 - beta2), (float)eps, (float)weight_decay,
+                     (float)(lr / bc1), (float)sqrt(bc2), adamw);
+  PF_CHECK_LAUNCH("pf_adam_step");
   return PF_OK;
 }

@@ -110,6 +110,8 @@ _SIGNATURES = {
     "pf_cast": [_P, _I, _P, _I, _L, _P],
     "pf_transpose_cast": [_P, _I, _L, _P, _I, _L, _L, _L, _P],
     "pf_fill": [_P, _I, _F, _L, _P],
+    "pf_adam_step": [_P, _I, _L, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, _L,
+                     _I, _P],
     "pf_copy_strided": [_P, _I, POINTER(c_int64), _P, _I, POINTER(c_int64), POINTER(c_int64), _I, _I, _P],
     "pf_rope": [_P, _P, _I, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P],
     "pf_grad_accumulate_f32": [_P, _P, _I, _L, _P],
@@ -412,6 +414,22 @@ class HipKernels:
     def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
         args = (_ptr(src), _dt(src), ld_src, _ptr(dst), _dt(dst), ld_dst, rows, cols)
         return self._prep("pf_transpose_cast", args, (src, dst))
+
+    def adam_table(self, params, grads, exp_avgs, exp_avg_sqs):
+        """Device table of pf_adam_item for one param group (built once, pointers are static)."""
+        rows = [[p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), p.numel()]
+                for p, g, m, v in zip(params, grads, exp_avgs, exp_avg_sqs)]
+        for r in rows:
+            if any(x % 16 for x in r[:4]):
+                raise RuntimeError("adam: tensors must be 16-byte aligned")
+        table = torch.tensor(rows, dtype=torch.int64).to(params[0].device)
+        return table, len(rows), max(r[4] for r in rows)
+
+    def adam_step(self, table, n_items, max_n, lr, beta1, beta2, eps, weight_decay, step, adamw, stream):
+        rc = self.lib.pf_adam_step(table.data_ptr(), n_items, max_n, lr, beta1, beta2, eps, weight_decay, step,
+                                   int(adamw), stream)
+        if rc != 0:
+            raise RuntimeError("pf_adam_step failed: %s" % self.lib.pf_last_error().decode())
 
     def fill(self, dst, value, n):
         return self._prep("pf_fill", (_ptr(dst), _dt(dst), float(value), n), (dst,))

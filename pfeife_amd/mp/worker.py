@@ -286,8 +286,59 @@ class StageWorker:
                 self.optimizer = cls(params, **self.option.optimizer_kwargs)
 
     def optimizer_step(self):
-        if self.optimizer is not None:
-            self.optimizer.step()
+        opt = self.optimizer
+        if opt is None:
+            return
+        if self._fused_adam_applicable(opt):
+            self._fused_adam_step(opt)
+        else:
+            opt.step()
+
+    def _fused_adam_applicable(self, opt):
+        """torch.optim.Adam / AdamW in their plain configuration on fp32 GPU parameters run as one
+        HIP launch per param group; anything else keeps PyTorch's own step()."""
+        if not hasattr(self.kernels, "adam_step") or type(opt) not in (torch.optim.Adam, torch.optim.AdamW):
+            return False
+        for g in opt.param_groups:
+            if g.get("amsgrad") or g.get("maximize") or g.get("capturable") or g.get("differentiable"):
+                return False
+            if torch.is_tensor(g["lr"]) or g.get("decoupled_weight_decay", False) and type(opt) is torch.optim.Adam:
+                return False
+            for p in g["params"]:
+                if p.grad is None:
+                    continue
+                if (p.dtype != torch.float32 or p.grad.dtype != torch.float32 or not p.is_cuda
+                        or not p.is_contiguous() or not p.grad.is_contiguous() or p.grad.is_sparse):
+                    return False
+        return True
+
+    def _fused_adam_step(self, opt):
+        cache = self.__dict__.setdefault("_adam_tables", {})
+        s = self.stream()
+        for gi, g in enumerate(opt.param_groups):
+            params = [p for p in g["params"] if p.grad is not None]
+            if not params:
+                continue
+            for p in params:   # state exactly as torch.optim.Adam initialises it
+                st = opt.state[p]
+                if len(st) == 0:
+                    st["step"] = torch.tensor(0.0, dtype=torch.float32)
+                    st["exp_avg"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+                    st["exp_avg_sq"] = torch.zeros_like(p, memory_format=torch.preserve_format)
+            sig = tuple((p.data_ptr(), p.grad.data_ptr(), opt.state[p]["exp_avg"].data_ptr()) for p in params)
+            ent = cache.get(gi)
+            if ent is None or ent[0] != sig:
+                table = self.kernels.adam_table([p.data for p in params], [p.grad for p in params],
+                                                [opt.state[p]["exp_avg"] for p in params],
+                                                [opt.state[p]["exp_avg_sq"] for p in params])
+                ent = cache[gi] = (sig, table)
+            step = int(opt.state[params[0]]["step"].item()) + 1
+            b1, b2 = g["betas"]
+            table, n_items, max_n = ent[1]
+            self.kernels.adam_step(table, n_items, max_n, float(g["lr"]), float(b1), float(b2), float(g["eps"]),
+                                   float(g["weight_decay"]), step, type(opt) is torch.optim.AdamW, s)
+            for p in params:
+                opt.state[p]["step"] += 1
 
     # -- reporting -----------------------------------------------------------------------
     def memory_report(self):
