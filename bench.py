@@ -254,6 +254,9 @@ def main():
     ap.add_argument("--workload", default="vit_l16_fp16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="issue every kernel launch individually instead of replaying captured hipGraphs "
+                         "(use for rocprofv3 --pmc runs: counters are collected per dispatched kernel)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain copy kernel (ew_kernel<Scale>, 256 MiB read + 256 MiB written) three "
                          "times, as the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -269,6 +272,8 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     device = torch.device("cuda", 0)
+    if args.no_graph:
+        os.environ["PFEIFE_NO_GRAPH"] = "1"
     runner, batch, info = build_workload(args.workload, device)
     log("[bench] workload", args.workload, "building stage programs (first step) ...")
     t0 = time.perf_counter()

@@ -379,6 +379,7 @@ class Lowerer:
         self.device = torch.device(device)
         self.cd = compute_dtype or torch.float32
         self.mixed = self.cd != torch.float32
+        self.dw_transpose_min_elems = 4 * 1024 * 1024
         self.params = params or ParamStore(kernels, self.device)
         self.pool = pool or BufferPool(self.device)
         self._ws = None
@@ -626,10 +627,12 @@ def lower_linear(L, node):
             dy = B.matrix_in(g, cd)
         _, _, ld_dy = as_matrix(dy)
         if w.req_grad and w.param is not None:
-            if L.mixed and M % 8 == 0 and M >= 1024:
+            if L.mixed and M % 8 == 0 and M >= 1024 and N * K >= L.dw_transpose_min_elems:
                 # dW = dY^T X reduces over the token rows: with both operands copied transposed
-                # (cheap, HBM-bound) it runs on the row-row MFMA path, ~2x the rate of the
-                # transposing loaders
+                # (cheap, HBM-bound) it runs on the row-row MFMA path.  Measured: for weight
+                # matrices of >= 4M elements (enough 128x128 tiles for two workgroups per CU) that
+                # path is ~1.8x the rate of the transposing loaders; for smaller ones the two
+                # transposes cost what the faster product saves
                 dy_t = B.transposed(dy, M, N, ld_dy)
                 x_t = B.transposed(xm, M, K, lda)
                 B.emit(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1))
