@@ -379,7 +379,7 @@ class Lowerer:
         self.device = torch.device(device)
         self.cd = compute_dtype or torch.float32
         self.mixed = self.cd != torch.float32
-        self.dw_transpose_min_elems = 4 * 1024 * 1024
+        self.dw_transpose_min_elems = 8 * 1024 * 1024
         self.params = params or ParamStore(kernels, self.device)
         self.pool = pool or BufferPool(self.device)
         self._ws = None
@@ -630,7 +630,7 @@ def lower_linear(L, node):
             if L.mixed and M % 8 == 0 and M >= 1024 and N * K >= L.dw_transpose_min_elems:
                 # dW = dY^T X reduces over the token rows: with both operands copied transposed
                 # (cheap, HBM-bound) it runs on the row-row MFMA path.  Measured: for weight
-                # matrices of >= 4M elements (enough 128x128 tiles for two workgroups per CU) that
+                # matrices of >= 8M elements (enough 128x128 tiles for two workgroups per CU) that
                 # path is ~1.8x the rate of the transposing loaders; for smaller ones the two
                 # transposes cost what the faster product saves
                 dy_t = B.transposed(dy, M, N, ld_dy)
