@@ -108,9 +108,9 @@ def build_workload(name, device):
 # in profiles/vit_l16_fp16_pmc_traffic.md.
 MEASURED_TRAFFIC = {
     "vit_l16_fp16": {
-        "gemm16_kernel<1, 128, 64, 64, 2, 2, false, false>": 9.04e7,
+        "gemm16_kernel<1, 128, 64, 64, 2, 2, false, false>": 9.32e7,
         "gemm16_kernel<1, 128, 128, 64, 2, 2, true, true>": 1.105e8,
-        "gemm16_kernel<1, 128, 128, 64, 2, 2, false, false>": 1.240e8,
+        "gemm16_kernel<1, 128, 128, 64, 2, 2, false, false>": 1.141e8,
         "gemm16_kernel<1, 64, 64, 64, 2, 2, true, true>": 4.56e7,
     },
 }
