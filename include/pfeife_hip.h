@@ -286,6 +286,15 @@ int pf_bias_add(const void* x, int x_dtype, const void* bias, int bias_dtype, vo
 /* dtype conversion / copy of n contiguous elements (autocast's weight casts,
  * done once per optimiser step instead of once per micro-batch). */
 int pf_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, void* stream);
+/* Many casts in one launch (`items_dev` in DEVICE memory; vec != 0 promises 16-byte aligned
+ * src and dst): the once-per-step refresh of all 16-bit parameter shadows. */
+typedef struct pf_cast_item {
+  const void* src;
+  void* dst;
+  int64_t n;
+  int32_t src_dtype, dst_dtype, vec, reserved;
+} pf_cast_item;
+int pf_cast_batch(const pf_cast_item* items_dev, int n_items, int64_t max_n, void* stream);
 /* dst[c*ld_dst + r] = src[r*ld_src + c] with dtype conversion: the transposed 16-bit
  * shadow of a weight matrix, made once per optimiser step, lets the input-gradient
  * product dx = dy W read W with its reduction dimension contiguous. */

@@ -413,6 +413,13 @@ class OracleKernels:
 
         return launch
 
+    def cast_batch(self, pairs):
+        def launch(stream=None):
+            for src, dst in pairs:
+                dst.copy_(src.to(dst.dtype))
+
+        return launch
+
     def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
         def launch(stream=None):
             _rows(dst, cols, rows, ld_dst).copy_(_rows(src, rows, cols, ld_src).t().to(dst.dtype))

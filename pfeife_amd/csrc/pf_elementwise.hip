@@ -255,6 +255,21 @@ __global__ __launch_bounds__(256) void transpose16_kernel(const uint16_t* src, i
   }
 }
 
+// ---- multi-tensor cast: the per-step refresh of every 16-bit weight shadow in one launch ----
+__global__ __launch_bounds__(256) void cast_batch_kernel(const pf_cast_item* items) {
+  const pf_cast_item it = items[blockIdx.y];
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nv = it.vec ? it.n / 8 : 0;
+  for (int64_t i = gtid; i < nv; i += gsz) {
+    float x[8];
+    ld_vec<8>(it.src, i * 8, it.src_dtype, x);
+    st_vec<8>(it.dst, i * 8, it.dst_dtype, x);
+  }
+  for (int64_t i = nv * 8 + gtid; i < it.n; i += gsz)
+    pf_store_from_f32(it.dst, i, it.dst_dtype, pf_load_as_f32(it.src, i, it.src_dtype));
+}
+
 // ---- multi-tensor Adam / AdamW ---------------------------------------------------------
 // One launch updates every parameter of a param group.  Items live in device memory;
 // block y walks item y in a grid-stride loop.  The arithmetic follows torch.optim.Adam's
@@ -519,5 +534,18 @@ extern "C" int pf_adam_step(const pf_adam_item* items_dev, int n_items, int64_t 
                      (float)lr, (float)(1.0 - beta1), (float)beta2, (float)(1.0 - beta2), (float)eps, (float)weight_decay,
                      (float)(lr / bc1), (float)sqrt(bc2), adamw);
   PF_CHECK_LAUNCH("pf_adam_step");
+  return PF_OK;
+}
+
+extern "C" int pf_cast_batch(const pf_cast_item* items_dev, int n_items, int64_t max_n, void* stream) {
+  PF_REQUIRE(n_items >= 0 && max_n >= 0, "pf_cast_batch: bad arguments");
+  if (n_items == 0 || max_n == 0) return PF_OK;
+  PF_REQUIRE(items_dev != nullptr && n_items <= 65535, "pf_cast_batch: bad item list");
+  int64_t bx = (max_n / 8 + 255) / 256;
+  if (bx > 64) bx = 64;
+  if (bx < 1) bx = 1;
+  hipLaunchKernelGGL(cast_batch_kernel, dim3((unsigned)bx, (unsigned)n_items), dim3(256), 0, (hipStream_t)stream,
+                     items_dev);
+  PF_CHECK_LAUNCH("pf_cast_batch");
   return PF_OK;
 }

@@ -48,6 +48,10 @@ class ParamStore:
         self.zero = []         # launches: zero-fill of every gradient accumulator (once per step)
         self.params = []       # parameters that receive gradients, in first-use order
         self._keep = []
+        self.cast_pairs = []   # (fp32 master, 16-bit shadow): refreshed by ONE batched launch per step
+        self._arena = None     # current block of the gradient arena
+        self._arena_used = 0
+        self.arena_block = 64 * 1024 * 1024   # fp32 elements per arena block (256 MiB)
 
     def shadow(self, tensor, dtype):
         if tensor.dtype == dtype:
@@ -59,10 +63,53 @@ class ParamStore:
             src = tensor.detach()
             if not src.is_contiguous():
                 raise Unsupported("non-contiguous parameter %s" % (tuple(tensor.shape),))
-            self.refresh.append(self.kernels.cast(src, sh, src.numel()))
+            if hasattr(self.kernels, "cast_batch"):
+                self.cast_pairs.append((src, sh))
+            else:
+                self.refresh.append(self.kernels.cast(src, sh, src.numel()))
             self._shadow[key] = sh
             self._keep.append(tensor)
         return sh
+
+    def refresh_launches(self):
+        """Launches that bring every shadow up to date with its master (once per step)."""
+        out = list(self.refresh)
+        if self.cast_pairs:
+            out.insert(0, self.kernels.cast_batch(list(self.cast_pairs)))
+        return out
+
+    def _arena_alloc(self, shape, device):
+        """fp32 gradient accumulator carved out of a large block, so that one fill per block
+        zeroes every gradient of the step (optimizer.zero_grad(set_to_none=False))."""
+        n = 1
+        for d in shape:
+            n *= int(d)
+        pad = (n + 63) // 64 * 64   # keep every accumulator 256-byte aligned
+        if n >= self.arena_block // 4:
+            t = torch.zeros(shape, dtype=torch.float32, device=device)
+            self.zero.append(self.kernels.fill(t, 0.0, t.numel()))
+            return t
+        if self._arena is None or self._arena_used + pad > self._arena.numel():
+            self._arena = torch.zeros(self.arena_block, dtype=torch.float32, device=device)
+            self._arena_used = 0
+            self.zero.append(None)          # placeholder: the block's fill is sized when known
+            self._arena_slots = getattr(self, "_arena_slots", []) + [(len(self.zero) - 1, self._arena)]
+        t = self._arena[self._arena_used:self._arena_used + n].view(shape)
+        self._arena_used += pad
+        return t
+
+    def zero_launches(self):
+        """Launches that zero every gradient accumulator (one fill per arena block)."""
+        out = []
+        slots = dict((i, a) for i, a in getattr(self, "_arena_slots", []))
+        for i, launch in enumerate(self.zero):
+            if launch is not None:
+                out.append(launch)
+            else:
+                a = slots[i]
+                used = self._arena_used if a is self._arena else a.numel()
+                out.append(self.kernels.fill(a, 0.0, used))
+        return out
 
     def shadow_t(self, tensor, dtype):
         """Transposed copy [cols, rows] of a 2-d parameter in `dtype`, refreshed once per step."""
@@ -97,10 +144,12 @@ class ParamStore:
         g = self._grads.get(id(param))
         if g is None:
             if param.grad is None or param.grad.dtype != torch.float32 or not param.grad.is_contiguous():
-                param.grad = torch.zeros(param.shape, dtype=torch.float32, device=param.device)
-            g = param.grad
+                param.grad = self._arena_alloc(param.shape, param.device)
+                g = param.grad
+            else:
+                g = param.grad
+                self.zero.append(self.kernels.fill(g, 0.0, g.numel()))
             self._grads[id(param)] = g
-            self.zero.append(self.kernels.fill(g, 0.0, g.numel()))
             self.params.append(param)
         elif param.grad is not g:
             # user code replaced .grad (e.g. zero_grad(set_to_none=True)); programs hold raw pointers

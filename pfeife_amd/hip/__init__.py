@@ -108,6 +108,7 @@ _SIGNATURES = {
     "pf_groupnorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _L, _I, _F, _P],
     "pf_groupnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P],
     "pf_cast": [_P, _I, _P, _I, _L, _P],
+    "pf_cast_batch": [_P, _I, _L, _P],
     "pf_transpose_cast": [_P, _I, _L, _P, _I, _L, _L, _L, _P],
     "pf_fill": [_P, _I, _F, _L, _P],
     "pf_adam_step": [_P, _I, _L, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, _L,
@@ -410,6 +411,17 @@ class HipKernels:
 
     def cast(self, src, dst, n):
         return self._prep("pf_cast", (_ptr(src), _dt(src), _ptr(dst), _dt(dst), n), (src, dst))
+
+    def cast_batch(self, pairs):
+        """One launch casting every (src, dst) pair of contiguous tensors."""
+        rows = []
+        for src, dst in pairs:
+            vec = 1 if (src.data_ptr() % 16 == 0 and dst.data_ptr() % 16 == 0) else 0
+            rows.append([src.data_ptr(), dst.data_ptr(), src.numel(),
+                         dtype_code(src.dtype) | (dtype_code(dst.dtype) << 32), vec])
+        table = torch.tensor(rows, dtype=torch.int64).to(pairs[0][1].device)
+        args = (table.data_ptr(), len(rows), max(r[2] for r in rows))
+        return self._prep("pf_cast_batch", args, (table, pairs))
 
     def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
         args = (_ptr(src), _dt(src), ld_src, _ptr(dst), _dt(dst), ld_dst, rows, cols)

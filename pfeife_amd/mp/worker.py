@@ -211,7 +211,7 @@ class StageWorker:
                     prog.fwd_graph = self.kernels.capture(prog.fwd, s)
                 if prog.bwd_graph is None and prog.bwd:
                     prog.bwd_graph = self.kernels.capture(prog.bwd, s)
-        pre = list(self.params.zero) + list(self.params.refresh)
+        pre = self.params.zero_launches() + self.params.refresh_launches()
         self.begin_graph = self.kernels.capture(pre, s) if pre else None
         self._begin_len = (len(self.params.zero), len(self.params.refresh))
         self.graphs_ready = True
@@ -237,9 +237,9 @@ class StageWorker:
         if self.graphs_ready and self.begin_graph is not None:
             self.begin_graph(s)
         else:
-            for launch in self.params.zero:      # optimizer.zero_grad(set_to_none=False)
+            for launch in self.params.zero_launches():      # optimizer.zero_grad(set_to_none=False)
                 launch(s)
-            for launch in self.params.refresh:   # one master -> 16-bit cast per step, not per micro-batch
+            for launch in self.params.refresh_launches():   # one master -> 16-bit cast per step
                 launch(s)
         for slot in self.mbs.values():
             slot.grad_seen.clear()
