@@ -1,0 +1,69 @@
+"""The public API surface user scripts rely on (SURVEY boundary table): names, argparse
+flags, option parsing, import paths of the reference package."""
+import argparse
+
+import pytest
+import torch
+
+
+def test_reference_import_paths_resolve_to_this_build():
+    import pfeife
+    from pfeife import PipeOption
+    from pfeife.batch import split_args_kwargs
+    from pfeife.loss import CrossEntropyLoss, HFCrossEntropyLoss, MaskedLMOutputLoss, NormalizeLoss, RescaleLoss, SumLoss
+    from pfeife.mp import (PartialModule, PartialRunner, check_initialized, get_device, get_state,
+                           initialize_pfeife, partial_compiler)
+    from pfeife.mp.partial.module import PartialRunner as PR2
+    import pfeife_amd
+
+    assert PipeOption is pfeife_amd.PipeOption and PartialRunner is PR2
+    assert callable(split_args_kwargs) and callable(partial_compiler) and callable(initialize_pfeife)
+
+
+def test_option_from_args_matches_reference_flags():
+    from pfeife_amd.option import PipeOption
+
+    parser = PipeOption.add_arguments(argparse.ArgumentParser())
+    args = parser.parse_args(["--device_cnt", "2", "--batch_size", "16", "--batch_cnt", "4", "--mixed_precision", "fp16",
+                              "--split_points", "10, 20,blocks.12", "--loop_cnt", "2", "--device_map", "0:2",
+                              "--optimizer_type", "adamw", "--verbose"])
+    opt = PipeOption.from_args(args)
+    assert opt.device_cnt == 2 and opt.batch_size == 16 and opt.batch_cnt == 4 and opt.loop_cnt == 2
+    assert opt.mixed_precision == torch.float16
+    assert opt.split_points == [10, 20, "blocks.12"]
+    assert opt.device_map == ["cuda:0", "cuda:1"]
+    assert opt.optimizer_type == "adamw" and opt.optimizer_kwargs == {"lr": 1e-3}
+    assert opt.scheduler == "single_comm" and opt.partitioner == "beam_single"
+    d = PipeOption()
+    assert d.device_cnt == 2 and d.batch_cnt == 2 and d.batch_size == 4 and d.mixed_precision is None
+    assert d.optimizer_type == "adam" and d.optimizer_kwargs == {"lr": 1e-5}
+    assert PipeOption(mixed_precision="bf16").mixed_precision == torch.bfloat16
+    a2 = parser.parse_args(["--old_ver", "--device_map", "1,3"])
+    o2 = PipeOption.from_args(a2)
+    assert o2.no_side_effect and o2.no_io_cache and o2.single_comm_thread and o2.device_map == ["cuda:1", "cuda:3"]
+
+
+def test_state_requires_initialisation_and_single_process():
+    from pfeife_amd.mp import net_states
+
+    net_states._reset_state_for_tests()
+    with pytest.raises(RuntimeError, match="not initialized"):
+        net_states.get_state()
+    st = net_states.initialize_pfeife(device="cpu")
+    assert st.world_size == 1 and st.rank == 0 and st.pp_size == 1 and st.dp_size == 1
+    assert st.is_main_rank and st.is_main_process and net_states.get_device() == torch.device("cpu")
+    assert net_states.initialize_pfeife(device="cpu") is st
+
+
+def test_loss_wrappers_keep_reference_signatures():
+    import inspect
+
+    from pfeife_amd import loss
+
+    for name in ("LossWrapper", "SumLoss", "MaskedLMOutputLoss", "RescaleLoss", "NormalizeLoss", "CrossEntropyLoss",
+                 "HFCrossEntropyLoss"):
+        cls = getattr(loss, name)
+        assert list(inspect.signature(cls.forward).parameters)[:4] == ["self", "input", "target", "model"]
+    assert loss.CrossEntropyLoss().num_labels == 10
+    with pytest.raises(RuntimeError, match="GPU tensors"):
+        loss.CrossEntropyLoss(4)(torch.zeros(2, 4), torch.zeros(2, dtype=torch.long))
