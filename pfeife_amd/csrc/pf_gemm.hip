@@ -386,13 +386,14 @@ __global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)
       SB::store(rb1, buf1 + BM * LD, k1, K, tid, B_FIRST);
     }
     __syncthreads();
-    if (kt + 1 >= nk) break;
-    // odd phase: tile kt+1 is in buf1, tile kt+2 is landing in set 0, set 1 is free
+    // odd phase: tile kt+1 is in buf1, tile kt+2 is landing in set 0, set 1 is free.  (No early
+    // exit between the phases: a single loop exit keeps the accumulators' live ranges simple,
+    // which saves ~50 registers per lane.)
     if (kt + 3 < nk) {
       SA::load(ra1, rs_a, offa, (uint32_t)(kt + 3) * step_a, tid, A_FIRST);
       SB::load(rb1, rs_b, offb, (uint32_t)(kt + 3) * step_b, tid, B_FIRST);
     }
-    compute(buf1);
+    if (kt + 1 < nk) compute(buf1);
     if (kt + 2 < nk) {
       const int64_t k2 = (int64_t)(kt + 2) * BK;
       SA::store(ra0, buf0, k2, K, tid, A_FIRST);
