@@ -80,11 +80,13 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
 #pragma unroll
     for (int k = 0; k < W; ++k) pg[i][k] = pb[i][k] = 0.f;
 
+  constexpr bool CACHE = (NV * W <= 32);   // keep the row's dy and x in registers between the two passes
   for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < rows; row += (int64_t)gridDim.x * 4) {
     const int64_t base = row * d;
     const float mu = rms ? 0.f : mean[row];
     const float rs = rstd[row];
     float c1 = 0.f, c2 = 0.f;
+    float cdy[CACHE ? NV : 1][W], cxh[CACHE ? NV : 1][W], cg[CACHE ? NV : 1][W];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int64_t c = ((int64_t)lane + i * 64) * W;
@@ -99,6 +101,11 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
           const float xh = (vx[k] - mu) * rs;
           c1 += gg;
           c2 += gg * xh;
+          if constexpr (CACHE) {
+            cdy[i][k] = vdy[k];
+            cxh[i][k] = xh;
+            cg[i][k] = gg;
+          }
         }
       }
     }
@@ -108,16 +115,29 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
     for (int i = 0; i < NV; ++i) {
       const int64_t c = ((int64_t)lane + i * 64) * W;
       if (c < d) {
-        float vdy[W], vx[W], g[W], o[W];
-        ld_vec<W>(dy, base + c, dy_dt, vdy);
-        ld_vec<W>(x, base + c, x_dt, vx);
-        ld_vec<W>(gamma, c, PF_F32, g);
+        float vdy[W], xhv[W], ggv[W], o[W];
+        if constexpr (CACHE) {
+#pragma unroll
+          for (int k = 0; k < W; ++k) {
+            vdy[k] = cdy[i][k];
+            xhv[k] = cxh[i][k];
+            ggv[k] = cg[i][k];
+          }
+        } else {
+          float vx[W], g[W];
+          ld_vec<W>(dy, base + c, dy_dt, vdy);
+          ld_vec<W>(x, base + c, x_dt, vx);
+          ld_vec<W>(gamma, c, PF_F32, g);
+#pragma unroll
+          for (int k = 0; k < W; ++k) {
+            ggv[k] = vdy[k] * g[k];
+            xhv[k] = (vx[k] - mu) * rs;
+          }
+        }
 #pragma unroll
         for (int k = 0; k < W; ++k) {
-          const float gg = vdy[k] * g[k];
-          const float xh = (vx[k] - mu) * rs;
-          o[k] = rs * (gg - c1 - xh * c2);
-          pg[i][k] += vdy[k] * xh;
+          o[k] = rs * (ggv[k] - c1 - xhv[k] * c2);
+          pg[i][k] += vdy[k] * xhv[k];
           pb[i][k] += vdy[k];
         }
         if (dx_add) {
