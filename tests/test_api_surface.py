@@ -1,4 +1,4 @@
-"""The public API surface user scripts rely on (SURVEY boundary table): names, argparse
+"""The public API surface user scripts rely on: names, argparse
 flags, option parsing, import paths of the reference package."""
 import argparse
 

@@ -122,7 +122,7 @@ def test_vit_tiny_fp32_two_stages():
 
 @pytest.mark.parametrize("mixed", [None, "fp16", "bf16"])
 def test_vit_s16_config_c1(mixed):
-    """BASELINE config 0: ViT-S/16, micro-batch 4 x 4, two stages split at block 6, CE loss."""
+    """The CPU-runnable reference configuration: ViT-S/16, micro-batch 4 x 4, two stages split at block 6, CE loss."""
     from pfeife_amd.bench_models.vit import VIT_S16
 
     m, r, l, rl, _ = _run_vit(VIT_S16, 16, 4, "blocks.6", mixed)
@@ -179,7 +179,7 @@ def _check_grads(model, ref, mixed):
 
 @pytest.mark.parametrize("mixed", [None, "bf16"])
 def test_llama_style_four_stages_looped(mixed):
-    """BASELINE config 2 at reduced width: Llama-style decoder, 4 stages looped over 2
+    """The Llama-style decoder configuration at reduced width, 4 stages looped over 2
     pipeline ranks, micro-batch 2 x 8, next-token CE inside the last stage."""
     import torch.nn.functional as F
 
@@ -222,7 +222,7 @@ def test_llama_style_four_stages_looped(mixed):
 
 @pytest.mark.parametrize("mixed", [None, "bf16"])
 def test_vit_g_block_share_head_dim_88(mixed):
-    """BASELINE config 3 at reduced depth: ViT-g/14 blocks (dim 1408, 16 heads of 88,
+    """The ViT-g/14 block-share configuration at reduced depth: blocks (dim 1408, 16 heads of 88,
     MLP 6144, 257 tokens) fed with activations, sum loss on the output."""
     from oracle.stage_oracle import run_pipeline_step
     from pfeife_amd.bench_models.vit import BlockStack, ViTConfig
@@ -261,7 +261,7 @@ def test_vit_g_block_share_head_dim_88(mixed):
 
 @pytest.mark.parametrize("mixed", [None, "fp16", "bf16"])
 def test_unet_stage_sdxl_style(mixed):
-    """BASELINE config 4 at reduced width: ResNet blocks (GroupNorm 32, 3x3 convs, time
+    """The SDXL UNet-stage configuration at reduced width: ResNet blocks (GroupNorm 32, 3x3 convs, time
     embedding), spatial transformers with self- and cross-attention to 77 context tokens,
     GEGLU; MSE loss against an N(0,1) target computed in user code.  In fp16 the user code
     scales the loss (the reference script wraps it in a GradScaler,
