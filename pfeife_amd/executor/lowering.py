@@ -111,6 +111,24 @@ class ParamStore:
                 out.append(self.kernels.fill(a, 0.0, used))
         return out
 
+    def scale_grads_launches(self, factor):
+        """Launches multiplying every gradient accumulator by `factor` (loss-scale removal)."""
+        out = []
+        slots = dict((i, a) for i, a in getattr(self, "_arena_slots", []))
+        done = set()
+        for i, launch in enumerate(self.zero):
+            if launch is None:
+                a = slots[i]
+                used = self._arena_used if a is self._arena else a.numel()
+                out.append(self.kernels.axpby(a, factor, None, 0.0, a, used))
+                done.add(a.data_ptr())
+        for p in self.params:
+            g = self._grads[id(p)]
+            base = g._base if g._base is not None else g
+            if base.data_ptr() not in done:
+                out.append(self.kernels.axpby(g, factor, None, 0.0, g, g.numel()))
+        return out
+
     def shadow_t(self, tensor, dtype):
         """Transposed copy [cols, rows] of a 2-d parameter in `dtype`, refreshed once per step."""
         key = (tensor.data_ptr(), tuple(tensor.shape), tensor.dtype, dtype, "T")

@@ -256,10 +256,14 @@ class StageWorker:
         if g.shape != buf.shape:
             raise RuntimeError("loss gradient of output %d has shape %s, expected %s"
                                % (out_idx, tuple(g.shape), tuple(buf.shape)))
+        scale = self.option.loss_scale
         if g.device == buf.device and g.is_contiguous() and buf.is_contiguous() and g.dtype.is_floating_point:
-            self.kernels.cast(g, buf, g.numel())(self.stream())
+            if scale != 1.0:
+                self.kernels.axpby(g, scale, None, 0.0, buf, g.numel())(self.stream())
+            else:
+                self.kernels.cast(g, buf, g.numel())(self.stream())
         else:
-            buf.copy_(g)
+            buf.copy_(g * scale if scale != 1.0 else g)
 
     def finish_micro_batch(self, mb):
         """Outputs whose hook never fired: zero gradient, except scalars which get 1
@@ -267,7 +271,7 @@ class StageWorker:
         slot = self.mbs[mb]
         for oi, buf in slot.loss_grads.items():
             if oi not in slot.grad_seen:
-                self.kernels.fill(buf, 1.0 if buf.dim() == 0 else 0.0, buf.numel())(self.stream())
+                self.kernels.fill(buf, self.option.loss_scale if buf.dim() == 0 else 0.0, buf.numel())(self.stream())
 
     def run_job(self, stage, mb, is_fwd):
         prog = self.mbs[mb].stage_programs[stage]
@@ -287,6 +291,13 @@ class StageWorker:
 
     def optimizer_step(self):
         opt = self.optimizer
+        if self.option.loss_scale != 1.0:   # gradients leave the step unscaled, with or without an optimizer
+            key = (len(self.params.params), len(self.params.zero))
+            if getattr(self, "_unscale_key", None) != key:
+                self._unscale = self.params.scale_grads_launches(1.0 / self.option.loss_scale)
+                self._unscale_key = key
+            for launch in self._unscale:
+                launch(self.stream())
         if opt is None:
             return
         if self._fused_adam_applicable(opt):

@@ -86,6 +86,11 @@ class PipeOption:
         self.use_fsdp = get("use_fsdp", False)
         self.mixed_precision = _PRECISIONS.get(get("mixed_precision", None), get("mixed_precision", None))
 
+        # extension: static loss scale applied ONCE, to the gradients entering the last stage, and
+        # removed again before the optimizer step (the reference's GradScaler scales at every
+        # stage, so its stage i of L sees S^(L-i); see the design notes)
+        self.loss_scale = float(get("loss_scale", 1.0))
+
         self.no_side_effect = get("no_side_effect", False)
         self.no_io_cache = get("no_io_cache", False)
         self.single_comm_thread = get("single_comm_thread", False)

@@ -141,3 +141,31 @@ def test_unsupported_node_fails_loudly():
     with pytest.raises(Exception) as ei:
         runner.step(torch.randn(2, 8))
     assert "no HIP lowering" in str(ei.value) or isinstance(ei.value, Unsupported)
+
+
+def test_static_loss_scale_is_applied_once_and_removed():
+    """option.loss_scale multiplies the gradients entering the last stage and is divided out
+    before the optimizer step: final gradients equal the unscaled ones (powers of two: exactly)."""
+    from pfeife_amd.mp import partial_compiler
+
+    grads = []
+    for scale in (1.0, 1024.0):
+        torch.manual_seed(0)
+        model = VisionTransformer(CFG)
+        option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=["blocks.2"],
+                            optimizer=dict(type="sgd", lr=0.0), loss_scale=scale)
+        runner = make_runner(option)
+        cmodel = torch.compile(model, backend=partial_compiler)
+        crit = nn.CrossEntropyLoss()
+
+        def fn(x, y):
+            loss = crit(cmodel(x).float(), y)
+            loss.backward()
+            return loss.detach()
+
+        runner.set_exec_fn(fn)
+        g = torch.Generator().manual_seed(42)
+        runner.step(torch.randn(4, 3, 32, 32, generator=g), torch.randint(0, 10, (4,), generator=g))
+        grads.append({n: p.grad.clone() for n, p in model.named_parameters()})
+    for n in grads[0]:
+        assert torch.equal(grads[0][n], grads[1][n]), n
