@@ -73,3 +73,39 @@ def split_args_kwargs(args, kwargs, batch_split):
     else:
         kwargs_split = shard_dict_of_args(kwargs, batch_split)
     return args_split, kwargs_split
+
+
+def merge_chunks(chunks, out=None):
+    """Inverse of the split for one tensor argument: stack the per-micro-batch tensors
+    (`batch_cnt` chunks along dimension 0, chunk i holding the rows `chunk_rows` assigns to it)
+    back into one batch-major tensor with the pf_merge_scatter kernel.  The reference returns
+    the per-micro-batch values as a Python list (pfeife/mp/partial/module.py:99-102) and leaves
+    any stacking to user code; this is that stacking done on the device."""
+    chunks = [c for c in chunks]
+    if not chunks:
+        raise ValueError("merge_chunks: no chunks")
+    first = chunks[0]
+    if first.device.type != "cuda":
+        raise RuntimeError("merge_chunks: the merge kernel needs GPU tensors (got %s)" % first.device)
+    from .hip import HipKernels
+
+    k = getattr(merge_chunks, "_k", None)
+    if k is None:
+        k = merge_chunks._k = HipKernels(first.device.index)
+    tail = tuple(first.shape[1:])
+    for c in chunks:
+        if tuple(c.shape[1:]) != tail or c.dtype != first.dtype or c.device != first.device:
+            raise ValueError("merge_chunks: chunks differ in trailing shape, dtype or device")
+    total = sum(int(c.shape[0]) for c in chunks)
+    if out is None:
+        out = torch.empty((total,) + tail, dtype=first.dtype, device=first.device)
+    elif tuple(out.shape) != (total,) + tail or not out.is_contiguous():
+        raise ValueError("merge_chunks: bad output tensor")
+    row_bytes = out[0].numel() * out.element_size() if total else 0
+    start = 0
+    for c in chunks:
+        rows = int(c.shape[0])
+        if rows:
+            k.run("merge_scatter", c.contiguous(), out, row_bytes=row_bytes, row_start=start, n_rows=rows)
+        start += rows
+    return out

@@ -388,3 +388,20 @@ def test_fused_adam_matches_torch_optimizer(opt_type, wd):
         real = results[1][1][n] > 1e-10
         torch.testing.assert_close(results[0][0][n][real], results[1][0][n][real], rtol=2e-5, atol=2e-6, msg=n)
         torch.testing.assert_close(results[0][1][n][real], results[1][1][n][real], rtol=1e-4, atol=1e-9, msg=n)
+
+
+def test_split_then_merge_round_trip_on_device():
+    """split_args_kwargs (views) followed by merge_chunks (pf_merge_scatter) is the identity,
+    bit for bit, including ragged chunk sizes and integer dtypes."""
+    from pfeife_amd.batch import merge_chunks, split_args_kwargs
+
+    g = torch.Generator().manual_seed(0)
+    for N, n, tail, dtype in [(64, 4, (3, 8, 8), torch.float32), (10, 4, (5,), torch.int64), (7, 3, (), torch.float16),
+                              (5, 8, (2, 2), torch.bfloat16)]:
+        if dtype.is_floating_point:
+            x = torch.randn((N,) + tail, generator=g).to(dtype).cuda()
+        else:
+            x = torch.randint(0, 1000, (N,) + tail, generator=g).to(dtype).cuda()
+        args, _ = split_args_kwargs((x,), {}, n)
+        merged = merge_chunks([a[0] for a in args])
+        assert torch.equal(merged, x)
