@@ -212,13 +212,13 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const bool dead = (mx == -INFINITY);
     const float mref = dead ? 0.f : mx;
-    const float alpha = dead ? 1.f : exp2f(m - mx);
+    const float alpha = dead ? 1.f : __builtin_amdgcn_exp2f(m - mx);
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = exp2f(s[t][r] - mref);   // masked entries: exp2(-inf) = 0
+        const float p = __builtin_amdgcn_exp2f(s[t][r] - mref);   // masked entries: exp2(-inf) = 0
         s[t][r] = p;
         psum += p;
       }
@@ -356,12 +356,12 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
         for (int r = 0; r < 16; ++r) {
           const int kj = k0 + t * 32 + acc_row(r, lane);
           const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
-          const float p = ok ? exp2f(s[t][r] * sc - lse2) : 0.f;
+          const float p = ok ? __builtin_amdgcn_exp2f(s[t][r] * sc - lse2) : 0.f;
           s[t][r] = p * (dp[t][r] - dlt) * a.scale;   // dS^T
         }
       } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[t][r] = exp2f(s[t][r] * sc - lse2) * (dp[t][r] - dlt) * a.scale;
+        for (int r = 0; r < 16; ++r) s[t][r] = __builtin_amdgcn_exp2f(s[t][r] * sc - lse2) * (dp[t][r] - dlt) * a.scale;
       }
     }
 #pragma unroll
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int ql = t * 32 + acc_row(r, lane);
-        float p = exp2f(s[t][r] * sc - sLse[ql]);
+        float p = __builtin_amdgcn_exp2f(s[t][r] * sc - sLse[ql]);
         if (masked && kj > q0 + ql + shift) p = 0.f;
         s[t][r] = p;                                         // P
         dp[t][r] = p * (dp[t][r] - sDelta[ql]) * a.scale;    // dS
