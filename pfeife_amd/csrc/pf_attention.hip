@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     }
     // only the tile on the causal diagonal and the ragged last tile need per-element masks
     const bool masked = (k0 + KT > a.Tk) || (a.causal && k0 + KT - 1 > q0 + shift);
-    float mx = m;
+    float mx = m;   // running maximum of the RAW scores (scale > 0, so the ordering is the same)
     if (masked) {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -197,37 +197,36 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
         for (int r = 0; r < 16; ++r) {
           const int kj = k0 + t * 32 + acc_row(r, lane);
           const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
-          s[t][r] = ok ? s[t][r] * sc : -INFINITY;
+          s[t][r] = ok ? s[t][r] : -INFINITY;
           mx = fmaxf(mx, s[t][r]);
         }
     } else {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          s[t][r] *= sc;
-          mx = fmaxf(mx, s[t][r]);
-        }
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[t][r]);
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const bool dead = (mx == -INFINITY);
-    const float mref = dead ? 0.f : mx;
-    const float alpha = dead ? 1.f : __builtin_amdgcn_exp2f(m - mx);
+    const float moff = dead ? 0.f : -mx * sc;
+    const float alpha = dead ? 1.f : __builtin_amdgcn_exp2f((m - mx) * sc);
     float psum = 0.f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(s[t][r] - mref);   // masked entries: exp2(-inf) = 0
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[t][r], sc, moff));   // masked entries: exp2(-inf) = 0
         s[t][r] = p;
         psum += p;
       }
     l = l * alpha + psum;
     m = mx;
+    if (__any(alpha != 1.f)) {   // wavefront-uniform: once the maxima have settled nothing is rescaled
 #pragma unroll
-    for (int o = 0; o < NO; ++o)
+      for (int o = 0; o < NO; ++o)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[o][r] *= alpha;
+        for (int r = 0; r < 16; ++r) oacc[o][r] *= alpha;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const uint4 pf = pack8<DT>(s[j >> 1], 8 * (j & 1));
@@ -253,7 +252,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
           *(uint2*)(O + h0) = w;
         }
       }
-    if ((lane >> 5) == 0) a.lse[((int64_t)bh) * a.Tq + qi] = (l > 0.f) ? (m + log2f(l)) / LOG2E : -INFINITY;
+    if ((lane >> 5) == 0) a.lse[((int64_t)bh) * a.Tq + qi] = (l > 0.f) ? (m * sc + log2f(l)) / LOG2E : -INFINITY;
   }
 }
 
@@ -357,11 +356,11 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
           const int kj = k0 + t * 32 + acc_row(r, lane);
           const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
           const float p = ok ? __builtin_amdgcn_exp2f(s[t][r] * sc - lse2) : 0.f;
-          s[t][r] = p * (dp[t][r] - dlt) * a.scale;   // dS^T
+          s[t][r] = p * (dp[t][r] - dlt);   // dS^T / scale (the scale is applied to dQ at the end)
         }
       } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[t][r] = __builtin_amdgcn_exp2f(s[t][r] * sc - lse2) * (dp[t][r] - dlt) * a.scale;
+        for (int r = 0; r < 16; ++r) s[t][r] = __builtin_amdgcn_exp2f(s[t][r] * sc - lse2) * (dp[t][r] - dlt);
       }
     }
 #pragma unroll
@@ -382,8 +381,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
       for (int g = 0; g < 4; ++g) {
         const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
         if (h0 < a.hd)
-          *(uint2*)(DQ + h0) = make_uint2(M32<DT>::pack(acc[o][4 * g], acc[o][4 * g + 1]),
-                                          M32<DT>::pack(acc[o][4 * g + 2], acc[o][4 * g + 3]));
+          *(uint2*)(DQ + h0) = make_uint2(M32<DT>::pack(acc[o][4 * g] * a.scale, acc[o][4 * g + 1] * a.scale),
+                                          M32<DT>::pack(acc[o][4 * g + 2] * a.scale, acc[o][4 * g + 3] * a.scale));
       }
   }
 }
@@ -474,7 +473,7 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
         float p = __builtin_amdgcn_exp2f(s[t][r] * sc - sLse[ql]);
         if (masked && kj > q0 + ql + shift) p = 0.f;
         s[t][r] = p;                                         // P
-        dp[t][r] = p * (dp[t][r] - sDelta[ql]) * a.scale;    // dS
+        dp[t][r] = p * (dp[t][r] - sDelta[ql]);              // dS / scale (applied to dK at the end)
       }
     }
 #pragma unroll
@@ -498,8 +497,8 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
       for (int g = 0; g < 4; ++g) {
         const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
         if (h0 < a.hd) {
-          *(uint2*)(DK + h0) = make_uint2(M32<DT>::pack(dk[o][4 * g], dk[o][4 * g + 1]),
-                                          M32<DT>::pack(dk[o][4 * g + 2], dk[o][4 * g + 3]));
+          *(uint2*)(DK + h0) = make_uint2(M32<DT>::pack(dk[o][4 * g] * a.scale, dk[o][4 * g + 1] * a.scale),
+                                          M32<DT>::pack(dk[o][4 * g + 2] * a.scale, dk[o][4 * g + 3] * a.scale));
           *(uint2*)(DV + h0) = make_uint2(M32<DT>::pack(dv[o][4 * g], dv[o][4 * g + 1]),
                                           M32<DT>::pack(dv[o][4 * g + 2], dv[o][4 * g + 3]));
         }
