@@ -74,14 +74,22 @@ __device__ __forceinline__ void epilogue_vec8(const Epi& e, int64_t c_base, int6
     for (int k = 0; k < 8; ++k) v[k] = pf_round_to(e.in_dtype, v[k]);
   }
   if (e.aux_out) st_vec<8>(e.aux_out, row * e.ld_aux_out + col, e.in_dtype, v);
-  if (e.act != PF_ACT_NONE) {
+  if (e.act == PF_ACT_GELU) {   // the common case without a per-element switch
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = pf_gelu_erf(v[k]);
+  } else if (e.act != PF_ACT_NONE) {
 #pragma unroll
     for (int k = 0; k < 8; ++k) v[k] = pf_act(e.act, v[k]);
   }
   if (e.dact != PF_ACT_NONE) {
     ld_vec<8>(e.aux_in, row * e.ld_aux_in + col, e.in_dtype, t);
+    if (e.dact == PF_ACT_GELU) {
 #pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] *= pf_act_grad(e.dact, t[k]);
+      for (int k = 0; k < 8; ++k) v[k] *= pf_gelu_erf_grad(t[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 8; ++k) v[k] *= pf_act_grad(e.dact, t[k]);
+    }
   }
   if (e.residual) {
     ld_vec<8>(e.residual, row * e.ld_res + col, e.res_dtype, t);
