@@ -295,7 +295,7 @@ template <int R, int BK, int NT> struct Stage<R, BK, NT, true> {
 // tile kt+1 is already in registers (or landing) and tile kt+2 is being issued,
 // which covers the ~1 us L2/HBM latency at two workgroups per CU.
 template <int DT, int BM, int BN, int BK, int WGM, int WGN, bool AT, bool BT>
-__global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)) ? 1 : 2)) void gemm16_kernel(const pf_gemm_desc p,
+__global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)) ? 1 : 2)  /* 8 wavefronts: 1 or 2 workgroups = 2 or 4 waves per SIMD */) void gemm16_kernel(const pf_gemm_desc p,
                                                                                               const GemmGrid g) {
   constexpr int NT = 64 * WGM * WGN;           // threads: WGM x WGN wavefronts
   constexpr int WM = BM / WGM, WN = BN / WGN;  // per-wavefront sub-tile
@@ -589,7 +589,11 @@ int choose_tile(const pf_gemm_desc& d) {
 template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
   switch (choose_tile(d)) {
-    case 0: return launch16<DT, 128, 128, 64, 2, 2>(d, st);
+    case 0:
+      // eight wavefronts (32x64 each) hide more latency per workgroup; measured +5..20% when both
+      // operands use the same loader, -30% when exactly one of them is transposed
+      if (d.a_trans == d.b_trans) return launch16<DT, 128, 128, 64, 4, 2>(d, st);
+      return launch16<DT, 128, 128, 64, 2, 2>(d, st);
     case 1: return launch16<DT, 128, 64, 64, 2, 2>(d, st);
     default: return launch16<DT, 64, 64, 64, 2, 2>(d, st);
   }
@@ -661,6 +665,11 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
 extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   PF_REQUIRE(desc && out && cap > 0, "pf_gemm_variant: bad arguments");
   static const char* tile_names[3] = {"128, 128, 64, 2, 2", "128, 64, 64, 2, 2", "64, 64, 64, 2, 2"};
+  if (desc->in_dtype != PF_F32 && choose_tile(*desc) == 0 && desc->a_trans == desc->b_trans) {
+    snprintf(out, (size_t)cap, "gemm16_kernel<%d, 128, 128, 64, 4, 2, %s, %s>", desc->in_dtype,
+             desc->a_trans ? "true" : "false", desc->b_trans ? "true" : "false");
+    return PF_OK;
+  }
   if (desc->in_dtype == PF_F32) {
     snprintf(out, (size_t)cap, "gemm32_kernel");
   } else {
