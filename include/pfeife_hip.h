@@ -86,6 +86,11 @@ int pf_graph_destroy(void* graph_exec);
  *
  * in_dtype PF_F16/PF_BF16 run on v_mfma_f32_32x32x16 with fp32 accumulation;
  * in_dtype PF_F32 runs a full-precision fp32 FMA kernel (the fp32 parity path).
+ * 16-bit products whose operands are both reduction-contiguous (a_trans = b_trans = 0,
+ * K a multiple of 64) or both reduction-strided (a_trans = b_trans = 1) take the
+ * direct-to-LDS kernel (tiles stream global -> LDS without staging registers, 3-5 stages
+ * deep; transposing LDS reads for the strided case); every other 16-bit product takes a
+ * register-staged kernel.
  *
  * Replaces: aten::linear / aten::addmm / aten::mm / aten::bmm forward and
  * backward, the autocast casts around them, aten::gelu(+backward), the
@@ -122,14 +127,18 @@ typedef struct pf_gemm_desc {
   const void* residual;
   int64_t ld_res;
   int32_t res_dtype;
-  int32_t reserved;
+  int32_t variant; /* 0: automatic tile choice; otherwise one kernel variant by id (tuning
+                      harnesses): 1..3 direct-to-LDS kernel with 256x256 / 256x128 / 128x128
+                      tiles, 11..14 register-staged kernel with 128x128 (8 wavefronts),
+                      128x128, 128x64, 64x64 tiles; PF_ERR_INVALID if it cannot run the problem */
 } pf_gemm_desc;
 
 int pf_gemm(const pf_gemm_desc* desc, void* stream);
 /* Name of the kernel instantiation pf_gemm would launch for `desc`, spelled the
- * way a profiler prints it (e.g. "gemm16_kernel<1, 128, 128, false, false>":
- * dtype, tile M, tile N, a_trans, b_trans).  Lets a harness attribute measured
- * kernel time to problem shapes.  No counterpart in the reference. */
+ * way a profiler prints it, e.g. "gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 0>"
+ * (dtype, tile M, tile N, stage depth, wavefront grid, stages, a_trans, b_trans, epilogue
+ * class) or "gemm16_kernel<1, 128, 64, 64, 2, 2, false, true>".  Lets a harness attribute
+ * measured kernel time to problem shapes.  No counterpart in the reference. */
 int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap);
 
 /* ---- normalisation (HBM-bound, one wavefront per row) ---------------------

@@ -13,148 +13,13 @@
 //
 //   fp32 operands: a plain register-tiled FMA kernel (full fp32 accuracy; it is
 //   the parity path, not the throughput path).
-#include <type_traits>
+#include "pf_gemm_common.h"
 
-#include "pf_common.h"
+// direct-to-LDS kernels, one translation unit per operand dtype
+int pf_gemm_x_f16(const pf_gemm_desc& d, int tile, hipStream_t st);
+int pf_gemm_x_bf16(const pf_gemm_desc& d, int tile, hipStream_t st);
 
 namespace {
-
-struct GemmGrid {
-  int tiles_m, tiles_n, per_xcd;
-  int vec_epi;  // every epilogue operand is 16-byte aligned with leading dimensions % 8 == 0
-};
-
-// Epilogue operands, copied out of the descriptor so that they live in scalar registers.
-struct Epi {
-  float alpha;
-  int beta, round_mid, act, dact, in_dtype, c_dtype, bias_dtype, res_dtype;
-  const void* bias;
-  void* aux_out;
-  const void* aux_in;
-  const void* residual;
-  void* C;
-  int64_t ldc, ld_aux_out, ld_aux_in, ld_res;
-};
-
-__device__ __forceinline__ Epi make_epi(const pf_gemm_desc& p) {
-  Epi e;
-  e.alpha = p.alpha; e.beta = p.beta; e.round_mid = p.round_mid; e.act = p.act; e.dact = p.dact;
-  e.in_dtype = p.in_dtype; e.c_dtype = p.c_dtype; e.bias_dtype = p.bias_dtype; e.res_dtype = p.res_dtype;
-  e.bias = p.bias; e.aux_out = p.aux_out; e.aux_in = p.aux_in; e.residual = p.residual; e.C = p.C;
-  e.ldc = p.ldc; e.ld_aux_out = p.ld_aux_out; e.ld_aux_in = p.ld_aux_in; e.ld_res = p.ld_res;
-  return e;
-}
-
-// one element (scalar path: fp32 kernel and ragged / unaligned tails)
-__device__ __forceinline__ void epilogue_scalar(const Epi& e, int64_t c_base, int64_t row, int64_t col, float acc) {
-  float v = e.alpha * acc;
-  if (e.bias) v += pf_load_as_f32(e.bias, col, e.bias_dtype);
-  if (e.round_mid) v = pf_round_to(e.in_dtype, v);
-  if (e.aux_out) pf_store_from_f32(e.aux_out, row * e.ld_aux_out + col, e.in_dtype, v);
-  if (e.act != PF_ACT_NONE) v = pf_act(e.act, v);
-  if (e.dact != PF_ACT_NONE) v *= pf_act_grad(e.dact, pf_load_as_f32(e.aux_in, row * e.ld_aux_in + col, e.in_dtype));
-  if (e.residual) v += pf_load_as_f32(e.residual, row * e.ld_res + col, e.res_dtype);
-  const int64_t ci = c_base + row * e.ldc + col;
-  if (e.beta) v += pf_load_as_f32(e.C, ci, e.c_dtype);
-  pf_store_from_f32(e.C, ci, e.c_dtype, v);
-}
-
-// 8 consecutive columns of one row (vector path)
-__device__ __forceinline__ void epilogue_vec8(const Epi& e, int64_t c_base, int64_t row, int64_t col, float (&v)[8]) {
-  float t[8];
-#pragma unroll
-  for (int k = 0; k < 8; ++k) v[k] *= e.alpha;
-  if (e.bias) {
-    ld_vec<8>(e.bias, col, e.bias_dtype, t);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] += t[k];
-  }
-  if (e.round_mid) {
-#pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] = pf_round_to(e.in_dtype, v[k]);
-  }
-  if (e.aux_out) st_vec<8>(e.aux_out, row * e.ld_aux_out + col, e.in_dtype, v);
-  if (e.act == PF_ACT_GELU) {   // the common case without a per-element switch
-#pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] = pf_gelu_erf(v[k]);
-  } else if (e.act != PF_ACT_NONE) {
-#pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] = pf_act(e.act, v[k]);
-  }
-  if (e.dact != PF_ACT_NONE) {
-    ld_vec<8>(e.aux_in, row * e.ld_aux_in + col, e.in_dtype, t);
-    if (e.dact == PF_ACT_GELU) {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] *= pf_gelu_erf_grad(t[k]);
-    } else {
-#pragma unroll
-      for (int k = 0; k < 8; ++k) v[k] *= pf_act_grad(e.dact, t[k]);
-    }
-  }
-  if (e.residual) {
-    ld_vec<8>(e.residual, row * e.ld_res + col, e.res_dtype, t);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] += t[k];
-  }
-  const int64_t ci = c_base + row * e.ldc + col;
-  if (e.beta) {
-    ld_vec<8>(e.C, ci, e.c_dtype, t);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) v[k] += t[k];
-  }
-  st_vec<8>(e.C, ci, e.c_dtype, v);
-}
-
-// XCD-aware tile id: consecutive workgroup ids are dealt round-robin to the 8
-// XCDs, so give each XCD a contiguous range of tiles (its L2 then sees a compact
-// set of A rows / B columns). Returns -1 for the padding workgroups.
-__device__ __forceinline__ int gemm_tile_id(int tiles, int per_xcd) {
-  const int pid = blockIdx.x;
-  const int t = (pid & 7) * per_xcd + (pid >> 3);
-  return t < tiles ? t : -1;
-}
-
-// Tile id -> (tile row, tile column) in grouped order: ids walk down GROUP_M tile
-// rows before moving to the next tile column, so the ~32-64 workgroups an XCD runs
-// at the same time cover a compact patch of C and share their A rows and B columns
-// through that XCD's L2 instead of streaming whole operands from HBM.
-constexpr int GROUP_M = 8;
-__device__ __forceinline__ void gemm_tile_rc(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int per_group = GROUP_M * tiles_n;
-  const int group = t / per_group;
-  const int first_m = group * GROUP_M;
-  const int gm = tiles_m - first_m < GROUP_M ? tiles_m - first_m : GROUP_M;
-  const int r = t - group * per_group;
-  tm = first_m + r % gm;
-  tn = r / gm;
-}
-
-// ---------------------------------------------------------------------------
-// 16-bit MFMA kernel
-// ---------------------------------------------------------------------------
-constexpr int EPI_LD = 40;       // floats per row of the 32x32 epilogue staging tile
-
-template <int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (N > 0) {
-    static_for<N - 1>(f);
-    f(std::integral_constant<int, N - 1>{});
-  }
-}
-
-template <int DT> struct Mfma;
-template <> struct Mfma<PF_F16> {
-  static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, a), __builtin_bit_cast(half8_t, b), c, 0,
-                                                  0, 0);
-  }
-};
-template <> struct Mfma<PF_BF16> {
-  static __device__ __forceinline__ float16_t run(uint4 a, uint4 b, float16_t c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c,
-                                                   0, 0, 0);
-  }
-};
 
 // Global -> register -> LDS staging of one operand tile: R rows of the output
 // dimension x BK reduction elements, LDS rows padded by 8 halves (16 bytes) so
@@ -168,16 +33,6 @@ template <> struct Mfma<PF_BF16> {
 // offset register per vector, so a whole tile's loads are in flight together.
 // Only the reduction tail (K not a multiple of BK, last tile) is masked in
 // software, at LDS-store time.
-typedef int v4i_t __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-__device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t byte_off) {
-  const v4i_t x = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_off, 0, 0);
-  return make_uint4((uint32_t)x.x, (uint32_t)x.y, (uint32_t)x.z, (uint32_t)x.w);
-}
-
 template <int R, int BK, int NT, bool TRANS> struct Stage;
 
 template <int R, int BK, int NT> struct Stage<R, BK, NT, false> {
@@ -523,8 +378,6 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const pf_gemm_desc p, const
   }
 }
 
-bool epi_ptr_ok(const void* p, int64_t ld) { return p == nullptr || (pf_aligned(p, 16) && ld % 8 == 0); }
-
 template <int DT, int BM, int BN, int BK, int WGM, int WGN>
 int launch16(const pf_gemm_desc& d, hipStream_t st) {
   constexpr int NT = 64 * WGM * WGN;
@@ -533,9 +386,7 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
   g.tiles_n = (int)((d.N + BN - 1) / BN);
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   g.per_xcd = (int)((total + 7) / 8);
-  g.vec_epi = epi_ptr_ok(d.C, d.ldc) && d.c_stride1 % 8 == 0 && d.c_stride2 % 8 == 0 &&
-              (d.bias == nullptr || pf_aligned(d.bias, 16)) && epi_ptr_ok(d.aux_out, d.ld_aux_out) &&
-              epi_ptr_ok(d.aux_in, d.ld_aux_in) && epi_ptr_ok(d.residual, d.ld_res);
+  g.vec_epi = epi_vec_ok(d);
   const dim3 grid((unsigned)(g.per_xcd * 8), (unsigned)(d.batch1 * d.batch2), 1);
   size_t lds = 2 * (size_t)(BM + BN) * (BK + 8) * sizeof(uint16_t);
   const size_t lds_epi = (size_t)(WGM * WGN) * (BN / WGN / 32) * 32 * EPI_LD * sizeof(float);
@@ -567,35 +418,78 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
   return PF_OK;
 }
 
-// Tile choice.  Measured on MI355X these kernels are bound by L2 -> CU operand
-// traffic, which per FLOP halves when the tile edge doubles; 128x128 with two
-// workgroups resident per CU is the largest configuration that keeps its
-// accumulators, two sets of staging registers and the fragment registers inside
-// the register file, so it is the ceiling here.  Smaller tiles are for problems
-// that would otherwise leave most of the 256 CUs without a workgroup.
-//   0: 128x128   1: 128x64   2: 64x64      (BK 64, 4 wavefronts)
-// (A 256x128 tile run by 8 wavefronts was measured too: same throughput as 128x128, so it is not built.)
-int choose_tile(const pf_gemm_desc& d) {
-  const int64_t nb = (d.batch1 > 0 ? d.batch1 : 1) * (d.batch2 > 0 ? d.batch2 : 1);
+// Variant ids (pf_gemm_desc.variant; 0 = automatic):
+//   1..3   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128
+//   11..14 register-staged kernel: 128x128 by 8 wavefronts, 128x128, 128x64, 64x64 by 4
+enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
+
+// Register-staged tiles: 128x128 with two workgroups resident per CU is the largest that keeps
+// accumulators, two sets of staging registers and fragments in the register file; smaller tiles
+// are for problems that would otherwise leave most of the 256 CUs without a workgroup.
+int choose_staged(const pf_gemm_desc& d) {
+  const int64_t nb = d.batch1 * d.batch2;
   auto tiles = [&](int bm, int bn) { return ((d.M + bm - 1) / bm) * ((d.N + bn - 1) / bn) * nb; };
-  if (tiles(128, 128) >= 256 && d.M >= 128 && d.N >= 128) return 0;
-  // weight-gradient products (both operands transposed) reduce over thousands of tokens and
-  // have few output tiles: the larger tile's operand reuse beats filling every CU
-  if (d.a_trans && d.b_trans && d.K >= 1024 && tiles(128, 128) >= 96 && d.M >= 128 && d.N >= 128) return 0;
-  if (tiles(128, 64) >= 256 && d.M >= 128) return 1;
-  return 2;
+  const bool big = (tiles(128, 128) >= 256 || (d.a_trans && d.b_trans && d.K >= 1024 && tiles(128, 128) >= 96)) &&
+                   d.M >= 128 && d.N >= 128;
+  // eight wavefronts (32x64 each) hide more latency per workgroup; measured +5..20% when both
+  // operands use the same loader, -30% when exactly one of them is transposed
+  if (big) return d.a_trans == d.b_trans ? V_R128W8 : V_R128;
+  if (tiles(128, 64) >= 256 && d.M >= 128) return V_R128x64;
+  return V_R64;
 }
+
+// Can the direct-to-LDS kernel run this problem with tile `xt`?  It takes both operands
+// reduction-contiguous or both reduction-strided; a ragged reduction tail is zero-filled by the
+// hardware range check only in the second case (whole k-rows fall outside the operand).
+bool x_supports(const pf_gemm_desc& d, int xt) {
+  const int bk = xt == PF_XT_256x256 ? 32 : 64;
+  if (d.a_trans != d.b_trans) return false;
+  if (!d.a_trans && d.K % bk != 0) return false;
+  return d.K >= bk;
+}
+
+// Automatic choice: a small cost model fitted to measurements on MI355X (microseconds).  One
+// workgroup per CU; a tile step of 64 along K costs t64 (MFMA issue for the big tile, operand
+// delivery from L2 for the small ones, which also slow down once every CU streams at the same
+// time); a launch costs ~8 us of fixed latency (dispatch, first tile, epilogue).
+int choose_variant(const pf_gemm_desc& d) {
+  const int64_t nb = d.batch1 * d.batch2;
+  if (d.M < 128 || d.N < 128 || d.M * d.N < 128 * 128 * 16) return choose_staged(d);
+  struct Cand { int v, xt, bm, bn; double t64, t64_busy; };
+  static const Cand cands[3] = {{V_X256, PF_XT_256x256, 256, 256, 1.45, 1.45},
+                                {V_X256x128, PF_XT_256x128, 256, 128, 0.85, 0.90},
+                                {V_X128, PF_XT_128x128, 128, 128, 0.50, 0.62}};
+  int best = -1;
+  double best_t = 0;
+  for (const Cand& c : cands) {
+    if (!x_supports(d, c.xt)) continue;
+    const int64_t tiles = ((d.M + c.bm - 1) / c.bm) * ((d.N + c.bn - 1) / c.bn) * nb;
+    const int64_t rounds = (tiles + 255) / 256;
+    const double t = 8.0 + (double)rounds * ((double)d.K / 64.0) * (tiles > 256 ? c.t64_busy : c.t64);
+    if (best < 0 || t < best_t) { best = c.v; best_t = t; }
+  }
+  return best < 0 ? choose_staged(d) : best;
+}
+
+int resolve_variant(const pf_gemm_desc& d) { return d.variant == V_AUTO ? choose_variant(d) : d.variant; }
 
 template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
-  switch (choose_tile(d)) {
-    case 0:
-      // eight wavefronts (32x64 each) hide more latency per workgroup; measured +5..20% when both
-      // operands use the same loader, -30% when exactly one of them is transposed
-      if (d.a_trans == d.b_trans) return launch16<DT, 128, 128, 64, 4, 2>(d, st);
-      return launch16<DT, 128, 128, 64, 2, 2>(d, st);
-    case 1: return launch16<DT, 128, 64, 64, 2, 2>(d, st);
-    default: return launch16<DT, 64, 64, 64, 2, 2>(d, st);
+  const int v = resolve_variant(d);
+  switch (v) {
+    case V_X256: case V_X256x128: case V_X128: {
+      const int xt = v == V_X256 ? PF_XT_256x256 : (v == V_X256x128 ? PF_XT_256x128 : PF_XT_128x128);
+      if (!x_supports(d, xt)) {
+        pf_set_error("pf_gemm: variant %d needs both operands stored alike and (unless transposed) K a multiple of the stage depth", v);
+        return PF_ERR_INVALID;
+      }
+      return DT == PF_F16 ? pf_gemm_x_f16(d, xt, st) : pf_gemm_x_bf16(d, xt, st);
+    }
+    case V_R128W8: return launch16<DT, 128, 128, 64, 4, 2>(d, st);
+    case V_R128: return launch16<DT, 128, 128, 64, 2, 2>(d, st);
+    case V_R128x64: return launch16<DT, 128, 64, 64, 2, 2>(d, st);
+    case V_R64: return launch16<DT, 64, 64, 64, 2, 2>(d, st);
+    default: pf_set_error("pf_gemm: unknown variant %d", d.variant); return PF_ERR_INVALID;
   }
 }
 
@@ -664,17 +558,28 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
 
 extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   PF_REQUIRE(desc && out && cap > 0, "pf_gemm_variant: bad arguments");
-  static const char* tile_names[3] = {"128, 128, 64, 2, 2", "128, 64, 64, 2, 2", "64, 64, 64, 2, 2"};
-  if (desc->in_dtype != PF_F32 && choose_tile(*desc) == 0 && desc->a_trans == desc->b_trans) {
-    snprintf(out, (size_t)cap, "gemm16_kernel<%d, 128, 128, 64, 4, 2, %s, %s>", desc->in_dtype,
-             desc->a_trans ? "true" : "false", desc->b_trans ? "true" : "false");
+  pf_gemm_desc d = *desc;
+  if (d.batch1 <= 0) d.batch1 = 1;
+  if (d.batch2 <= 0) d.batch2 = 1;
+  if (d.in_dtype == PF_F32 || d.K == 0) {
+    snprintf(out, (size_t)cap, "gemm32_kernel");
     return PF_OK;
   }
-  if (desc->in_dtype == PF_F32) {
-    snprintf(out, (size_t)cap, "gemm32_kernel");
-  } else {
-    snprintf(out, (size_t)cap, "gemm16_kernel<%d, %s, %s, %s>", desc->in_dtype, tile_names[choose_tile(*desc)],
-             desc->a_trans ? "true" : "false", desc->b_trans ? "true" : "false");
+  const char* at = d.a_trans ? "true" : "false";
+  const char* bt = d.b_trans ? "true" : "false";
+  const int v = resolve_variant(d);
+  switch (v) {
+    case V_X256: case V_X256x128: case V_X128: {
+      static const char* shapes[4] = {"", "256, 256, 32, 2, 2, 5", "256, 128, 64, 2, 2, 3", "128, 128, 64, 2, 2, 3"};
+      int ec = epi_class(d, epi_vec_ok(d));
+      if (d.a_trans && ec != EC_ACC32 && ec != EC_STORE32) ec = EC_GENERIC;
+      snprintf(out, (size_t)cap, "gemm16x_kernel<%d, %s, %s, %s, %d>", d.in_dtype, shapes[v], at, bt, ec);
+      return PF_OK;
+    }
+    case V_R128W8: snprintf(out, (size_t)cap, "gemm16_kernel<%d, 128, 128, 64, 4, 2, %s, %s>", d.in_dtype, at, bt); return PF_OK;
+    case V_R128: snprintf(out, (size_t)cap, "gemm16_kernel<%d, 128, 128, 64, 2, 2, %s, %s>", d.in_dtype, at, bt); return PF_OK;
+    case V_R128x64: snprintf(out, (size_t)cap, "gemm16_kernel<%d, 128, 64, 64, 2, 2, %s, %s>", d.in_dtype, at, bt); return PF_OK;
+    case V_R64: snprintf(out, (size_t)cap, "gemm16_kernel<%d, 64, 64, 64, 2, 2, %s, %s>", d.in_dtype, at, bt); return PF_OK;
+    default: pf_set_error("pf_gemm_variant: unknown variant %d", d.variant); return PF_ERR_INVALID;
   }
-  return PF_OK;
 }

@@ -1,0 +1,4 @@
+// bf16 instantiations of the direct-to-LDS MFMA kernel.
+#include "pf_gemm_x.h"
+
+int pf_gemm_x_bf16(const pf_gemm_desc& d, int tile, hipStream_t st) { return gemm_x_launch<PF_BF16>(d, tile, st); }

@@ -57,7 +57,7 @@ class GemmDesc(Structure):
         ("act", c_int32), ("dact", c_int32),
         ("aux_in", c_void_p), ("ld_aux_in", c_int64),
         ("residual", c_void_p), ("ld_res", c_int64),
-        ("res_dtype", c_int32), ("reserved", c_int32),
+        ("res_dtype", c_int32), ("variant", c_int32),
     ]
 
 
@@ -242,7 +242,7 @@ class HipKernels:
     # -- dense contractions ----------------------------------------------------
     def gemm(self, a, b, c, M, N, K, lda, ldb, ldc, a_trans=0, b_trans=0, batch=(1, 1), sa=(0, 0), sb=(0, 0),
              sc=(0, 0), alpha=1.0, beta=0, bias=None, round_mid=0, aux_out=None, ld_aux_out=0, act=0, dact=0,
-             aux_in=None, ld_aux_in=0, residual=None, ld_res=0):
+             aux_in=None, ld_aux_in=0, residual=None, ld_res=0, variant=0):
         if a.dtype != b.dtype:
             raise RuntimeError("gemm: operand dtypes differ (%s, %s)" % (a.dtype, b.dtype))
         d = GemmDesc()
@@ -260,12 +260,13 @@ class HipKernels:
         d.act, d.dact = int(act), int(dact)
         d.aux_in, d.ld_aux_in = _ptr(aux_in), ld_aux_in
         d.residual, d.ld_res, d.res_dtype = _ptr(residual), ld_res, _dt(residual)
+        d.variant = int(variant)
         for t in (aux_out, aux_in):
             if t is not None and t.dtype != a.dtype:
                 raise RuntimeError("gemm: aux tensors must have the operand dtype")
         launch = self._prep("pf_gemm", (byref(d),), (d, a, b, c, bias, aux_out, aux_in, residual))
-        name = ctypes.create_string_buffer(96)
-        self.lib.pf_gemm_variant(byref(d), name, 96)
+        name = ctypes.create_string_buffer(128)
+        self.lib.pf_gemm_variant(byref(d), name, 128)
         launch.variant = name.value.decode()
         launch.flops = 2.0 * M * N * K * batch[0] * batch[1]
         return launch

@@ -19,6 +19,8 @@ OBJ_DIR = os.path.join(HERE, "build")
 SOURCES = [
     "pf_runtime.cpp",
     "pf_gemm.hip",
+    "pf_gemm_x_f16.hip",
+    "pf_gemm_x_bf16.hip",
     "pf_attention.hip",
     "pf_norm.hip",
     "pf_elementwise.hip",
@@ -58,7 +60,7 @@ def build(verbose=True, jobs=None):
     if not os.path.exists(HIPCC):
         raise RuntimeError("hipcc not found at %s (set HIPCC)" % HIPCC)
     os.makedirs(OBJ_DIR, exist_ok=True)
-    jobs = jobs or min(len(SOURCES), max(1, (os.cpu_count() or 2) // 2))
+    jobs = jobs or min(len(SOURCES), max(1, os.cpu_count() or 2))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         results = list(pool.map(_compile_one, SOURCES))
     objs = [o for o, _ in results]
