@@ -182,10 +182,10 @@ enum {
   EC_GENERIC = -1,
   EC_STORE16 = 0,  // C 16-bit
   EC_STORE32 = 1,  // C fp32
-  EC_ACT16 = 2,    // C 16-bit, pre-activation saved (aux_out), activation
+  EC_ACT16 = 2,    // C 16-bit, pre-activation saved (aux_out), GELU
   EC_RES32 = 3,    // C fp32, fp32 residual added
   EC_ACC32 = 4,    // C fp32 accumulated in place (beta = 1)
-  EC_DACT16 = 5,   // C 16-bit, multiplied by act'(aux_in)
+  EC_DACT16 = 5,   // C 16-bit, multiplied by GELU'(aux_in)
   EC_ACC16 = 6,    // C 16-bit accumulated in place (beta = 1)
 };
 // Epilogue class of a problem (see the EC_* list): the straight-line classes need 16-byte
@@ -204,8 +204,8 @@ inline int epi_class(const pf_gemm_desc& d, int vec_ok) {
   const int n = (act ? 1 : 0) + (dact ? 1 : 0) + (res ? 1 : 0) + (beta ? 1 : 0);
   if (n == 0) return c16 ? EC_STORE16 : EC_STORE32;
   if (n > 1) return EC_GENERIC;
-  if (act) return c16 ? EC_ACT16 : EC_GENERIC;
-  if (dact) return c16 ? EC_DACT16 : EC_GENERIC;
+  if (act) return (c16 && d.act == PF_ACT_GELU) ? EC_ACT16 : EC_GENERIC;
+  if (dact) return (c16 && d.dact == PF_ACT_GELU) ? EC_DACT16 : EC_GENERIC;
   if (res) return (c32 && d.res_dtype == PF_F32) ? EC_RES32 : EC_GENERIC;
   return c32 ? EC_ACC32 : EC_ACC16;
 }

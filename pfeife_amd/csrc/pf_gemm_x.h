@@ -354,31 +354,43 @@ __global__ __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 10
   const int wr_off = ((lane >> 5) * 4) * SLD + (lane & 31);
 
   if constexpr (EC != EC_GENERIC) {
-    // Straight-line epilogue.  All global accesses are raw buffer operations whose range check
-    // drops rows past M (and lanes past N, which get an out-of-range offset), so there is no
-    // branch, hence no join at which the compiler would have to wait for every outstanding
-    // vector memory operation (loads AND the previous pass's stores share one in-order counter).
-    // Operand loads of the next 32-row block are issued before the stores of the current one.
+    // Compact branch-free epilogue: 16 rows of the wavefront's block at a time, ONE copy of the
+    // arithmetic in a rolled loop (unrolled, an epilogue runs to 200 KB of code that streams once
+    // through an instruction cache which starts cold at every launch).
+    // All global accesses are raw buffer operations whose range check drops rows past M (and
+    // lanes past N, which get an out-of-range offset): no branch, so no join at which the
+    // compiler would wait for every outstanding vector memory operation (loads AND the stores of
+    // the previous pass share one in-order counter).  The one operand a class reads (residual,
+    // old C or aux_in) comes in by direct-to-LDS loads, double buffered: the loads of the next 16
+    // rows are issued before the stores of the current ones, and since the counter retires in
+    // order, "those loads have landed" is "at most <the operations issued after them>
+    // outstanding", a compile-time number because nothing here is predicated.
     constexpr bool C32 = EC == EC_STORE32 || EC == EC_RES32 || EC == EC_ACC32;
     constexpr bool LOADS = EC == EC_RES32 || EC == EC_ACC32 || EC == EC_DACT16 || EC == EC_ACC16;
     constexpr bool LOAD32 = EC == EC_RES32 || EC == EC_ACC32;
-    constexpr int NP = 32 / RPP;     // passes per 32-row block
+    constexpr int HB = 16;                 // rows per step
+    constexpr int NHB = TM * 2;            // steps
+    constexpr int NP = HB / RPP;           // passes per step (a pass: every lane 8 columns of one row)
+    constexpr int LPP = LOADS ? (LOAD32 ? 2 : 1) : 0;               // load instructions per pass
+    constexpr int SPP = (C32 ? 2 : 1) + (EC == EC_ACT16 ? 1 : 0);   // store instructions per pass
     constexpr int ESC = C32 ? 4 : 2;
+    constexpr int WAVE_LDS = HB * SLD * 4 + 2 * NP * 2 * 1024;      // stage + two operand buffers
+    static_assert(NW * WAVE_LDS <= 160 * 1024, "epilogue patches exceed LDS");
+    static_assert(NP * (SPP + LPP) <= 63, "too many operations in flight for the 6-bit counter");
+    float* stg = (float*)((char*)smem + wave * WAVE_LDS);
+    const uint32_t raw0 = lds0 + (uint32_t)(wave * WAVE_LDS + HB * SLD * 4);
     const uint32_t OOB = 0x80000000u;
     const int64_t row0 = m0 + wm0 + rd_row;
     const bool col_ok = c8 < N;
-    // C
     const __amdgpu_buffer_rsrc_t rs_c = make_rsrc((const char*)epi.C + c_base * ESC, (uint32_t)(((M - 1) * epi.ldc + N) * ESC));
     const uint32_t off_c = col_ok ? (uint32_t)((row0 * epi.ldc + c8) * ESC) : OOB;
     const uint32_t step_c = (uint32_t)(epi.ldc * ESC);
-    // the one operand that is read (residual / old C / aux_in), if any
     const void* lp = EC == EC_RES32 ? epi.residual : (EC == EC_DACT16 ? epi.aux_in : (const void*)((const char*)epi.C + c_base * ESC));
     const int64_t ld_l = EC == EC_RES32 ? epi.ld_res : (EC == EC_DACT16 ? epi.ld_aux_in : epi.ldc);
     constexpr int ESL = LOAD32 ? 4 : 2;
     const __amdgpu_buffer_rsrc_t rs_l = make_rsrc(LOADS ? lp : epi.C, LOADS ? (uint32_t)(((M - 1) * ld_l + N) * ESL) : 0u);
     const uint32_t off_l = col_ok ? (uint32_t)((row0 * ld_l + c8) * ESL) : OOB;
     const uint32_t step_l = (uint32_t)(ld_l * ESL);
-    // aux_out
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(EC == EC_ACT16 ? epi.aux_out : epi.C,
                                                   EC == EC_ACT16 ? (uint32_t)(((M - 1) * epi.ld_aux_out + N) * 2) : 0u);
     const uint32_t off_x = col_ok ? (uint32_t)((row0 * epi.ld_aux_out + c8) * 2) : OOB;
@@ -386,65 +398,85 @@ __global__ __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 10
     const float alpha = epi.alpha;
     const bool round_mid = epi.round_mid != 0;
 
-    v4i_t raw[2][NP][LOAD32 ? 2 : 1];
-    auto fetch = [&](auto ic, auto setc) {
-      constexpr int i = decltype(ic)::value, set = decltype(setc)::value;
+    auto fetch = [&](int hb) {   // rows past the block (hb == NHB) are requested too; nobody reads them
       if constexpr (LOADS) {
+        const uint32_t dst = raw0 + (uint32_t)((hb & 1) * NP * LPP) * 1024u;
 #pragma unroll
         for (int pp = 0; pp < NP; ++pp) {
-          const uint32_t o = off_l + (uint32_t)(i * 32 + pp * RPP) * step_l;
-          raw[set][pp][0] = __builtin_amdgcn_raw_buffer_load_b128(rs_l, (int)o, 0, 0);
-          if constexpr (LOAD32) raw[set][pp][1] = __builtin_amdgcn_raw_buffer_load_b128(rs_l, (int)(o + 16), 0, 0);
+          const uint32_t o = off_l + (uint32_t)(hb * HB + pp * RPP) * step_l;
+#pragma unroll
+          for (int h = 0; h < LPP; ++h)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_l, (PF_LDS(void))(uintptr_t)(dst + (uint32_t)(pp * LPP + h) * 1024u), 16,
+                                                     (int)(o + 16 * h), 0, 0, 0);
         }
       }
     };
-    fetch(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-    static_for<TM>([&](auto ic) {
-      constexpr int i = decltype(ic)::value;
-      static_for<TN>([&](auto jc) {
-        constexpr int j = decltype(jc)::value;
+    fetch(0);
+#pragma nounroll
+    for (int hb = 0; hb < NHB; ++hb) {
+      static_for<NHB>([&](auto cc) {
+        constexpr int c = decltype(cc)::value;
+        if (hb == c) {
+          static_for<TN>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) stage[wr_off + (8 * (r >> 2) + (r & 3)) * SLD + j * 32] = acc[i][j][r];
+            for (int r8 = 0; r8 < 8; ++r8)
+              stg[wr_off + (8 * (r8 >> 2) + (r8 & 3)) * SLD + j * 32] = acc[c / 2][j][(c % 2) * 8 + r8];
+          });
+        }
       });
-      if constexpr (i + 1 < TM) fetch(std::integral_constant<int, i + 1>{}, std::integral_constant<int, (i + 1) & 1>{});
-#pragma unroll
+      if constexpr (LOADS) {
+        fetch(hb + 1);
+        if (hb == 0) wait_vm<NP * LPP>(); else wait_vm<NP * (SPP + LPP)>();
+      }
+      const uint32_t rawb = raw0 + (uint32_t)((hb & 1) * NP * LPP) * 1024u + (uint32_t)lane * 16u;
+      const uint32_t stg_addr = lds0 + (uint32_t)(wave * WAVE_LDS + (rd_row * SLD + rd_col) * 4);
+#pragma nounroll
       for (int pp = 0; pp < NP; ++pp) {
-        const float4* src = (const float4*)(stage + (pp * RPP + rd_row) * SLD + rd_col);
-        const float4 x = src[0], y = src[1];
-        float8_t v = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+        // LDS reads by inline assembly: the compiler cannot tell these addresses from the
+        // destinations of the direct-to-LDS loads in flight and would wait for all of them (and,
+        // the counter being shared, for every store issued so far) before each ordinary read
+        v4i_t sx, sy, ra, rb;
+        const uint32_t sa = stg_addr + (uint32_t)((pp * RPP) * SLD * 4);
+        asm volatile("ds_read_b128 %0, %1" : "=v"(sx) : "v"(sa) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(sy) : "v"(sa) : "memory");
+        if constexpr (LOADS) {
+          const uint32_t rp = rawb + (uint32_t)(pp * LPP) * 1024u;
+          asm volatile("ds_read_b128 %0, %1" : "=v"(ra) : "v"(rp) : "memory");
+          if constexpr (LOAD32) asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rb) : "v"(rp) : "memory");
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        float8_t v;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v[k] = __int_as_float(sx[k]);
+          v[4 + k] = __int_as_float(sy[k]);
+        }
         v = v * alpha + bias8;
         if (round_mid) {
 #pragma unroll
           for (int k = 0; k < 8; ++k) v[k] = Codec<DT>::round(v[k]);
         }
-        const uint32_t rowk = (uint32_t)(i * 32 + pp * RPP);
-        if constexpr (EC == EC_ACT16) {
+        const uint32_t rowk = (uint32_t)(hb * HB + pp * RPP);
+        if constexpr (EC == EC_ACT16) {   // GELU only (other activations take the generic class)
           __builtin_amdgcn_raw_buffer_store_b128(pack16<DT>(v), rs_x, (int)(off_x + rowk * step_x), 0, 0);
-          if (epi.act == PF_ACT_GELU) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = pf_gelu_erf(v[k]);
-          } else {
-#pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = pf_act(epi.act, v[k]);
-          }
+          for (int k = 0; k < 8; ++k) v[k] = pf_gelu_erf(v[k]);
         }
-        if constexpr (EC == EC_DACT16) {
-          const float8_t t = unpack16<DT>(raw[i & 1][pp][0]);
-          if (epi.dact == PF_ACT_GELU) {
+        if constexpr (EC == EC_DACT16 || EC == EC_ACC16) {
+          const float8_t t = unpack16<DT>(ra);
+          if constexpr (EC == EC_DACT16) {
 #pragma unroll
             for (int k = 0; k < 8; ++k) v[k] *= pf_gelu_erf_grad(t[k]);
           } else {
-#pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] *= pf_act_grad(epi.dact, t[k]);
+            v += t;
           }
         }
-        if constexpr (EC == EC_ACC16) v += unpack16<DT>(raw[i & 1][pp][0]);
         if constexpr (LOAD32) {
-          const v4i_t a = raw[i & 1][pp][0], b = raw[i & 1][pp][1];
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            v[k] += __int_as_float(a[k]);
-            v[4 + k] += __int_as_float(b[k]);
+            v[k] += __int_as_float(ra[k]);
+            v[4 + k] += __int_as_float(rb[k]);
           }
         }
         const uint32_t oc = off_c + rowk * step_c;
@@ -461,7 +493,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 10
           __builtin_amdgcn_raw_buffer_store_b128(pack16<DT>(v), rs_c, (int)oc, 0, 0);
         }
       }
-    });
+    }
     return;
   }
 
@@ -505,7 +537,9 @@ template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, boo
 int launch16x_t(const pf_gemm_desc& d, const GemmGrid& g, hipStream_t st) {
   constexpr int NT = 64 * WGM * WGN;
   constexpr size_t lds_main = (size_t)ST * (BM + BN) * BK * 2;
-  constexpr size_t lds_epi = (size_t)(WGM * WGN) * epi_row_blocks(WGM * WGN, BN / WGN, BM / WGM / 32) * 32 * (BN / WGN + 8) * sizeof(float);
+  constexpr size_t lds_gen = (size_t)(WGM * WGN) * epi_row_blocks(WGM * WGN, BN / WGN, BM / WGM / 32) * 32 * (BN / WGN + 8) * sizeof(float);
+  constexpr size_t lds_fast = (size_t)(WGM * WGN) * (16 * (BN / WGN + 8) * 4 + 2 * (16 / (64 / (BN / WGN / 8))) * 2 * 1024);
+  constexpr size_t lds_epi = EC == EC_GENERIC ? lds_gen : lds_fast;
   constexpr size_t lds = lds_main > lds_epi ? lds_main : lds_epi;
   static_assert(lds <= 160 * 1024, "tile pipeline exceeds the 160 KB of LDS");
   auto kern = gemm16x_kernel<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>;
