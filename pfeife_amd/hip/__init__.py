@@ -165,6 +165,11 @@ def _ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def _es(t):
+    """bytes per element of a tensor operand (0 for an absent one)"""
+    return 0 if t is None else t.element_size()
+
+
 def _dt(t, default=PF_F32):
     return default if t is None else dtype_code(t.dtype)
 
@@ -193,7 +198,9 @@ class HipKernels:
             raise RuntimeError("pfeife_amd: pf_init failed: %s" % last_error())
 
     # -- helpers -------------------------------------------------------------
-    def _prep(self, fname, args, keep):
+    def _prep(self, fname, args, keep, nbytes=None):
+        """A prepared launch: `launch(stream)`.  `nbytes`: algorithmic HBM bytes of the launch (each
+        operand touched once at its storage dtype), for harnesses that report achieved GB/s."""
         fn = getattr(self.lib, fname)
         lib = self.lib
 
@@ -203,6 +210,7 @@ class HipKernels:
                 raise RuntimeError("%s failed (%d): %s" % (_name, rc, lib.pf_last_error().decode()))
 
         launch.kernel = fname
+        launch.bytes = nbytes
         return launch
 
     def run(self, name, *a, **kw):
@@ -232,6 +240,13 @@ class HipKernels:
         replay.kernel = "pf_graph_launch"
         replay.handle = h
         return replay
+
+    def destroy_graph(self, replay):
+        """Frees the hipGraphExec behind a replay callable returned by `capture` (idempotent)."""
+        h = getattr(replay, "handle", None)
+        if h:
+            replay.handle = None
+            self.lib.pf_graph_destroy(h)
 
     def colreduce_workspace(self, rows, cols):
         return int(self.lib.pf_colreduce_workspace(rows, cols))
@@ -303,12 +318,13 @@ class HipKernels:
     # -- normalisation -----------------------------------------------------------
     def layernorm_fwd(self, x, gamma, beta, y, mean, rstd, rows, d, eps):
         args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(beta), _ptr(y), _dt(y), _ptr(mean), _ptr(rstd), rows, d, eps)
-        return self._prep("pf_layernorm_fwd", args, (x, gamma, beta, y, mean, rstd))
+        return self._prep("pf_layernorm_fwd", args, (x, gamma, beta, y, mean, rstd), rows * d * (_es(x) + _es(y)))
 
     def layernorm_bwd(self, dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws, rows, d, defer=0):
         args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx_add), _dt(dx_add),
                 _ptr(dx), _dt(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), rows, d, int(defer))
-        return self._prep("pf_layernorm_bwd", args, (dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws))
+        return self._prep("pf_layernorm_bwd", args, (dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws),
+                          rows * d * (_es(dy) + _es(x) + _es(dx) + _es(dx_add)))
 
     def groupnorm_workspace(self, B, C, groups):
         return int(self.lib.pf_groupnorm_workspace(B, C, groups))
@@ -316,25 +332,27 @@ class HipKernels:
     def groupnorm_fwd(self, x, gamma, beta, y, mean, rstd, B, HW, C, groups, eps):
         args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(beta), _ptr(y), _dt(y), _ptr(mean), _ptr(rstd), B, HW, C, groups,
                 eps)
-        return self._prep("pf_groupnorm_fwd", args, (x, gamma, beta, y, mean, rstd))
+        return self._prep("pf_groupnorm_fwd", args, (x, gamma, beta, y, mean, rstd), B * HW * C * (2 * _es(x) + _es(y)))
 
     def groupnorm_bwd(self, dy, x, gamma, mean, rstd, dx, dgamma, dbeta, ws, B, HW, C, groups, defer=0):
         args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(mean), _ptr(rstd), _ptr(dx), _dt(dx),
                 _ptr(dgamma), _ptr(dbeta), _ptr(ws), B, HW, C, groups, int(defer))
-        return self._prep("pf_groupnorm_bwd", args, (dy, x, gamma, mean, rstd, dx, dgamma, dbeta, ws))
+        return self._prep("pf_groupnorm_bwd", args, (dy, x, gamma, mean, rstd, dx, dgamma, dbeta, ws),
+                          B * HW * C * (2 * _es(dy) + 2 * _es(x) + _es(dx)))
 
     def rmsnorm_fwd(self, x, gamma, y, rstd, rows, d, eps):
         args = (_ptr(x), _dt(x), _ptr(gamma), _ptr(y), _dt(y), _ptr(rstd), rows, d, eps)
-        return self._prep("pf_rmsnorm_fwd", args, (x, gamma, y, rstd))
+        return self._prep("pf_rmsnorm_fwd", args, (x, gamma, y, rstd), rows * d * (_es(x) + _es(y)))
 
     def rmsnorm_bwd(self, dy, x, gamma, rstd, dx_add, dx, dgamma, ws, rows, d, defer=0):
         args = (_ptr(dy), _dt(dy), _ptr(x), _dt(x), _ptr(gamma), _ptr(rstd), _ptr(dx_add), _dt(dx_add), _ptr(dx),
                 _dt(dx), _ptr(dgamma), _ptr(ws), rows, d, int(defer))
-        return self._prep("pf_rmsnorm_bwd", args, (dy, x, gamma, rstd, dx_add, dx, dgamma, ws))
+        return self._prep("pf_rmsnorm_bwd", args, (dy, x, gamma, rstd, dx_add, dx, dgamma, ws),
+                          rows * d * (_es(dy) + _es(x) + _es(dx) + _es(dx_add)))
 
     def colsum_accumulate(self, x, rows, cols, ld, acc, ws, defer=0):
         args = (_ptr(x), _dt(x), rows, cols, ld, _ptr(acc), _ptr(ws), int(defer))
-        return self._prep("pf_colsum_accumulate", args, (x, acc, ws))
+        return self._prep("pf_colsum_accumulate", args, (x, acc, ws), rows * cols * _es(x))
 
     def norm_bwd_partials(self, rows):
         return int(self.lib.pf_norm_bwd_partials(rows))
@@ -357,22 +375,23 @@ class HipKernels:
     # -- softmax / losses ----------------------------------------------------------
     def softmax_fwd(self, s, ld_s, p, ld_p, rows, cols, q_len, causal):
         args = (_ptr(s), ld_s, _ptr(p), _dt(p), ld_p, rows, cols, q_len, int(causal))
-        return self._prep("pf_softmax_fwd", args, (s, p))
+        return self._prep("pf_softmax_fwd", args, (s, p), rows * cols * (_es(s) + _es(p)))
 
     def softmax_bwd(self, dp, ld_dp, p, ld_p, ds, ld_ds, rows, cols, scale):
         args = (_ptr(dp), ld_dp, _ptr(p), _dt(p), ld_p, _ptr(ds), _dt(ds), ld_ds, rows, cols, scale)
-        return self._prep("pf_softmax_bwd", args, (dp, p, ds))
+        return self._prep("pf_softmax_bwd", args, (dp, p, ds), rows * cols * (_es(dp) + _es(p) + _es(ds)))
 
     def cross_entropy_fwd(self, logits, targets, row_loss, row_lse, loss, rows, classes, ignore_index):
         args = (_ptr(logits), _dt(logits), _ptr(targets), _ptr(row_loss), _ptr(row_lse), _ptr(loss), rows, classes,
                 ignore_index)
-        return self._prep("pf_cross_entropy_fwd", args, (logits, targets, row_loss, row_lse, loss))
+        return self._prep("pf_cross_entropy_fwd", args, (logits, targets, row_loss, row_lse, loss), rows * classes * _es(logits))
 
     def cross_entropy_bwd(self, logits, targets, row_lse, dloss, loss, dlogits, rows, classes, ignore_index):
         n_valid = loss.data_ptr() + 4
         args = (_ptr(logits), _dt(logits), _ptr(targets), _ptr(row_lse), _ptr(dloss), n_valid, _ptr(dlogits),
                 _dt(dlogits), rows, classes, ignore_index)
-        return self._prep("pf_cross_entropy_bwd", args, (logits, targets, row_lse, dloss, loss, dlogits))
+        return self._prep("pf_cross_entropy_bwd", args, (logits, targets, row_lse, dloss, loss, dlogits),
+                          rows * classes * (_es(logits) + _es(dlogits)))
 
     def mse_fwd(self, a, b, partial, loss, n):
         args = (_ptr(a), _dt(a), _ptr(b), _dt(b), _ptr(partial), _ptr(loss), n)
@@ -388,30 +407,30 @@ class HipKernels:
 
     # -- elementwise -----------------------------------------------------------------
     def act_fwd(self, x, y, act, n):
-        return self._prep("pf_act_fwd", (_ptr(x), _ptr(y), _dt(x), int(act), n), (x, y))
+        return self._prep("pf_act_fwd", (_ptr(x), _ptr(y), _dt(x), int(act), n), (x, y), 2 * n * _es(x))
 
     def act_bwd(self, dy, x, dx, act, n):
-        return self._prep("pf_act_bwd", (_ptr(dy), _ptr(x), _ptr(dx), _dt(x), int(act), n), (dy, x, dx))
+        return self._prep("pf_act_bwd", (_ptr(dy), _ptr(x), _ptr(dx), _dt(x), int(act), n), (dy, x, dx), 3 * n * _es(x))
 
     def glu_fwd(self, gate, ld_gate, up, ld_up, y, ld_y, act, rows, cols):
         args = (_ptr(gate), ld_gate, _ptr(up), ld_up, _ptr(y), ld_y, _dt(gate), int(act), rows, cols)
-        return self._prep("pf_glu_fwd", args, (gate, up, y))
+        return self._prep("pf_glu_fwd", args, (gate, up, y), 3 * rows * cols * _es(gate))
 
     def glu_bwd(self, dy, ld_dy, gate, ld_gate, up, ld_up, dgate, ld_dgate, dup, ld_dup, act, rows, cols):
         args = (_ptr(dy), ld_dy, _ptr(gate), ld_gate, _ptr(up), ld_up, _ptr(dgate), ld_dgate, _ptr(dup), ld_dup,
                 _dt(gate), int(act), rows, cols)
-        return self._prep("pf_glu_bwd", args, (dy, gate, up, dgate, dup))
+        return self._prep("pf_glu_bwd", args, (dy, gate, up, dgate, dup), 5 * rows * cols * _es(gate))
 
     def axpby(self, a, alpha, b, beta, out, n):
         args = (_ptr(a), _dt(a), alpha, _ptr(b), _dt(b), beta, _ptr(out), _dt(out), n)
-        return self._prep("pf_axpby", args, (a, b, out))
+        return self._prep("pf_axpby", args, (a, b, out), n * (_es(a) + _es(b) + _es(out)))
 
     def bias_add(self, x, bias, y, n, bias_len, rows_per_bias=0):
         args = (_ptr(x), _dt(x), _ptr(bias), _dt(bias), _ptr(y), _dt(y), n, bias_len, rows_per_bias)
         return self._prep("pf_bias_add", args, (x, bias, y))
 
     def cast(self, src, dst, n):
-        return self._prep("pf_cast", (_ptr(src), _dt(src), _ptr(dst), _dt(dst), n), (src, dst))
+        return self._prep("pf_cast", (_ptr(src), _dt(src), _ptr(dst), _dt(dst), n), (src, dst), n * (_es(src) + _es(dst)))
 
     def cast_batch(self, pairs):
         """One launch casting every (src, dst) pair of contiguous tensors."""
@@ -426,7 +445,7 @@ class HipKernels:
 
     def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
         args = (_ptr(src), _dt(src), ld_src, _ptr(dst), _dt(dst), ld_dst, rows, cols)
-        return self._prep("pf_transpose_cast", args, (src, dst))
+        return self._prep("pf_transpose_cast", args, (src, dst), rows * cols * (_es(src) + _es(dst)))
 
     def adam_table(self, params, grads, exp_avgs, exp_avg_sqs):
         """Device table of pf_adam_item for one param group (built once, pointers are static)."""
@@ -461,7 +480,7 @@ class HipKernels:
         return self._prep("pf_rope", args, (x, y, cos_t, sin_t))
 
     def grad_accumulate(self, acc, g, n):
-        return self._prep("pf_grad_accumulate_f32", (_ptr(acc), _ptr(g), _dt(g), n), (acc, g))
+        return self._prep("pf_grad_accumulate_f32", (_ptr(acc), _ptr(g), _dt(g), n), (acc, g), n * (8 + _es(g)))
 
     # -- micro-batch split / merge, embedding ---------------------------------------------
     def split_gather(self, src, dst, row_bytes, row_start, n_rows, index=None):

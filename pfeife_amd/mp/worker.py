@@ -191,10 +191,45 @@ class StageWorker:
                 if ref[0] == sid and oi in slot.loss_grads:
                     out_grads[ref[1]].append(slot.loss_grads[oi])
             L.lower_backward(prog, out_grads)
+        self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
         self.mbs[mb] = slot
         self.graphs_ready = False   # new programs (and possibly new parameters): capture again
-        self.begin_graph = None
+        self._drop_begin_graph()
         return slot
+
+    def _drop_graphs(self, slot):
+        """Frees the captured hipGraphs of a micro-batch slot that is being replaced or released."""
+        if slot is None or not hasattr(self.kernels, "destroy_graph"):
+            return
+        for prog in slot.stage_programs.values():
+            for attr in ("fwd_graph", "bwd_graph"):
+                g = getattr(prog, attr, None)
+                if g is not None:
+                    self.kernels.destroy_graph(g)
+                    setattr(prog, attr, None)
+
+    def _drop_begin_graph(self):
+        if self.begin_graph is not None and hasattr(self.kernels, "destroy_graph"):
+            self.kernels.destroy_graph(self.begin_graph)
+        self.begin_graph = None
+
+    def release(self):
+        """Frees every captured graph and drops the stage programs and their buffers (the worker
+        cannot run another step afterwards)."""
+        if self.stream_obj is not None:
+            self.stream_obj.synchronize()
+        for slot in self.mbs.values():
+            self._drop_graphs(slot)
+        self._drop_begin_graph()
+        self.mbs = {}
+        self.graphs_ready = False
+        self.static_inputs = {}
+        self.part_graph = None
+        self.optimizer = None
+        self.params = ParamStore(self.kernels, self.device)
+        self.pool = BufferPool(self.device)
+        self.lowerer = Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
+        self.__dict__.pop("_adam_tables", None)
 
     # -- per step --------------------------------------------------------------------
     def stream(self):
@@ -212,6 +247,7 @@ class StageWorker:
                 if prog.bwd_graph is None and prog.bwd:
                     prog.bwd_graph = self.kernels.capture(prog.bwd, s)
         pre = self.params.zero_launches() + self.params.refresh_launches()
+        self._drop_begin_graph()
         self.begin_graph = self.kernels.capture(pre, s) if pre else None
         self._begin_len = (len(self.params.zero), len(self.params.refresh))
         self.graphs_ready = True
