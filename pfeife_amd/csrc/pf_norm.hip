@@ -9,10 +9,14 @@
 
 namespace {
 
-constexpr int COLRED_MAX_BLOCKS = 512;
+constexpr int COLRED_MAX_BLOCKS = 1024;
 
 // ---- forward ---------------------------------------------------------------
-template <int W>
+// NV > 0: the row (d <= 64*W*NV) is loaded ONCE into registers, all loads in flight together;
+// mean, then the sum of squared deviations, then the output come from the registers: one memory
+// round trip per row instead of three dependent ones (the kernel is latency-bound, a row is
+// 2-8 KB).  NV == 0: any d, three sweeps over the row (the second and third hit L2).
+template <int W, int NV>
 __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, const float* gamma, const float* beta,
                                                        void* y, int y_dt, float* mean, float* rstd, int64_t rows,
                                                        int64_t d, float eps, int rms) {
@@ -20,6 +24,63 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
   const int64_t row = (int64_t)blockIdx.x * 4 + wave;
   if (row >= rows) return;
   const int64_t base = row * d;
+  if constexpr (NV > 0) {
+    float v[NV][W], g[NV][W], b[NV][W];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int64_t c = ((int64_t)lane + i * 64) * W;
+      if (c < d) {
+        ld_vec<W>(x, base + c, x_dt, v[i]);
+        ld_vec<W>(gamma, c, PF_F32, g[i]);
+        if (beta) ld_vec<W>(beta, c, PF_F32, b[i]);
+      } else {
+#pragma unroll
+        for (int k = 0; k < W; ++k) v[i][k] = 0.f;
+      }
+    }
+    float mu = 0.f;
+    if (!rms) {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int k = 0; k < W; ++k) s += v[i][k];
+      mu = pf_wave_sum(s) / (float)d;
+    }
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      if (((int64_t)lane + i * 64) * W < d) {
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          const float t = v[i][k] - mu;
+          q += t * t;
+        }
+      }
+    }
+    const float var = pf_wave_sum(q) / (float)d;
+    const float rs = 1.0f / sqrtf(var + eps);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int64_t c = ((int64_t)lane + i * 64) * W;
+      if (c < d) {
+        float o[W];
+        if (beta) {
+#pragma unroll
+          for (int k = 0; k < W; ++k) o[k] = (v[i][k] - mu) * rs * g[i][k] + b[i][k];
+        } else {
+#pragma unroll
+          for (int k = 0; k < W; ++k) o[k] = (v[i][k] - mu) * rs * g[i][k];
+        }
+        st_vec<W>(y, base + c, y_dt, o);
+      }
+    }
+    if (lane == 0) {
+      if (mean) mean[row] = mu;
+      rstd[row] = rs;
+    }
+    return;
+  }
   float mu = 0.f;
   if (!rms) {
     float s = 0.f;
@@ -86,7 +147,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
     const float mu = rms ? 0.f : mean[row];
     const float rs = rstd[row];
     float c1 = 0.f, c2 = 0.f;
-    float cdy[CACHE ? NV : 1][W], cxh[CACHE ? NV : 1][W], cg[CACHE ? NV : 1][W];
+    float cdy[CACHE ? NV : 1][W], cxh[CACHE ? NV : 1][W], cg[CACHE ? NV : 1][W], cadd[CACHE ? NV : 1][W];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int64_t c = ((int64_t)lane + i * 64) * W;
@@ -95,6 +156,11 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
         ld_vec<W>(dy, base + c, dy_dt, vdy);
         ld_vec<W>(x, base + c, x_dt, vx);
         ld_vec<W>(gamma, c, PF_F32, g);
+        // the gradient already accumulated on x: requested with the other operands, so that the
+        // row costs one memory round trip, not a second one after the reductions
+        if constexpr (CACHE) {
+          if (dx_add) ld_vec<W>(dx_add, base + c, add_dt, cadd[i]);
+        }
 #pragma unroll
         for (int k = 0; k < W; ++k) {
           const float gg = vdy[k] * g[k];
@@ -141,10 +207,15 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
           pb[i][k] += vdy[k];
         }
         if (dx_add) {
-          float a[W];
-          ld_vec<W>(dx_add, base + c, add_dt, a);
+          if constexpr (CACHE) {
 #pragma unroll
-          for (int k = 0; k < W; ++k) o[k] += a[k];
+            for (int k = 0; k < W; ++k) o[k] += cadd[i][k];
+          } else {
+            float a[W];
+            ld_vec<W>(dx_add, base + c, add_dt, a);
+#pragma unroll
+            for (int k = 0; k < W; ++k) o[k] += a[k];
+          }
         }
         st_vec<W>(dx, base + c, dx_dt, o);
       }
@@ -210,11 +281,21 @@ __global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, in
 #pragma unroll
   for (int k = 0; k < W; ++k) s[k] = 0.f;
   if (c < cols) {
-    for (int64_t r = r0 + wave; r < r1; r += 4) {
-      float v[W];
-      ld_vec<W>(x, r * ld + c, x_dt, v);
+    // 8 rows requested together (the loop is short and latency-bound), summed in row order
+    for (int64_t r = r0 + wave; r < r1; r += 32) {
+      float v[8][W];
 #pragma unroll
-      for (int k = 0; k < W; ++k) s[k] += v[k];
+      for (int u = 0; u < 8; ++u) {
+        if (r + 4 * u < r1) ld_vec<W>(x, (r + 4 * u) * ld + c, x_dt, v[u]);
+        else {
+#pragma unroll
+          for (int k = 0; k < W; ++k) v[u][k] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int k = 0; k < W; ++k) s[k] += v[u][k];
     }
   }
 #pragma unroll
@@ -368,8 +449,14 @@ int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, voi
   PF_REQUIRE((rows + 3) / 4 < (1ll << 31), "%s: too many rows", name);
   const dim3 grid((unsigned)((rows + 3) / 4));
   const bool v = vec_ok(x, x_dt, d) && vec_ok(y, y_dt, d) && vec_ok(gamma, PF_F32, d) && vec_ok(beta, PF_F32, d);
-  if (v) hipLaunchKernelGGL(norm_fwd_kernel<8>, grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms);
-  else hipLaunchKernelGGL(norm_fwd_kernel<1>, grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms);
+#define PF_NF(W, NV) \
+  hipLaunchKernelGGL((norm_fwd_kernel<W, NV>), grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms)
+  if (v && d <= 64 * 8 * 1) PF_NF(8, 1);
+  else if (v && d <= 64 * 8 * 2) PF_NF(8, 2);
+  else if (v && d <= 64 * 8 * 4) PF_NF(8, 4);
+  else if (v) PF_NF(8, 0);
+  else PF_NF(1, 0);
+#undef PF_NF
   PF_CHECK_LAUNCH(name);
   return PF_OK;
 }

@@ -25,7 +25,7 @@ def _fresh_runner(option):
     return PartialRunner(option)
 
 
-def _run_vit(cfg, batch, batch_cnt, split, mixed, device_cnt=2, steps=1, seed=0, history=None):
+def _run_vit(cfg, batch, batch_cnt, split, mixed, device_cnt=2, steps=1, seed=0, history=None, oracle_device="cpu"):
     from oracle.stage_oracle import run_pipeline_step
     from pfeife_amd.bench_models.vit import VisionTransformer
     from pfeife_amd.mp import partial_compiler
@@ -62,8 +62,11 @@ def _run_vit(cfg, batch, batch_cnt, split, mixed, device_cnt=2, steps=1, seed=0,
                             {n: p.grad.detach().clone() for n, p in model.named_parameters()}))
     torch.cuda.synchronize()
 
-    # oracle: the reference's stage semantics on CPU (autocast for mixed precision)
-    k = int(split.split(".")[1]) if split else cfg.depth
+    # oracle: the reference's stage semantics on CPU (autocast for mixed precision).  An integer
+    # split point indexes compute nodes of the captured graph; the oracle then splits in the
+    # middle, which gives the same losses and gradients (a pipelined step equals un-pipelined
+    # gradient accumulation wherever the boundary is).
+    k = int(split.split(".")[1]) if isinstance(split, str) else (cfg.depth // 2 if split else cfg.depth)
 
     class Stage0(nn.Module):
         def __init__(self, m):
@@ -90,6 +93,7 @@ def _run_vit(cfg, batch, batch_cnt, split, mixed, device_cnt=2, steps=1, seed=0,
             return m.head(m.norm(t)[:, 0])
 
     adt = {"fp16": torch.float16, "bf16": torch.bfloat16}.get(mixed)
+    ref.to(oracle_device)   # "cuda": the oracle's stage executor on PyTorch's own ATen kernels
     stages = [Stage0(ref), Stage1(ref)] if split else [nn.Sequential(Stage0(ref), Stage1(ref))]
     ref_losses = run_pipeline_step(stages, lambda o, t: crit(o.float(), t), x, y, batch_cnt,
                                    device_cnt=device_cnt, autocast_dtype=adt)
@@ -103,7 +107,7 @@ def _check(model, ref, losses, ref_losses, mixed):
         a, b = float(a), float(b)
         assert abs(a - b) <= ltol * abs(b), ("loss", a, b)
     for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
-        gp, gq = p.grad.float().cpu(), q.grad.float()
+        gp, gq = p.grad.float().cpu(), q.grad.float().cpu()
         assert torch.isfinite(gp).all(), n
         if mixed is None:
             assert (gp - gq).abs().max() <= 1e-4 * gq.abs().max() + 1e-9, (n, float((gp - gq).abs().max()))
@@ -127,6 +131,64 @@ def test_vit_s16_config_c1(mixed):
 
     m, r, l, rl, _ = _run_vit(VIT_S16, 16, 4, "blocks.6", mixed)
     _check(m, r, l, rl, mixed)
+
+
+def _gemm_variants(runner):
+    names = set()
+    for slot in runner.worker.mbs.values():
+        for prog in slot.stage_programs.values():
+            for launch in list(prog.fwd) + list(prog.bwd):
+                if getattr(launch, "kernel", "") == "pf_gemm":
+                    names.add(launch.variant)
+    return names
+
+
+def test_vit_l_width_fp16_headline_geometry():
+    """The headline configuration's own dimensions (ViT-L/16: dim 1024, 16 heads, MLP 4096, 197 tokens,
+    micro-batch 16 x 4, two stages, fp16) at reduced depth (2 + 2 blocks).  The oracle's stage executor
+    runs on the GPU here, on PyTorch's own ATen kernels under autocast (which is what the reference
+    executes): on the test machine's host cores the fp16 autocast path takes minutes at this width.
+    Every matrix product has the headline's shape (3152 token rows), and the step must run on the
+    kernel instantiations the benchmark times."""
+    from pfeife_amd.bench_models.vit import ViTConfig
+
+    cfg = ViTConfig(image_size=224, patch_size=16, dim=1024, depth=4, heads=16, mlp_dim=4096, num_classes=1000)
+    m, r, l, rl, runner = _run_vit(cfg, 64, 4, "blocks.2", "fp16", oracle_device="cuda")
+    _check(m, r, l, rl, "fp16")
+    names = _gemm_variants(runner)
+    want = ["gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 2>",    # fc1: GELU epilogue
+            "gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 5>",    # dX of fc2: GELU' epilogue
+            "gemm16x_kernel<1, 128, 128, 64, 2, 2, 3, false, false, 3>",    # proj / fc2: fp32 residual epilogue
+            "gemm16x_kernel<1, 128, 128, 64, 2, 2, 3, true, true, 4>"]      # weight gradients, accumulated
+    for w in want:
+        assert w in names, (w, sorted(names))
+
+
+def test_ragged_batch_on_device():
+    """N % batch_cnt != 0: torch.tensor_split gives micro-batches of 3, 3, 2, 2 samples
+    (pfeife/batch.py:45); every one gets its own stage programs."""
+    from pfeife_amd.bench_models.vit import ViTConfig
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=4, heads=4, mlp_dim=128, num_classes=16)
+    for mixed in (None, "bf16"):
+        m, r, l, rl, runner = _run_vit(cfg, 10, 4, "blocks.2", mixed)
+        _check(m, r, l, rl, mixed)
+        sizes = [slot.input_sig[0][0][0] for _, slot in sorted(runner.worker.mbs.items())]
+        assert sizes == [3, 3, 2, 2], sizes
+
+
+def test_integer_split_points_on_device():
+    """split_points given as integers (pfeife/schedule/planner.py:635-665): they index the compute
+    nodes of the captured graph; the step must match the oracle and really run two stages."""
+    from pfeife_amd.bench_models.vit import ViTConfig
+    from pfeife_amd.graph.partition_graph import compute_nodes
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=4, heads=4, mlp_dim=128, num_classes=10)
+    m, r, l, rl, runner = _run_vit(cfg, 8, 4, 40, None)
+    _check(m, r, l, rl, None)
+    pg = runner.worker.part_graph
+    assert len(pg.nodes) == 2
+    assert all(len(slot.stage_programs) == 2 for slot in runner.worker.mbs.values())
 
 
 def test_vit_single_stage_and_repeatability():
