@@ -183,6 +183,16 @@ int64_t pf_colreduce_workspace(int64_t rows, int64_t cols);
  * Replaces the sum-to-size of aten::addmm's bias gradient + AccumulateGrad. */
 int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
                          float* workspace, int defer_reduce, void* stream);
+/* The same reduction for callers that cannot allocate device memory or carry a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the
+ * partial rows live in a device array built into the library, pf_colsum_static_capacity()
+ * floats (8 MiB) per GPU, held until the process ends.  Always finishes the reduction into
+ * `acc` (no deferred mode).  PF_ERR_INVALID when pf_colsum_partials(rows) * cols exceeds the
+ * capacity.  Calls that overlap in time on one GPU share the array and race; calls on one
+ * stream are ordered.  Allocates nothing.  No counterpart in the reference. */
+int pf_colsum_accumulate_static(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld, float* acc,
+                                void* stream);
+int64_t pf_colsum_static_capacity(void);
 /* Deferred column reductions.  With defer_reduce != 0 the three functions above only
  * write their per-workgroup partial rows into `workspace` (layout: norm backward
  * [pf_norm_bwd_partials(rows)][2][d] = dgamma then dbeta partials; column sum

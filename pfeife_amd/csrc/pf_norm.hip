@@ -5,6 +5,8 @@
 // second/third pass, so HBM sees it once.  Parameter gradients (dgamma, dbeta,
 // bias gradients) are reduced deterministically in two stages: per-workgroup
 // column partials in a caller-supplied workspace, then one thread per column.
+#include <mutex>
+
 #include "pf_common.h"
 
 namespace {
@@ -666,4 +668,66 @@ extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, in
                      (int)chunks, cols, cols, acc);
   PF_CHECK_LAUNCH("pf_colsum_accumulate(finalize)");
   return PF_OK;
+}
+
+
+// ---- column sum without any allocation ---------------------------------------------------
+// The partial rows of the two-stage column reduction live in a device array that is part of
+// the library image (each GPU the library runs on holds its own copy until the process ends)
+// instead of a caller-supplied workspace.  Host code may only use the array's device address,
+// fetched once per device with that device current; the array's name is a host-side stand-in.
+constexpr int64_t STATIC_SCRATCH_FLOATS = 256 * 8192;   // 256 partial rows x 8192 columns = 8 MiB
+static __device__ __align__(256) float pf_colsum_scratch[STATIC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[MAX_DEVICES] = {};
+
+// address of the current device's copy of the scratch array (looked up once per device)
+int scratch_for_current_device(float** out, const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    pf_set_error("%s: cannot identify the current device (%s)", who, e == hipSuccess ? "index out of range" : hipGetErrorString(e));
+    return PF_ERR_HIP;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(pf_colsum_scratch));
+    if (e != hipSuccess || p == nullptr) {
+      pf_set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+      return PF_ERR_HIP;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return PF_OK;
+}
+}  // namespace
+
+// called by pf_init with the device current
+int pf_norm_init_device() {
+  float* p = nullptr;
+  return scratch_for_current_device(&p, "pf_init");
+}
+
+extern "C" int64_t pf_colsum_static_capacity(void) { return STATIC_SCRATCH_FLOATS; }
+
+extern "C" int pf_colsum_accumulate_static(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t ld,
+                                           float* acc, void* stream) {
+  PF_REQUIRE(rows >= 0 && cols >= 0 && ld >= cols, "pf_colsum_accumulate_static: bad shape");
+  if (rows == 0 || cols == 0) return PF_OK;
+  PF_REQUIRE(x && acc, "pf_colsum_accumulate_static: null pointer");
+  const int64_t need = (int64_t)pf_colsum_partials(rows) * cols;
+  PF_REQUIRE(need <= STATIC_SCRATCH_FLOATS,
+             "pf_colsum_accumulate_static: %lld partial rows x %lld columns = %lld floats exceed the built-in scratch "
+             "of %lld floats; use pf_colsum_accumulate with a workspace",
+             (long long)pf_colsum_partials(rows), (long long)cols, (long long)need, (long long)STATIC_SCRATCH_FLOATS);
+  float* scratch = nullptr;
+  const int rc = scratch_for_current_device(&scratch, "pf_colsum_accumulate_static");
+  if (rc != PF_OK) return rc;
+  // every partial the finalize pass reads is written by this call's first pass: nothing to clear
+  return pf_colsum_accumulate(x, x_dtype, rows, cols, ld, acc, scratch, 0, stream);
 }

@@ -4,7 +4,9 @@
 
 #include "pf_common.h"
 
-#define PF_ABI_VERSION 2
+int pf_norm_init_device();   // pf_norm.hip
+
+#define PF_ABI_VERSION 3
 
 static thread_local char g_err[512] = "";
 
@@ -42,7 +44,7 @@ extern "C" int pf_init(int device) {
     pf_set_error("pf_init: hipSetDevice: %s", hipGetErrorString(e));
     return PF_ERR_HIP;
   }
-  return PF_OK;
+  return pf_norm_init_device();   // device addresses of the library's built-in scratch arrays
 }
 
 // ---- hipGraph capture of launch lists ---------------------------------------------

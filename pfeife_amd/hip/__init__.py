@@ -16,7 +16,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpfeife_hip.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 PF_F32, PF_F16, PF_BF16, PF_I64, PF_I32, PF_U8 = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU = 0, 1, 2, 3, 4
@@ -89,6 +89,7 @@ _SIGNATURES = {
     "pf_rmsnorm_fwd": [_P, _I, _P, _P, _I, _P, _L, _L, _F, _P],
     "pf_rmsnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _P, _L, _L, _I, _P],
     "pf_colsum_accumulate": [_P, _I, _L, _L, _L, _P, _P, _I, _P],
+    "pf_colsum_accumulate_static": [_P, _I, _L, _L, _L, _P, _P],
     "pf_colreduce_finalize_batch": [_P, _I, _L, _P],
     "pf_norm_bwd_partials": None,
     "pf_colsum_partials": None,
@@ -121,7 +122,8 @@ _SIGNATURES = {
     "pf_embedding_fwd": [_P, _I, _P, _P, _I, _L, _L, _L, _P],
     "pf_embedding_bwd": [_P, _I, _P, _P, _L, _L, _L, _P],
 }
-_RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L], "pf_groupnorm_workspace": [_L, _L, _I]}
+_RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L], "pf_groupnorm_workspace": [_L, _L, _I],
+            "pf_colsum_static_capacity": []}
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + list(_RET_I64) + ["pf_version", "pf_last_error"])
 
 _lib = None
