@@ -206,14 +206,28 @@ def hbm_kernel_rates(runner, reps=3):
     if opt is not None and w._fused_adam_applicable(opt):
         n_par = sum(p.numel() for g in opt.param_groups for p in g["params"] if p.grad is not None)
         stream = w.stream_obj   # the optimizer step is issued on the worker's own stream
-        w.optimizer_step()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        ev0.record(stream)
-        for _ in range(reps):
-            w.optimizer_step()
-        ev1.record(stream)
-        ev1.synchronize()
-        ms = ev0.elapsed_time(ev1) / reps
+
+        def timed(fn):
+            fn()
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record(stream)
+            for _ in range(reps):
+                fn()
+            ev1.record(stream)
+            ev1.synchronize()
+            return ev0.elapsed_time(ev1) / reps
+
+        if w.dyn_scale:
+            # the in-place unscale + overflow check over the fp32 gradient buffers that precedes the step
+            w.optimizer_step()            # builds the launch list
+            n_g = sum(n for _, n in w.params.grad_buffers())
+            ms = timed(lambda: [launch(w.stream()) for launch in w._unscale])
+            gbs = 8.0 * n_g / (ms * 1e-3) / 1e9
+            out.append(dict(kernel="pf_scaler_unscale", on_path=True, launches_per_step=len(w._unscale),
+                            ms_per_step=round(ms, 3), avg_launch_us=round(1e3 * ms / len(w._unscale), 2),
+                            bytes_per_launch=round(8.0 * n_g / len(w._unscale)), achieved=round(gbs, 1),
+                            peak=PEAK_HBM_GBS, unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4)))
+        ms = timed(lambda: w._fused_adam_step(opt, scaled=w.dyn_scale))
         nb = 28.0 * n_par   # read p, g, m, v; write p, m, v (fp32)
         gbs = nb / (ms * 1e-3) / 1e9
         out.append(dict(kernel="pf_adam_step", on_path=True, launches_per_step=len(opt.param_groups),
@@ -324,11 +338,30 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
     for _ in range(max(0, warmup - 1)):
         runner.step(*batch)
     torch.cuda.synchronize()
+    w = runner.worker
+    applied = lambda: float(w.scaler_state[3]) if w.dyn_scale else float(w.steps_done)
+    if w.dyn_scale:
+        # dynamic loss scaling starts high and halves on overflow (skipping that optimizer step):
+        # extra untimed steps until one is applied, so that every timed step does the full work
+        for extra in range(24):
+            before = applied()
+            runner.step(*batch)
+            torch.cuda.synchronize()
+            if applied() > before:
+                break
+        log("[bench] dynamic loss scale settled at %g after %d extra warm-up steps" % (w.scaler_scale(), extra + 1))
+    before = applied()
     t0 = time.perf_counter()
     for _ in range(steps):
         losses = runner.step(*batch)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    skipped = steps - int(round(applied() - before))
+    scaling = dict(mode="dynamic" if w.dyn_scale else "static",
+                   scale=w.scaler_scale() if w.dyn_scale else float(runner.option.loss_scale),
+                   skipped_optimizer_steps_in_timed_region=skipped)
+    if skipped:
+        log("[bench] WARNING: %d of %d timed steps overflowed and skipped their optimizer step" % (skipped, steps))
     ms = 1e3 * dt / steps
     value = info["batch"] * steps / dt
     log("[bench] %.2f ms/step, %.1f samples/s, last losses %s" % (ms, value, [round(float(l), 4) for l in losses]))
@@ -352,7 +385,7 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
                100 * r["frac"], PEAK_HBM_GBS, "" if r["on_path"] else "  [off-path micro-benchmark]"))
     flops_step = model_flops_per_step(info)
     cfg = info["cfg"]
-    res = dict(value=value, ms=ms, host_ms=host_ms, roof=roof, hbm=rates, info=info,
+    res = dict(value=value, ms=ms, host_ms=host_ms, roof=roof, hbm=rates, info=info, loss_scaling=scaling,
                model_tflops=None if flops_step is None else round(flops_step / (ms * 1e-3) / 1e12, 2),
                workload="%s: %s micro-batch %d x %d, %d stages split at %s, schedule drawn for %d ranks, "
                         "all stages on one GPU, Adam" % (
@@ -442,7 +475,8 @@ def main():
             others.append(dict(workload=res["workload"], value=round(res["value"], 2), unit="samples/s", steps=3,
                                ms_per_step=round(res["ms"], 3), model_tflops=res["model_tflops"],
                                host_enqueue_ms_per_step=round(res["host_ms"], 3), dominant_kernel=roof.get("kernel"),
-                               frac=roof.get("frac"), all_gemm_tflops=roof.get("all_gemm_tflops")))
+                               frac=roof.get("frac"), all_gemm_tflops=roof.get("all_gemm_tflops"),
+                               loss_scaling=res["loss_scaling"]))
             release(r2)
 
     info = head["info"]
@@ -465,6 +499,7 @@ def main():
         "cpu_baseline": cpu,
         "model_tflops": head["model_tflops"],
         "host_enqueue_ms_per_step": round(head["host_ms"], 3),
+        "loss_scaling": head["loss_scaling"],
         "other_workloads": others,
     }
     print(json.dumps(rec), flush=True)

@@ -234,7 +234,9 @@ int pf_softmax_bwd(const float* dp, int64_t ld_dp, const void* p, int p_dtype, i
  * [B,H,Tq] (written by forward, read by backward); delta: fp32 [B,H,Tq] scratch written
  * and read by backward.  hd must be a multiple of 8 and <= 96 (PF_ERR_UNSUPPORTED
  * otherwise: the caller then uses pf_gemm + pf_softmax).  causal: key j is visible to
- * query i iff j <= i + (Tk - Tq).
+ * query i iff j <= i + (Tk - Tq) (bottom-right alignment; for Tq != Tk this is NOT
+ * aten::scaled_dot_product_attention's top-left is_causal mask, so the host lowering
+ * only passes causal when Tq == Tk).
  * Replaces aten::scaled_dot_product_attention and its backward inside a stage
  * (pfeife/mp/worker.py:1494, :1585-1587). */
 typedef struct pf_attn_desc {
@@ -356,6 +358,30 @@ typedef struct pf_adam_item {
 int pf_adam_step(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1, double beta2,
                  double eps, double weight_decay, int64_t step, int adamw, void* stream);
 
+/* ---- dynamic loss scaling on the device ---------------------------------------------
+ * torch.amp.GradScaler's rule without a host synchronisation.  `state` is float[8] in DEVICE
+ * memory: {scale, growth tracker, found_inf, completed optimizer steps, then four floats of
+ * scratch for pf_adam_step_scaled}; the caller initialises it to {init_scale, 0, 0, 0, ...}.
+ *   pf_scale_by_state   dst = src * scale          (GradScaler.scale applied to the gradient
+ *                                                   entering the last stage)
+ *   pf_scaler_unscale   grads *= 1/scale in place; found_inf = 1 if any element is not finite
+ *                       (GradScaler.unscale_); call it for every gradient buffer of the step
+ *   pf_adam_step_scaled pf_adam_step that does nothing when found_inf is set (GradScaler.step)
+ *                       and takes its step count for the bias corrections from the state
+ *                       (it writes the two correction terms into state[4..5] first)
+ *   pf_scaler_update    GradScaler.update: on overflow scale *= backoff_factor; otherwise the
+ *                       step count and the growth tracker advance and every `growth_interval`
+ *                       clean steps scale *= growth_factor; clears found_inf
+ * Replaces WorkerScaler (pfeife/mp/worker.py:133-145) and scaler.step(optimizer) +
+ * scaler.update() (pfeife/mp/worker.py:1432-1436). */
+int pf_scale_by_state(const void* src, int src_dtype, const float* state, void* dst, int dst_dtype, int64_t n,
+                      void* stream);
+int pf_scaler_unscale(float* grads, int64_t n, float* state, void* stream);
+int pf_adam_step_scaled(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1,
+                        double beta2, double eps, double weight_decay, int adamw, float* scaler_state,
+                        void* stream);
+int pf_scaler_update(float* state, double growth_factor, double backoff_factor, int growth_interval, void* stream);
+
 /* ---- gradient accumulation --------------------------------------------------
  * acc[i] += g[i] for i < n, acc fp32, g of dtype g_dtype: autograd's
  * AccumulateGrad `param.grad.add_(new_grad)` executed once per parameter per
@@ -377,11 +403,13 @@ int pf_merge_scatter(const void* src, void* dst, int64_t row_bytes, int64_t row_
                      const int64_t* index, void* stream);
 /* Embedding lookup out[i, :] = table[ids[i], :] with dtype conversion, and its
  * backward dtable[ids[i], :] += dout[i, :] (fp32 accumulate, atomics-free:
- * one wavefront owns a table row).  Replaces aten::embedding(+dense backward). */
+ * one wavefront owns a group of table rows and adds in id-list order).  Entries
+ * equal to padding_idx (-1: none) contribute nothing, so that row's gradient
+ * stays zero.  Replaces aten::embedding(+embedding_dense_backward). */
 int pf_embedding_fwd(const void* table, int t_dtype, const int64_t* ids, void* out, int o_dtype, int64_t n_ids,
                      int64_t dim, int64_t vocab, void* stream);
 int pf_embedding_bwd(const void* dout, int d_dtype, const int64_t* ids, float* dtable_acc, int64_t n_ids,
-                     int64_t dim, int64_t vocab, void* stream);
+                     int64_t dim, int64_t vocab, int64_t padding_idx, void* stream);
 
 #ifdef __cplusplus
 }

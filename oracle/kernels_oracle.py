@@ -432,6 +432,38 @@ class OracleKernels:
 
         return launch
 
+    # -- dynamic loss scaling: torch.amp.GradScaler's rule (pfeife/mp/worker.py:133-145, 1432-1436)
+    # on a float32[8] state {scale, growth tracker, found_inf, completed steps, 4 unused here}
+    def scale_by_state(self, src, state, dst, n):
+        def launch(stream=None):
+            _flat(dst, n).copy_((_flat(src, n).float() * state[0]).to(dst.dtype))
+
+        return launch
+
+    def scaler_unscale(self, grads, n, state):
+        def launch(stream=None):
+            g = _flat(grads, n)
+            g.mul_(1.0 / state[0])
+            if not torch.isfinite(g).all():
+                state[2] = 1.0
+
+        return launch
+
+    def scaler_update(self, state, growth_factor, backoff_factor, growth_interval):
+        def launch(stream=None):
+            if float(state[2]) != 0.0:
+                state[0] *= backoff_factor
+                state[1] = 0.0
+            else:
+                state[1] += 1.0
+                state[3] += 1.0
+                if float(state[1]) >= growth_interval:
+                    state[0] *= growth_factor
+                    state[1] = 0.0
+            state[2] = 0.0
+
+        return launch
+
     def copy_strided(self, src, src_strides, dst, dst_strides, sizes, accumulate=0):
         def launch(stream=None):
             s = _strided(src, tuple(sizes), tuple(src_strides))
@@ -503,8 +535,12 @@ class OracleKernels:
 
         return launch
 
-    def embedding_bwd(self, dout, ids, dtable, n_ids, dim, vocab):
+    def embedding_bwd(self, dout, ids, dtable, n_ids, dim, vocab, padding_idx=-1):
         def launch(stream=None):
-            _rows(dtable, vocab, dim, dim).index_add_(0, _flat(ids, n_ids), _rows(dout, n_ids, dim, dim).float())
+            i = _flat(ids, n_ids)
+            g = _rows(dout, n_ids, dim, dim).float()
+            if padding_idx >= 0:      # aten::embedding_dense_backward leaves the padding row at zero
+                g = g * (i != padding_idx).unsqueeze(1)
+            _rows(dtable, vocab, dim, dim).index_add_(0, i, g)
 
         return launch

@@ -66,23 +66,35 @@ __global__ __launch_bounds__(256) void embedding_fwd_kernel(const void* table, i
   }
 }
 
-// One wavefront owns one vocabulary row: it scans the id list 64 entries at a
-// time and adds the matching output-gradient rows in id-list order, so no two
-// wavefronts write the same row and the summation order is fixed.
+// One wavefront owns EMB_ROWS consecutive vocabulary rows: it scans the id list once, 64 entries
+// at a time (the next 64 are already in flight), and adds the output-gradient rows whose id
+// falls in its range, in id-list order.  No two wavefronts write the same row and the
+// summation order within a row is the list order, so the result is deterministic; the id list
+// is read vocab / EMB_ROWS times instead of once per row.  Ids outside [0, vocab) and the
+// padding index (whose row keeps a zero gradient, as in aten::embedding_dense_backward) match
+// no wavefront.
+constexpr int EMB_ROWS = 16;
+
 template <int W>
 __global__ __launch_bounds__(256) void embedding_bwd_kernel(const void* dout, int d_dt, const int64_t* ids,
-                                                            float* dtable, int64_t n_ids, int64_t dim, int64_t vocab) {
+                                                            float* dtable, int64_t n_ids, int64_t dim, int64_t vocab,
+                                                            int64_t padding_idx) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t v = (int64_t)blockIdx.x * 4 + wave;
-  if (v >= vocab) return;
+  const int64_t v0 = ((int64_t)blockIdx.x * 4 + wave) * EMB_ROWS;
+  if (v0 >= vocab) return;
+  const int64_t v1 = v0 + EMB_ROWS < vocab ? v0 + EMB_ROWS : vocab;
+  int64_t next = lane < n_ids ? ids[lane] : -1;
   for (int64_t base = 0; base < n_ids; base += 64) {
-    const int64_t j = base + lane;
-    const bool hit = j < n_ids && ids[j] == v;
+    const int64_t id = next;
+    const int64_t jn = base + 64 + lane;
+    next = jn < n_ids ? ids[jn] : -1;
+    const bool hit = id >= v0 && id < v1 && id != padding_idx;
     unsigned long long mask = __ballot(hit);
     while (mask) {
       const int b = __ffsll((long long)mask) - 1;
       mask &= mask - 1;
       const int64_t r = base + b;
+      const int64_t v = __shfl(id, b);
       for (int64_t c = (int64_t)lane * W; c < dim; c += 64 * W) {
         float g[W], a[W];
         ld_vec<W>(dout, r * dim + c, d_dt, g);
@@ -126,18 +138,19 @@ extern "C" int pf_embedding_fwd(const void* table, int t_dtype, const int64_t* i
 }
 
 extern "C" int pf_embedding_bwd(const void* dout, int d_dtype, const int64_t* ids, float* dtable_acc, int64_t n_ids,
-                                int64_t dim, int64_t vocab, void* stream) {
+                                int64_t dim, int64_t vocab, int64_t padding_idx, void* stream) {
   PF_REQUIRE(n_ids >= 0 && dim > 0 && vocab > 0 && pf_is_float_dtype(d_dtype), "pf_embedding_bwd: bad arguments");
+  PF_REQUIRE(padding_idx >= -1 && padding_idx < vocab, "pf_embedding_bwd: padding_idx must be -1 (none) or a row");
   if (n_ids == 0) return PF_OK;
   PF_REQUIRE(dout && ids && dtable_acc, "pf_embedding_bwd: null pointer");
   const bool vec = dim % 8 == 0 && pf_aligned(dout, 16) && pf_aligned(dtable_acc, 16);
-  const dim3 grid((unsigned)((vocab + 3) / 4));
+  const dim3 grid((unsigned)((vocab + 4 * EMB_ROWS - 1) / (4 * EMB_ROWS)));
   if (vec)
     hipLaunchKernelGGL(embedding_bwd_kernel<8>, grid, dim3(256), 0, (hipStream_t)stream, dout, d_dtype, ids,
-                       dtable_acc, n_ids, dim, vocab);
+                       dtable_acc, n_ids, dim, vocab, padding_idx);
   else
     hipLaunchKernelGGL(embedding_bwd_kernel<1>, grid, dim3(256), 0, (hipStream_t)stream, dout, d_dtype, ids,
-                       dtable_acc, n_ids, dim, vocab);
+                       dtable_acc, n_ids, dim, vocab, padding_idx);
   PF_CHECK_LAUNCH("pf_embedding_bwd");
   return PF_OK;
 }

@@ -275,11 +275,27 @@ __global__ __launch_bounds__(256) void cast_batch_kernel(const pf_cast_item* ite
 // block y walks item y in a grid-stride loop.  The arithmetic follows torch.optim.Adam's
 // single-tensor formulation operation by operation (lerp for the first moment, mul + addcmul
 // for the second, sqrt / bias_correction2_sqrt + eps, addcdiv).
+// With a loss-scaler state (float[8] = scale, growth tracker, found_inf, completed steps,
+// step_size, bias_c2_sqrt, 2 unused) the launch does nothing when found_inf is set
+// (GradScaler.step skipping the optimizer), and the bias corrections use the device-side count
+// of completed steps, which the host cannot know without a synchronisation: a one-thread launch
+// ahead of this one forms them in double and leaves them in state[4..5].
+__global__ void adam_coefficients_kernel(float* state, double lr, double beta1, double beta2) {
+  const double t = (double)state[3] + 1.0;
+  state[4] = (float)(lr / (1.0 - pow(beta1, t)));
+  state[5] = (float)sqrt(1.0 - pow(beta2, t));
+}
+
 __global__ __launch_bounds__(256) void adam_kernel(const pf_adam_item* items, float lr, float omb1, float beta2,
                                                    float omb2, float eps, float weight_decay, float step_size,
-                                                   float bias_c2_sqrt, int adamw) {
-  // omb1 = 1 - beta1, omb2 = 1 - beta2, step_size = lr / (1 - beta1^t): formed in double on the
-  // host like torch does, then rounded once
+                                                   float bias_c2_sqrt, int adamw, const float* scaler_state) {
+  // omb1 = 1 - beta1, omb2 = 1 - beta2, step_size = lr / (1 - beta1^t): formed in double
+  // like torch does, then rounded once
+  if (scaler_state != nullptr) {
+    if (scaler_state[2] != 0.f) return;   // uniform over the grid
+    step_size = scaler_state[4];
+    bias_c2_sqrt = scaler_state[5];
+  }
   const pf_adam_item it = items[blockIdx.y];
   const int64_t gsz = (int64_t)gridDim.x * blockDim.x * 4;
   for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < it.n; i += gsz) {
@@ -520,22 +536,159 @@ extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, co
   return PF_OK;
 }
 
+namespace {
+int adam_launch(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1, double beta2,
+                double eps, double weight_decay, int64_t step, int adamw, float* scaler_state, void* stream,
+                const char* name);
+}
+
 extern "C" int pf_adam_step(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1,
                             double beta2, double eps, double weight_decay, int64_t step, int adamw, void* stream) {
-  PF_REQUIRE(n_items >= 0 && max_n >= 0 && step >= 1, "pf_adam_step: bad arguments");
+  PF_REQUIRE(step >= 1, "pf_adam_step: bad step");
+  return adam_launch(items_dev, n_items, max_n, lr, beta1, beta2, eps, weight_decay, step, adamw, nullptr, stream,
+                     "pf_adam_step");
+}
+
+extern "C" int pf_adam_step_scaled(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1,
+                                   double beta2, double eps, double weight_decay, int adamw, float* scaler_state,
+                                   void* stream) {
+  PF_REQUIRE(scaler_state != nullptr, "pf_adam_step_scaled: null scaler state");
+  return adam_launch(items_dev, n_items, max_n, lr, beta1, beta2, eps, weight_decay, 1, adamw, scaler_state, stream,
+                     "pf_adam_step_scaled");
+}
+
+// ---- dynamic loss scaling (torch.amp.GradScaler's rule, on the device) -------------------
+namespace {
+// g *= 1/scale in place; found_inf = 1 when any element is not finite (plain store of the same
+// value from every block that sees one: no atomic needed, and deterministic)
+__device__ __forceinline__ unsigned nonfinite(float v) {   // all exponent bits set: inf or NaN
+  return (__float_as_uint(v) & 0x7f800000u) == 0x7f800000u ? 1u : 0u;
+}
+
+__global__ __launch_bounds__(256) void scaler_unscale_kernel(float* g, int64_t n, float* state) {
+  const float inv = 1.0f / state[0];
+  unsigned bad = 0;
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x * 4;
+  for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < n; i += gsz) {
+    if (i + 4 <= n) {
+      float4 v = *(float4*)(g + i);
+      v.x *= inv; v.y *= inv; v.z *= inv; v.w *= inv;
+      bad |= nonfinite(v.x) | nonfinite(v.y) | nonfinite(v.z) | nonfinite(v.w);
+      *(float4*)(g + i) = v;
+    } else {
+      for (int64_t j = i; j < n; ++j) {
+        const float v = g[j] * inv;
+        bad |= nonfinite(v);
+        g[j] = v;
+      }
+    }
+  }
+  if (bad) state[2] = 1.0f;
+}
+
+__global__ void scaler_update_kernel(float* state, float growth, float backoff, int interval) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float scale = state[0], tracker = state[1];
+  if (state[2] != 0.f) {
+    scale *= backoff;
+    tracker = 0.f;
+  } else {
+    tracker += 1.f;
+    state[3] += 1.f;
+    if (tracker >= (float)interval) {
+      scale *= growth;
+      tracker = 0.f;
+    }
+  }
+  state[0] = scale;
+  state[1] = tracker;
+  state[2] = 0.f;
+}
+
+struct ScaleByState {
+  const void* src; int src_dt; const float* state; void* dst; int dst_dt;
+  __device__ __forceinline__ void apply8(int64_t i) const {
+    float v[8];
+    ld_vec<8>(src, i, src_dt, v);
+    const float s = state[0];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] *= s;
+    st_vec<8>(dst, i, dst_dt, v);
+  }
+  __device__ __forceinline__ void apply1(int64_t i) const {
+    pf_store_from_f32(dst, i, dst_dt, pf_load_as_f32(src, i, src_dt) * state[0]);
+  }
+};
+
+__global__ __launch_bounds__(256) void scale_by_state_kernel(ScaleByState f, int64_t n, int vec) {
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t nv = vec ? n / 8 : 0;
+  for (int64_t i = gtid; i < nv; i += gsz) f.apply8(i * 8);
+  for (int64_t i = nv * 8 + gtid; i < n; i += gsz) f.apply1(i);
+}
+}  // namespace
+
+extern "C" int pf_scaler_unscale(float* grads, int64_t n, float* state, void* stream) {
+  PF_REQUIRE(n >= 0, "pf_scaler_unscale: negative size");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(grads && state && pf_aligned(grads, 16), "pf_scaler_unscale: null or unaligned pointer");
+  int64_t blocks = (n / 4 + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(scaler_unscale_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, grads, n, state);
+  PF_CHECK_LAUNCH("pf_scaler_unscale");
+  return PF_OK;
+}
+
+extern "C" int pf_scaler_update(float* state, double growth_factor, double backoff_factor, int growth_interval,
+                                void* stream) {
+  PF_REQUIRE(state && growth_factor >= 1.0 && backoff_factor > 0.0 && backoff_factor <= 1.0 && growth_interval >= 1,
+             "pf_scaler_update: bad arguments");
+  hipLaunchKernelGGL(scaler_update_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, state, (float)growth_factor,
+                     (float)backoff_factor, growth_interval);
+  PF_CHECK_LAUNCH("pf_scaler_update");
+  return PF_OK;
+}
+
+extern "C" int pf_scale_by_state(const void* src, int src_dtype, const float* state, void* dst, int dst_dtype, int64_t n,
+                                 void* stream) {
+  PF_REQUIRE(n >= 0, "pf_scale_by_state: negative size");
+  if (n == 0) return PF_OK;
+  PF_REQUIRE(src && dst && state, "pf_scale_by_state: null pointer");
+  PF_REQUIRE(pf_is_float_dtype(src_dtype) && pf_is_float_dtype(dst_dtype), "pf_scale_by_state: bad dtype");
+  ScaleByState f{src, src_dtype, state, dst, dst_dtype};
+  const int vec = pf_aligned(src, 16) && pf_aligned(dst, 16);
+  int64_t blocks = ((vec ? n / 8 : n) + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(scale_by_state_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, f, n, vec);
+  PF_CHECK_LAUNCH("pf_scale_by_state");
+  return PF_OK;
+}
+
+namespace {
+int adam_launch(const pf_adam_item* items_dev, int n_items, int64_t max_n, double lr, double beta1, double beta2,
+                double eps, double weight_decay, int64_t step, int adamw, float* scaler_state, void* stream,
+                const char* name) {
+  PF_REQUIRE(n_items >= 0 && max_n >= 0, "%s: bad arguments", name);
   if (n_items == 0 || max_n == 0) return PF_OK;
-  PF_REQUIRE(items_dev != nullptr && n_items <= 65535, "pf_adam_step: bad item list");
+  PF_REQUIRE(items_dev != nullptr && n_items <= 65535, "%s: bad item list", name);
   const double bc1 = 1.0 - pow(beta1, (double)step);
   const double bc2 = 1.0 - pow(beta2, (double)step);
   int64_t bx = (max_n / 4 + 255) / 256;
   if (bx > 64) bx = 64;   // enough blocks per tensor; small tensors leave most of them idle at once
   if (bx < 1) bx = 1;
+  if (scaler_state != nullptr)
+    hipLaunchKernelGGL(adam_coefficients_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, scaler_state, lr, beta1,
+                       beta2);
   hipLaunchKernelGGL(adam_kernel, dim3((unsigned)bx, (unsigned)n_items), dim3(256), 0, (hipStream_t)stream, items_dev,
                      (float)lr, (float)(1.0 - beta1), (float)beta2, (float)(1.0 - beta2), (float)eps, (float)weight_decay,
-                     (float)(lr / bc1), (float)sqrt(bc2), adamw);
-  PF_CHECK_LAUNCH("pf_adam_step");
+                     (float)(lr / bc1), (float)sqrt(bc2), adamw, scaler_state);
+  PF_CHECK_LAUNCH(name);
   return PF_OK;
 }
+}  // namespace
 
 extern "C" int pf_cast_batch(const pf_cast_item* items_dev, int n_items, int64_t max_n, void* stream) {
   PF_REQUIRE(n_items >= 0 && max_n >= 0, "pf_cast_batch: bad arguments");

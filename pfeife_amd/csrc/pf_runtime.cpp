@@ -6,7 +6,7 @@
 
 int pf_norm_init_device();   // pf_norm.hip
 
-#define PF_ABI_VERSION 3
+#define PF_ABI_VERSION 4
 
 static thread_local char g_err[512] = "";
 
@@ -70,7 +70,7 @@ extern "C" int pf_graph_capture_end(void* stream, void** graph_exec_out) {
   }
   hipGraphExec_t exec = nullptr;
   e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
-  hipGraphDestroy(graph);
+  (void)hipGraphDestroy(graph);
   if (e != hipSuccess) {
     pf_set_error("pf_graph_capture_end: instantiate: %s", hipGetErrorString(e));
     return PF_ERR_HIP;
@@ -90,6 +90,6 @@ extern "C" int pf_graph_launch(void* graph_exec, void* stream) {
 }
 
 extern "C" int pf_graph_destroy(void* graph_exec) {
-  if (graph_exec) hipGraphExecDestroy((hipGraphExec_t)graph_exec);
+  if (graph_exec) (void)hipGraphExecDestroy((hipGraphExec_t)graph_exec);
   return PF_OK;
 }

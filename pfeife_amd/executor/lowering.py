@@ -111,6 +111,25 @@ class ParamStore:
                 out.append(self.kernels.fill(a, 0.0, used))
         return out
 
+    def grad_buffers(self):
+        """(buffer, used elements) of every fp32 gradient accumulator: whole arenas where the
+        gradients live in one, single tensors otherwise."""
+        out = []
+        slots = dict((i, a) for i, a in getattr(self, "_arena_slots", []))
+        done = set()
+        for i, launch in enumerate(self.zero):
+            if launch is None:
+                a = slots[i]
+                used = self._arena_used if a is self._arena else a.numel()
+                out.append((a, used))
+                done.add(a.data_ptr())
+        for p in self.params:
+            g = self._grads[id(p)]
+            base = g._base if g._base is not None else g
+            if base.data_ptr() not in done:
+                out.append((g, g.numel()))
+        return out
+
     def scale_grads_launches(self, factor):
         """Launches multiplying every gradient accumulator by `factor` (loss-scale removal)."""
         out = []
@@ -840,6 +859,11 @@ def lower_sdpa(L, node):
     Tk = k.shape[2]
     if k.shape != (Bn, H, Tk, hd) or v.shape[:3] != (Bn, H, Tk):
         raise Unsupported("attention with mismatched head layout %s %s %s" % (q.shape, k.shape, v.shape))
+    if causal and Tq != Tk:
+        # F.scaled_dot_product_attention aligns a non-square causal mask at the top-left corner
+        # (tril(0)); the attention and softmax kernels align it bottom-right (key j visible to
+        # query i iff j <= i + Tk - Tq, the decode convention).  They agree only when Tq == Tk.
+        raise Unsupported("is_causal attention with Tq=%d != Tk=%d" % (Tq, Tk))
     hv = v.shape[3]
     scale = float(scale) if scale is not None else 1.0 / math.sqrt(hd)
     Tkp = (Tk + 7) // 8 * 8
@@ -1601,11 +1625,16 @@ def lower_to(L, node):
 def lower_embedding(L, node):
     ids = L.arg(node.args[0])
     table = L.arg(node.args[1])
-    if _kw(node, 2, "padding_idx") is not None and False:
-        raise Unsupported("embedding with padding_idx")
+    pad = _kw(node, 2, "padding_idx")
+    if pad is not None and not isinstance(pad, int):
+        raise Unsupported("embedding with a non-constant padding_idx")
     if ids.dtype != torch.int64 or not ids.buf.is_contiguous() or not table.buf.is_contiguous():
         raise Unsupported("embedding expects contiguous int64 ids")
     vocab, dim = table.shape
+    # F.embedding's convention: None = no padding row, negative values count from the end
+    padding_idx = -1 if pad is None else (pad + vocab if pad < 0 else pad)
+    if padding_idx >= vocab or (pad is not None and padding_idx < 0):
+        raise Unsupported("embedding padding_idx out of range")
     n = ids.buf.numel()
     out_dtype = table.dtype  # autocast leaves embedding outputs in the table's dtype (fp32 residual stream)
     out = L.alloc(tuple(ids.shape) + (dim,), out_dtype)
@@ -1617,7 +1646,7 @@ def lower_embedding(L, node):
         if g is None or table.param is None:
             return
         gc = g if g.is_contiguous() else _compact(B, g)
-        B.emit(B.k.embedding_bwd(gc, ids.buf, L.params.grad(table.param), n, dim, vocab))
+        B.emit(B.k.embedding_bwd(gc, ids.buf, L.params.grad(table.param), n, dim, vocab, padding_idx))
 
     if table.req_grad:
         L.add_backward(bwd)

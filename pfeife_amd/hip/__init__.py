@@ -16,7 +16,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpfeife_hip.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 PF_F32, PF_F16, PF_BF16, PF_I64, PF_I32, PF_U8 = 0, 1, 2, 3, 4, 5
 ACT_NONE, ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU = 0, 1, 2, 3, 4
@@ -114,13 +114,18 @@ _SIGNATURES = {
     "pf_fill": [_P, _I, _F, _L, _P],
     "pf_adam_step": [_P, _I, _L, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double, _L,
                      _I, _P],
+    "pf_adam_step_scaled": [_P, _I, _L, ctypes.c_double, ctypes.c_double, ctypes.c_double, ctypes.c_double,
+                            ctypes.c_double, _I, _P, _P],
+    "pf_scale_by_state": [_P, _I, _P, _P, _I, _L, _P],
+    "pf_scaler_unscale": [_P, _L, _P, _P],
+    "pf_scaler_update": [_P, ctypes.c_double, ctypes.c_double, _I, _P],
     "pf_copy_strided": [_P, _I, POINTER(c_int64), _P, _I, POINTER(c_int64), POINTER(c_int64), _I, _I, _P],
     "pf_rope": [_P, _P, _I, _P, _P, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P],
     "pf_grad_accumulate_f32": [_P, _P, _I, _L, _P],
     "pf_split_gather": [_P, _P, _L, _L, _L, _P, _P],
     "pf_merge_scatter": [_P, _P, _L, _L, _L, _P, _P],
     "pf_embedding_fwd": [_P, _I, _P, _P, _I, _L, _L, _L, _P],
-    "pf_embedding_bwd": [_P, _I, _P, _P, _L, _L, _L, _P],
+    "pf_embedding_bwd": [_P, _I, _P, _P, _L, _L, _L, _L, _P],
 }
 _RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L], "pf_groupnorm_workspace": [_L, _L, _I],
             "pf_colsum_static_capacity": []}
@@ -465,6 +470,24 @@ class HipKernels:
         if rc != 0:
             raise RuntimeError("pf_adam_step failed: %s" % self.lib.pf_last_error().decode())
 
+    def adam_step_scaled(self, table, n_items, max_n, lr, beta1, beta2, eps, weight_decay, adamw, state, stream):
+        rc = self.lib.pf_adam_step_scaled(table.data_ptr(), n_items, max_n, lr, beta1, beta2, eps, weight_decay,
+                                          int(adamw), state.data_ptr(), stream)
+        if rc != 0:
+            raise RuntimeError("pf_adam_step_scaled failed: %s" % self.lib.pf_last_error().decode())
+
+    # -- dynamic loss scaling (state: float32[8] on the device) ----------------------------
+    def scale_by_state(self, src, state, dst, n):
+        return self._prep("pf_scale_by_state", (_ptr(src), _dt(src), _ptr(state), _ptr(dst), _dt(dst), n),
+                          (src, state, dst), n * (_es(src) + _es(dst)))
+
+    def scaler_unscale(self, grads, n, state):
+        return self._prep("pf_scaler_unscale", (_ptr(grads), n, _ptr(state)), (grads, state), 8 * n)
+
+    def scaler_update(self, state, growth_factor, backoff_factor, growth_interval):
+        return self._prep("pf_scaler_update", (_ptr(state), float(growth_factor), float(backoff_factor),
+                                               int(growth_interval)), (state,))
+
     def fill(self, dst, value, n):
         return self._prep("pf_fill", (_ptr(dst), _dt(dst), float(value), n), (dst,))
 
@@ -497,6 +520,6 @@ class HipKernels:
         args = (_ptr(table), _dt(table), _ptr(ids), _ptr(out), _dt(out), n_ids, dim, vocab)
         return self._prep("pf_embedding_fwd", args, (table, ids, out))
 
-    def embedding_bwd(self, dout, ids, dtable, n_ids, dim, vocab):
-        args = (_ptr(dout), _dt(dout), _ptr(ids), _ptr(dtable), n_ids, dim, vocab)
+    def embedding_bwd(self, dout, ids, dtable, n_ids, dim, vocab, padding_idx=-1):
+        args = (_ptr(dout), _dt(dout), _ptr(ids), _ptr(dtable), n_ids, dim, vocab, int(padding_idx))
         return self._prep("pf_embedding_bwd", args, (dout, ids, dtable))

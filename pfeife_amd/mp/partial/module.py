@@ -44,6 +44,13 @@ class _ExecError:
         self.exc = exc
 
 
+class _StepAborted(BaseException):
+    """Raised inside a parked micro-batch thread when the step it belongs to has failed."""
+
+
+_ABORT = object()
+
+
 class PartialRunner:
     def __init__(self, option: PipeOption = None, optimizer=None, kernels=None):
         """`kernels` is for tests of the host logic only (a kernel table double);
@@ -97,9 +104,27 @@ class PartialRunner:
                 print("Found %d graphs in the main module" % len(PartialModule._all_modules))
 
         self.reset()
+        self.results = []
+        self._parked = set()
+        try:
+            return self._run_step(args, kwargs)
+        except BaseException:
+            self._abort_parked()
+            raise
+
+    def _abort_parked(self):
+        """A failed step leaves the micro-batch threads that already handed their inputs over
+        parked inside the compiled model; wake them with an abort so that each one unwinds out of
+        exec_fn and is ready for the next step()."""
+        for bid in sorted(self._parked):
+            PartialModule._module_queues[bid].put(_ABORT)
+            self._return_queues[bid].get()
+        self._parked = set()
+
+    def _run_step(self, args, kwargs):
+        option = self.option
         pp = PartialModule._pp_modules[0] if PartialModule._pp_modules else None
         worker = self.worker
-        self.results = []
 
         # every micro-batch thread runs user code up to the compiled model, hands its
         # inputs to the worker and parks there
@@ -108,7 +133,9 @@ class PartialRunner:
             tok = self._return_queues[bid].get()
             if isinstance(tok, _ExecError):
                 raise tok.exc
-            if tok is not STEP_TOKEN:
+            if tok is STEP_TOKEN:
+                self._parked.add(bid)
+            else:
                 # exec_fn returned without reaching a pipelined graph: nothing to schedule for it
                 self.results.append(tok)
                 if pp is not None:
@@ -135,6 +162,7 @@ class PartialRunner:
         returned (loss computed, backward hooks fired)."""
         PartialModule._module_queues[batch_idx].put(None)
         ret = self._return_queues[batch_idx].get()
+        self._parked.discard(batch_idx)
         if isinstance(ret, _ExecError):
             raise ret.exc
         self.worker.finish_micro_batch(batch_idx)
@@ -320,7 +348,8 @@ class PartialModule(nn.Module):
             if torch.is_tensor(v):
                 worker.distribute_input(mb, i, v)
         runner._return_queues[mb].put(STEP_TOKEN)   # inputs are in place; main thread may schedule
-        self._module_queues[mb].get()               # parked until this micro-batch's outputs exist
+        if self._module_queues[mb].get() is _ABORT:  # parked until this micro-batch's outputs exist
+            raise _StepAborted()
         return self._outputs_for_user(mb, probe=False)
 
 

@@ -65,6 +65,15 @@ class StageWorker:
         self.graphs_ready = False
         self.steps_done = 0
         self.begin_graph = None
+        # dynamic loss scaling: {scale, growth tracker, found_inf, completed steps, 4 scratch} on the device
+        self.dyn_scale = option.loss_scale == "dynamic"
+        self.scaler_state = None
+        if self.dyn_scale:
+            if not hasattr(kernels, "scaler_unscale"):
+                raise RuntimeError("dynamic loss scaling needs the HIP kernel table")
+            self.scaler_state = torch.tensor([option.init_scale] + [0.0] * 7, dtype=torch.float32,
+                                             device=self.device)
+            self._one = torch.ones((), dtype=torch.float32, device=self.device)
 
     # -- graph ---------------------------------------------------------------------
     def set_partition_graph(self, part_graph, example_inputs):
@@ -292,6 +301,11 @@ class StageWorker:
         if g.shape != buf.shape:
             raise RuntimeError("loss gradient of output %d has shape %s, expected %s"
                                % (out_idx, tuple(g.shape), tuple(buf.shape)))
+        if self.dyn_scale:
+            if not (g.device == buf.device and g.dtype.is_floating_point):
+                g = g.to(device=buf.device, dtype=buf.dtype)
+            self.kernels.scale_by_state(g.contiguous(), self.scaler_state, buf, g.numel())(self.stream())
+            return
         scale = self.option.loss_scale
         if g.device == buf.device and g.is_contiguous() and buf.is_contiguous() and g.dtype.is_floating_point:
             if scale != 1.0:
@@ -307,6 +321,9 @@ class StageWorker:
         slot = self.mbs[mb]
         for oi, buf in slot.loss_grads.items():
             if oi not in slot.grad_seen:
+                if self.dyn_scale and buf.dim() == 0:
+                    self.kernels.scale_by_state(self._one, self.scaler_state, buf, 1)(self.stream())
+                    continue
                 self.kernels.fill(buf, self.option.loss_scale if buf.dim() == 0 else 0.0, buf.numel())(self.stream())
 
     def run_job(self, stage, mb, is_fwd):
@@ -325,8 +342,34 @@ class StageWorker:
                 cls = get_optimizer_cls(self.option.optimizer_type)
                 self.optimizer = cls(params, **self.option.optimizer_kwargs)
 
+    def scaler_scale(self):
+        """Current loss scale (synchronises; for logging and tests)."""
+        return float(self.scaler_state[0].item()) if self.dyn_scale else float(self.option.loss_scale)
+
+    def _dynamic_optimizer_step(self, opt):
+        """GradScaler.unscale_ + step + update on the device (pfeife/mp/worker.py:1432-1436): the
+        gradients are unscaled in place and checked; an Adam/AdamW step reads the overflow flag
+        itself, any other optimizer is skipped after one host read of the flag."""
+        s = self.stream()
+        key = (len(self.params.params), len(self.params.zero))
+        if getattr(self, "_unscale_key", None) != key:
+            self._unscale = [self.kernels.scaler_unscale(buf, n, self.scaler_state)
+                             for buf, n in self.params.grad_buffers()]
+            self._unscale_key = key
+        for launch in self._unscale:
+            launch(s)
+        if opt is not None:
+            if self._fused_adam_applicable(opt):
+                self._fused_adam_step(opt, scaled=True)
+            elif float(self.scaler_state[2].item()) == 0.0:
+                opt.step()
+        o = self.option
+        self.kernels.scaler_update(self.scaler_state, o.growth_factor, o.backoff_factor, o.growth_interval)(s)
+
     def optimizer_step(self):
         opt = self.optimizer
+        if self.dyn_scale:
+            return self._dynamic_optimizer_step(opt)
         if self.option.loss_scale != 1.0:   # gradients leave the step unscaled, with or without an optimizer
             key = (len(self.params.params), len(self.params.zero))
             if getattr(self, "_unscale_key", None) != key:
@@ -359,7 +402,7 @@ class StageWorker:
                     return False
         return True
 
-    def _fused_adam_step(self, opt):
+    def _fused_adam_step(self, opt, scaled=False):
         cache = self.__dict__.setdefault("_adam_tables", {})
         s = self.stream()
         for gi, g in enumerate(opt.param_groups):
@@ -382,8 +425,15 @@ class StageWorker:
             step = int(opt.state[params[0]]["step"].item()) + 1
             b1, b2 = g["betas"]
             table, n_items, max_n = ent[1]
-            self.kernels.adam_step(table, n_items, max_n, float(g["lr"]), float(b1), float(b2), float(g["eps"]),
-                                   float(g["weight_decay"]), step, type(opt) is torch.optim.AdamW, s)
+            if scaled:
+                # skipped on overflow; the bias corrections use the device's count of completed steps
+                # (the host-side `step` entries below count attempted steps)
+                self.kernels.adam_step_scaled(table, n_items, max_n, float(g["lr"]), float(b1), float(b2),
+                                              float(g["eps"]), float(g["weight_decay"]),
+                                              type(opt) is torch.optim.AdamW, self.scaler_state, s)
+            else:
+                self.kernels.adam_step(table, n_items, max_n, float(g["lr"]), float(b1), float(b2), float(g["eps"]),
+                                       float(g["weight_decay"]), step, type(opt) is torch.optim.AdamW, s)
             for p in params:
                 opt.state[p]["step"] += 1
 

@@ -86,10 +86,20 @@ class PipeOption:
         self.use_fsdp = get("use_fsdp", False)
         self.mixed_precision = _PRECISIONS.get(get("mixed_precision", None), get("mixed_precision", None))
 
-        # extension: static loss scale applied ONCE, to the gradients entering the last stage, and
-        # removed again before the optimizer step (the reference's GradScaler scales at every
-        # stage, so its stage i of L sees S^(L-i); see the design notes)
-        self.loss_scale = float(get("loss_scale", 1.0))
+        # Loss scale, applied ONCE, to the gradients entering the last stage, and removed again
+        # before the optimizer step (the reference's GradScaler scales at every stage, so its
+        # stage i of L sees S^(L-i)).  "dynamic": torch.amp.GradScaler's rule (worker.py:133-145)
+        # kept on the device: overflowing steps are skipped and halve the scale, `growth_interval`
+        # clean steps double it.  A number: that static scale.  Default: dynamic for fp16 mixed
+        # precision (where the reference's scaler matters), 1.0 otherwise.
+        ls = get("loss_scale", None)
+        if ls is None:
+            ls = "dynamic" if self.mixed_precision is torch.float16 else 1.0
+        self.loss_scale = "dynamic" if isinstance(ls, str) and ls.lower() == "dynamic" else float(ls)
+        self.init_scale = float(get("init_scale", 65536.0))
+        self.growth_factor = float(get("growth_factor", 2.0))
+        self.backoff_factor = float(get("backoff_factor", 0.5))
+        self.growth_interval = int(get("growth_interval", 2000))
 
         self.no_side_effect = get("no_side_effect", False)
         self.no_io_cache = get("no_io_cache", False)
@@ -155,6 +165,8 @@ class PipeOption:
             no_io_cache=args.no_io_cache,
             single_comm_thread=args.single_comm_thread,
         )
+        if getattr(args, "loss_scale", None) is not None:
+            option_kwargs["loss_scale"] = args.loss_scale
         if device_map is not None:
             option_kwargs["device_map"] = device_map
 
@@ -200,4 +212,6 @@ class PipeOption:
         add("--single_comm_thread", action="store_true", help="use single communication thread for all devices.")
         add("--old_ver", action="store_true", help="apply the above three actions.")
         add("--print_graph", action="store_true")
+        add("--loss_scale", default=None,
+            help="'dynamic' (GradScaler's rule, the default with --mixed_precision fp16) or a fixed number")
         return parser

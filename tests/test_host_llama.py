@@ -73,3 +73,46 @@ def test_mixed_precision(mixed, tol):
     for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
         rel = (p.grad - q.grad).norm() / (q.grad.norm() + 1e-12)
         assert rel <= tol, (n, float(rel))
+
+
+def test_causal_attention_with_unequal_lengths_is_rejected():
+    """F.scaled_dot_product_attention(is_causal=True) with Tq != Tk masks top-left; the kernels
+    mask bottom-right, so the lowering must refuse instead of computing something else."""
+    from pfeife_amd.executor.lowering import Unsupported
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife, partial_compiler
+
+    class Cross(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Linear(16, 16)
+            self.b = torch.nn.Linear(16, 16)
+
+        def forward(self, x, ctx):
+            q = self.a(x).view(x.shape[0], -1, 2, 8).transpose(1, 2)
+            k = self.a(ctx).view(ctx.shape[0], -1, 2, 8).transpose(1, 2)
+            o = F.scaled_dot_product_attention(q, k, k, is_causal=True)
+            return self.b(o.transpose(1, 2).reshape(x.shape[0], -1, 16))
+
+    torch._dynamo.reset()
+    net_states._reset_state_for_tests()
+    initialize_pfeife(device="cpu")
+    torch.manual_seed(0)
+    model = Cross()
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=["b"],
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = PartialRunner(option, kernels=OracleKernels("cpu"))
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(x, ctx):
+        loss = cmodel(x, ctx).float().square().mean()
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    with pytest.raises(Exception) as err:
+        runner.step(torch.randn(4, 4, 16), torch.randn(4, 6, 16))
+    chain, e = [], err.value
+    while e is not None:
+        chain.append(e)
+        e = e.__cause__ or e.__context__
+    assert any(isinstance(c, Unsupported) and "is_causal" in str(c) for c in chain) or "is_causal" in str(err.value)

@@ -169,3 +169,123 @@ def test_static_loss_scale_is_applied_once_and_removed():
         grads.append({n: p.grad.clone() for n, p in model.named_parameters()})
     for n in grads[0]:
         assert torch.equal(grads[0][n], grads[1][n]), n
+
+
+def test_scaler_rule_of_the_kernel_oracle_matches_torch_gradscaler():
+    """scaler_unscale / scaler_update of the kernel oracle against torch.amp.GradScaler on the CPU,
+    over a sequence with overflows and growth."""
+    from oracle.kernels_oracle import OracleKernels
+
+    k = OracleKernels("cpu")
+    ref = torch.amp.GradScaler("cpu", init_scale=1024.0, growth_factor=2.0, backoff_factor=0.5, growth_interval=3)
+    state = torch.tensor([1024.0, 0.0, 0.0, 0.0])
+    p = torch.nn.Parameter(torch.zeros(4))
+    opt = torch.optim.SGD([p], lr=1.0)
+    done = 0
+    for step, bad in enumerate([False, False, True, False, False, False, True, True, False, False, False, False]):
+        ref.scale(torch.zeros(1))          # GradScaler creates its scale tensor on first use
+        g = torch.tensor([1.0, -2.0, 0.5, 4.0]) * float(ref.get_scale())
+        if bad:
+            g[1] = float("inf")
+        p.grad = g.clone()
+        before = p.detach().clone()
+        ref.step(opt)
+        ref.update()
+        mine = g.clone()
+        k.scaler_unscale(mine, 4, state)(None)
+        assert float(state[2]) == (1.0 if bad else 0.0)
+        if not bad:
+            assert torch.equal(mine, torch.tensor([1.0, -2.0, 0.5, 4.0]))
+            done += 1
+        assert torch.equal(p.detach(), before) == bad   # torch skipped exactly the overflowing steps
+        k.scaler_update(state, 2.0, 0.5, 3)(None)
+        assert float(state[0]) == float(ref.get_scale()), (step, float(state[0]), float(ref.get_scale()))
+        assert float(state[3]) == done and float(state[2]) == 0.0
+
+
+def test_dynamic_loss_scale_skips_overflowing_steps():
+    """PipeOption(loss_scale="dynamic"): gradients leave the step unscaled, a step whose gradients
+    overflow changes no parameter and halves the scale, clean steps grow it every growth_interval."""
+    from pfeife_amd.mp import partial_compiler
+
+    torch.manual_seed(0)
+    model = VisionTransformer(CFG)
+    ref = copy.deepcopy(model)
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=["blocks.2"],
+                        optimizer=dict(type="sgd", lr=0.1), loss_scale="dynamic", init_scale=256.0,
+                        growth_interval=2)
+    runner = make_runner(option)
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+    poison = [False]
+
+    def fn(x, y):
+        loss = crit(cmodel(x).float(), y)
+        (loss * float("inf") if poison[0] else loss).backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    x, y = torch.randn(4, 3, 32, 32, generator=g), torch.randint(0, 10, (4,), generator=g)
+    w = runner.worker
+    assert w.scaler_scale() == 256.0
+    runner.step(x, y)                                   # clean step 1
+    # same step without scaling on the reference copy: identical gradients (power-of-two scale)
+    ropt = torch.optim.SGD(ref.parameters(), lr=0.1)
+    for xs, ys in zip(x.chunk(2), y.chunk(2)):
+        crit(ref(xs), ys).backward()
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+    ropt.step()
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.detach() - q.detach()).abs().max() <= 1e-5 * q.detach().abs().max() + 1e-7, n
+    assert w.scaler_scale() == 256.0
+    poison[0] = True
+    before = {n: p.detach().clone() for n, p in model.named_parameters()}
+    runner.step(x, y)                                   # overflow: skipped, scale halves
+    for n, p in model.named_parameters():
+        assert torch.equal(p.detach(), before[n]), n
+    assert w.scaler_scale() == 128.0
+    poison[0] = False
+    runner.step(x, y)
+    runner.step(x, y)                                   # two clean steps: scale doubles
+    assert w.scaler_scale() == 256.0
+    assert float(w.scaler_state[3]) == 3.0
+
+
+def test_failed_step_releases_parked_micro_batches():
+    """exec_fn raising for a later micro-batch (or after the model returned) must not leave the
+    earlier micro-batch threads parked: the error reaches the caller and the next step() runs."""
+    from pfeife_amd.mp import partial_compiler
+
+    torch.manual_seed(0)
+    model = VisionTransformer(CFG)
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=["blocks.2"],
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = make_runner(option)
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+    fail = [None]
+
+    def fn(x, y):
+        if fail[0] == "before" and float(y[0]) < 0:
+            raise ValueError("bad labels")
+        loss = crit(cmodel(x).float(), y.abs())
+        if fail[0] == "after" and float(y[0]) < 0:
+            raise ValueError("bad loss")
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    x, y = torch.randn(4, 3, 32, 32, generator=g), torch.randint(1, 10, (4,), generator=g)
+    good = [float(v) for v in runner.step(x, y)]
+    ybad = y.clone()
+    ybad[2] = -ybad[2]                        # first sample of micro-batch 1
+    for mode in ("before", "after"):
+        fail[0] = mode
+        with pytest.raises(ValueError):
+            runner.step(x, ybad)
+        fail[0] = None
+        again = [float(v) for v in runner.step(x, y)]
+        assert again == good, mode

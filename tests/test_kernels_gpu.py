@@ -383,6 +383,15 @@ def test_embedding(hip, oracle, dtype):
     r = both(hip, oracle, "embedding_bwd", dict(dout=dout, ids=ids, dtable=rnd((vocab, dim), F32, 4)), ["dtable"],
              n_ids=n, dim=dim, vocab=vocab)
     close(r["dtable"], 1e-5, 1e-5)
+    # padding row keeps its old contents; ids spread over a vocabulary that is no multiple of the
+    # rows one wavefront owns, with the last row hit; same summation order as index_add: exact
+    vocab2 = 1003
+    ids2 = torch.randint(0, vocab2, (n,), generator=g)
+    ids2[5], ids2[17], ids2[100] = vocab2 - 1, 7, 7
+    r = both(hip, oracle, "embedding_bwd", dict(dout=dout, ids=ids2, dtable=rnd((vocab2, dim), F32, 5)), ["dtable"],
+             n_ids=n, dim=dim, vocab=vocab2, padding_idx=7)
+    assert torch.equal(*r["dtable"])
+    assert torch.equal(r["dtable"][0][7], rnd((vocab2, dim), F32, 5)[7])
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16, F32])
@@ -519,3 +528,56 @@ def test_transpose_16bit_register_path(hip, oracle, dtype):
                  cols=cols)
         assert torch.equal(r["dst"][0][:, :rows], src[:, :cols].t())
         assert torch.equal(r["dst"][1][:, :rows], src[:, :cols].t())
+
+
+def test_loss_scaler_kernels(hip, oracle):
+    """Dynamic loss scaling kept on the device: scale_by_state, scaler_unscale (power-of-two scale:
+    bit-exact, sets found_inf on inf/NaN anywhere in a large buffer) and scaler_update over a
+    sequence with two overflows against the oracle (itself pinned to torch.amp.GradScaler)."""
+    n = 256 * 1024 * 3 + 5
+    state0 = torch.tensor([4096.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0])
+    src = rnd((n,), F16, 1)
+    r = both(hip, oracle, "scale_by_state", dict(src=src, state=state0.clone(), dst=torch.zeros(n, dtype=F32)),
+             ["dst"], n=n)
+    assert torch.equal(*r["dst"])
+    g = rnd((n,), F32, 2, scale=4096.0)
+    r = both(hip, oracle, "scaler_unscale", dict(grads=g.clone(), state=state0.clone()), ["grads", "state"], n=n)
+    assert torch.equal(*r["grads"]) and torch.equal(*r["state"]) and float(r["state"][0][2]) == 0.0
+    for pos, bad in ((0, float("inf")), (n - 1, float("nan")), (n // 2 + 3, float("-inf"))):
+        gb = g.clone()
+        gb[pos] = bad
+        r = both(hip, oracle, "scaler_unscale", dict(grads=gb, state=state0.clone()), ["state"], n=n)
+        assert torch.equal(*r["state"]) and float(r["state"][0][2]) == 1.0, pos
+    dev, cpu = state0.clone().cuda(), state0.clone()
+    for found in (0, 0, 1, 0, 0, 0, 1, 1, 0, 0):
+        dev[2] = float(found)
+        cpu[2] = float(found)
+        hip.run("scaler_update", dev, 2.0, 0.5, 3)
+        oracle.run("scaler_update", cpu, 2.0, 0.5, 3)
+        torch.cuda.synchronize()
+        assert torch.equal(dev.cpu(), cpu), (found, dev.cpu(), cpu)
+
+
+def test_adam_step_scaled_skips_on_overflow_and_counts_steps_on_device(hip):
+    """pf_adam_step_scaled reads found_inf and the completed-step count from the scaler state:
+    with found_inf set nothing changes; otherwise it equals pf_adam_step at step = count + 1."""
+    n = 100003
+    mk = lambda: [rnd((n,), F32, 3).cuda(), rnd((n,), F32, 4).cuda(), torch.zeros(n, device="cuda"),
+                  torch.zeros(n, device="cuda")]
+    ref, got = mk(), mk()
+    state = torch.tensor([1.0, 0.0, 0.0, 2.0, 0.0, 0.0, 0.0, 0.0], device="cuda")          # two steps completed -> step 3
+    s = torch.cuda.current_stream().cuda_stream
+    tr, _, _ = hip.adam_table([ref[0]], [ref[1]], [ref[2]], [ref[3]])
+    tg, ni, mx = hip.adam_table([got[0]], [got[1]], [got[2]], [got[3]])
+    hip.adam_step(tr, ni, mx, 1e-3, 0.9, 0.999, 1e-8, 0.01, 3, True, s)
+    state[2] = 1.0
+    before = [t.clone() for t in got]
+    hip.adam_step_scaled(tg, ni, mx, 1e-3, 0.9, 0.999, 1e-8, 0.01, True, state, s)
+    torch.cuda.synchronize()
+    for a, b in zip(got, before):
+        assert torch.equal(a, b)
+    state[2] = 0.0
+    hip.adam_step_scaled(tg, ni, mx, 1e-3, 0.9, 0.999, 1e-8, 0.01, True, state, s)
+    torch.cuda.synchronize()
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)

@@ -219,6 +219,13 @@ def test_byte_movers_match_tensor_split_and_embedding(oracle):
     oracle.run("embedding_bwd", d, ids, dt, n_ids=6, dim=6, vocab=20)
     assert torch.equal(o, e.detach())
     torch.testing.assert_close(dt, table.grad)
+    # padding row: torch keeps its gradient at zero
+    table.grad = None
+    F.embedding(ids, table, padding_idx=3).backward(d)
+    dt = torch.zeros(20, 6)
+    oracle.run("embedding_bwd", d, ids, dt, n_ids=6, dim=6, vocab=20, padding_idx=3)
+    torch.testing.assert_close(dt, table.grad)
+    assert float(dt[3].abs().max()) == 0.0 and float(dt[7].abs().max()) > 0.0
 
 
 def test_streaming(oracle):

@@ -325,10 +325,11 @@ def test_vit_g_block_share_head_dim_88(mixed):
 def test_unet_stage_sdxl_style(mixed):
     """The SDXL UNet-stage configuration at reduced width: ResNet blocks (GroupNorm 32, 3x3 convs, time
     embedding), spatial transformers with self- and cross-attention to 77 context tokens,
-    GEGLU; MSE loss against an N(0,1) target computed in user code.  In fp16 the user code
-    scales the loss (the reference script wraps it in a GradScaler,
-    bench_models/models/train_sdxl.py:1310-1452): the mean-squared-error gradients are ~1e-5
-    and would otherwise sit in fp16's subnormal range on both sides of the comparison."""
+    GEGLU; MSE loss against an N(0,1) target computed in user code.  In fp16 the loss is scaled
+    (the reference script wraps it in a GradScaler, bench_models/models/train_sdxl.py:1310-1452):
+    the mean-squared-error gradients are ~1e-5 and would otherwise sit in fp16's subnormal range.
+    Here the scale is PipeOption's static loss_scale, applied and removed by the library; the
+    eager side scales its loss and divides its gradients."""
     loss_scale = 4096.0 if mixed == "fp16" else 1.0
     import torch.nn.functional as F
 
@@ -347,7 +348,7 @@ def test_unet_stage_sdxl_style(mixed):
     ctx = torch.randn(B, 77, cfg.context_dim, generator=g)
     target = torch.randn(B, cfg.channels, hw, hw, generator=g)
     option = PipeOption(device_cnt=1, batch_cnt=2, batch_size=2, mixed_precision=mixed,
-                        optimizer=dict(type="sgd", lr=0.0))
+                        optimizer=dict(type="sgd", lr=0.0), loss_scale=loss_scale)
     runner = _fresh_runner(option)
     model.cuda()
     cmodel = torch.compile(model, backend=partial_compiler)
@@ -355,7 +356,7 @@ def test_unet_stage_sdxl_style(mixed):
     def fn(h, t, c, y):
         out = cmodel(h, t, c)
         loss = F.mse_loss(out.float(), y.float())
-        (loss * loss_scale).backward()
+        loss.backward()
         return loss.detach()
 
     runner.set_exec_fn(fn)
@@ -375,6 +376,8 @@ def test_unet_stage_sdxl_style(mixed):
         loss = F.mse_loss(out.float(), target[sl].float())
         (loss * loss_scale).backward()
         want.append(loss.detach())
+    for p in ref.parameters():
+        p.grad.div_(loss_scale)
     ltol = 1e-5 if mixed is None else 2e-2
     for a, b in zip(losses, want):
         assert abs(float(a) - float(b)) <= ltol * abs(float(b)), (float(a), float(b))
@@ -450,6 +453,76 @@ def test_fused_adam_matches_torch_optimizer(opt_type, wd):
         real = results[1][1][n] > 1e-10
         torch.testing.assert_close(results[0][0][n][real], results[1][0][n][real], rtol=2e-5, atol=2e-6, msg=n)
         torch.testing.assert_close(results[0][1][n][real], results[1][1][n][real], rtol=1e-4, atol=1e-9, msg=n)
+
+
+def test_dynamic_loss_scale_matches_torch_gradscaler_and_adam():
+    """PipeOption(loss_scale="dynamic") with the fused Adam step against torch.amp.GradScaler +
+    torch.optim.Adam on an eager copy of the model: five steps, the third with an overflowing loss
+    (skipped by both, scale halved), growth every two clean steps.  Parameters, both moments and
+    the scale must agree (fp32 path, so the only difference is summation order)."""
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=2, mlp_dim=128, num_classes=10)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(8, 3, 32, 32, generator=g).cuda()
+    y = torch.randint(0, 10, (8,), generator=g).cuda()
+    torch.manual_seed(0)
+    model = VisionTransformer(cfg)
+    ref = copy.deepcopy(model).cuda()
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=4, split_points=["blocks.1"],
+                        optimizer=dict(type="adam", lr=1e-2), loss_scale="dynamic", init_scale=1024.0,
+                        growth_interval=2)
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+    poison = [False]
+
+    def fn(px, labels):
+        loss = crit(cmodel(px).float(), labels)
+        (loss * float("inf") if poison[0] else loss).backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    ropt = torch.optim.Adam(ref.parameters(), lr=1e-2)
+    scaler = torch.amp.GradScaler("cuda", init_scale=1024.0, growth_interval=2)
+    for step in range(5):
+        poison[0] = step == 2
+        runner.step(x, y)
+        ropt.zero_grad(set_to_none=False)
+        for xs, ys in zip(x.chunk(2), y.chunk(2)):
+            loss = crit(ref(xs), ys)
+            scaler.scale(loss * float("inf") if poison[0] else loss).backward()
+        scaler.step(ropt)
+        scaler.update()
+        torch.cuda.synchronize()
+        assert runner.worker.scaler_scale() == float(scaler.get_scale()), step
+        for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+            # Adam turns a gradient that is pure rounding noise into +-lr steps: compare where the
+            # second moment says the gradient is real
+            real = ropt.state[q]["exp_avg_sq"] > 1e-10 if q in ropt.state and len(ropt.state[q]) else None
+            a, b = (p.detach(), q.detach()) if real is None else (p.detach()[real], q.detach()[real])
+            torch.testing.assert_close(a, b, rtol=2e-4, atol=2e-5,
+                                       msg=lambda m: "%s step %d: %s" % (n, step, m))
+    assert float(runner.worker.scaler_state[3]) == 4.0        # four completed steps, one skipped
+    opt = runner.worker.optimizer
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        torch.testing.assert_close(opt.state[p]["exp_avg"], ropt.state[q]["exp_avg"], rtol=2e-3, atol=1e-6, msg=n)
+        torch.testing.assert_close(opt.state[p]["exp_avg_sq"], ropt.state[q]["exp_avg_sq"], rtol=2e-3, atol=1e-9,
+                                   msg=n)
+
+
+def test_fp16_defaults_to_dynamic_loss_scaling():
+    """mixed_precision="fp16" without an explicit loss_scale runs the device-side scaler (the
+    reference wraps fp16 training in a GradScaler, pfeife/mp/worker.py:133-145)."""
+    from pfeife_amd.bench_models.vit import ViTConfig
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=4, mlp_dim=128, num_classes=16)
+    m, r, l, rl, runner = _run_vit(cfg, 8, 2, "blocks.1", "fp16")
+    assert runner.worker.dyn_scale and runner.worker.scaler_state is not None
+    _check(m, r, l, rl, "fp16")     # gradients leave the step unscaled
 
 
 def test_split_then_merge_round_trip_on_device():
