@@ -57,6 +57,13 @@ int pf_graph_capture_begin(void* stream);
 int pf_graph_capture_end(void* stream, void** graph_exec_out);
 int pf_graph_launch(void* graph_exec, void* stream);
 int pf_graph_destroy(void* graph_exec);
+/* Orders stream `to` after everything issued on stream `from` so far (event record + wait).
+ * A job forks launches that nothing later in the job reads (weight and bias gradients, which
+ * only the optimizer consumes; torch.autograd orders them the same way only by accident of
+ * its queue, pfeife/mp/worker.py:1585-1587) onto a side stream and joins it at the end of the
+ * job, so that they fill the compute units the input-gradient chain leaves idle.  Inside a
+ * capture the fork and join become graph edges.  Both streams at the default priority. */
+int pf_stream_order_after(void* from, void* to);
 
 /* ---- dense contractions (MFMA) -------------------------------------------
  * One descriptor covers every matrix product a stage executes:
@@ -156,6 +163,23 @@ int pf_layernorm_bwd(const void* dy, int dy_dtype, const void* x, int x_dtype, c
                      const float* mean, const float* rstd, const void* dx_add, int add_dtype, void* dx,
                      int dx_dtype, float* dgamma_acc, float* dbeta_acc, float* workspace, int64_t rows,
                      int64_t d, int defer_reduce, void* stream);
+/* Normalisation backward with the follow-up work of a transformer block folded in.  Besides
+ * dx (as above, + dx_add) it can write dx_lp, a second copy of dx in fp16/bf16: the form in
+ * which the matrix products of the preceding layer read this gradient (torch autocast makes
+ * that copy with a separate aten::_to_copy).  With want_colsum it also leaves the column
+ * sums of dx_lp, i.e. the bias gradient of the linear layer whose output (+ residual) was
+ * normalised (aten::sum in linear's backward).  mean == NULL selects RMSNorm.  Parameter
+ * gradients and column sums are left as per-workgroup partial rows for
+ * pf_colreduce_finalize_batch: workspace holds pf_norm_bwd_partials(rows) rows of
+ * (want_colsum ? 3 : 2) * d floats, laid out [dgamma | dbeta | colsum].  want_colsum needs
+ * 16-byte aligned operands, d % 8 == 0 and d <= 2048 (PF_ERR_UNSUPPORTED otherwise). */
+typedef struct pf_norm_bwd_desc {
+  const void* dy; const void* x; const float* gamma; const float* mean; const float* rstd;
+  const void* dx_add; void* dx; void* dx_lp; float* workspace;
+  int64_t rows, d;
+  int32_t dy_dtype, x_dtype, add_dtype, dx_dtype, dx_lp_dtype, want_wgrad, want_colsum, reserved;
+} pf_norm_bwd_desc;
+int pf_norm_bwd_fused(const pf_norm_bwd_desc* desc, void* stream);
 /* RMSNorm: y = x * rsqrt(mean(x^2) + eps) * gamma.  rstd fp32 [rows].
  * Replaces the pow/mean/rsqrt/mul chain (or aten::rms_norm) of Llama-style blocks. */
 int pf_rmsnorm_fwd(const void* x, int x_dtype, const float* gamma, void* y, int y_dtype, float* rstd,

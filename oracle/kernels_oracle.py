@@ -209,6 +209,30 @@ class OracleKernels:
 
         return launch
 
+    def norm_bwd_fused(self, dy, x, gamma, mean, rstd, dx_add, dx, dx_lp, ws, rows, d, want_wgrad, want_colsum):
+        """Norm backward plus a 16-bit copy of dx and (want_colsum) the column sums of that copy;
+        one partial row set [dgamma | dbeta | colsum] in ws."""
+        inner = self.layernorm_bwd(dy, x, gamma, mean, rstd, dx_add, dx, None, None, None, rows, d, defer=0,
+                                   _rms=mean is None)
+
+        def launch(stream=None):
+            inner(None)
+            out = _rows(dx, rows, d, d)
+            if dx_lp is not None:
+                _rows(dx_lp, rows, d, d).copy_(out.to(dx_lp.dtype))
+            n = 3 if want_colsum else 2
+            if want_wgrad:
+                DY = _rows(dy, rows, d, d).float()
+                X = _rows(x, rows, d, d).float()
+                rs = _flat(rstd, rows).float()[:, None]
+                mu = torch.zeros_like(rs) if mean is None else _flat(mean, rows).float()[:, None]
+                _flat(ws, n * d)[:d].copy_((DY * (X - mu) * rs).sum(dim=0))
+                _flat(ws, n * d)[d:2 * d].copy_(DY.sum(dim=0))
+            if want_colsum:
+                _flat(ws, n * d)[2 * d:].copy_(_rows(dx_lp, rows, d, d).float().sum(dim=0))
+
+        return launch
+
     def groupnorm_workspace(self, B, C, groups):
         return B * 2 * C + B * groups * 2
 

@@ -18,6 +18,8 @@
 // Q, K, V, O and their gradients are [B, H, T, hd] tensors addressed with element
 // strides (batch, head, token) and unit stride along hd, so heads can live inside a
 // packed qkv projection and the output can be token-major.
+#include <mutex>
+
 #include "pf_common.h"
 
 namespace {
@@ -506,6 +508,356 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
   }
 }
 
+
+// =================================================================================
+// Short sequences (Tq, Tk <= SHORT_T, e.g. ViT's 197 or 257 tokens): the two operands a workgroup
+// sweeps over (K and V, or Q and dO) are loaded into LDS ONCE, whole, in their natural
+// [token][hd] layout; after a single barrier every wavefront runs its tile loop without
+// any further synchronisation.  Operands the MFMA needs transposed (V^T, K^T, Q^T, dO^T)
+// are read from the natural layout with the transposing LDS read (ds_read_b64_tr_b16),
+// so no transposed copy is made.
+// =================================================================================
+constexpr int SHORT_T = 288;   // 2 operands x 288 rows x (96 + 8) x 2 bytes = 117 KB of the 160 KB
+#define PF_LDS16(T) __attribute__((address_space(3))) T*
+typedef short short4v_t __attribute__((ext_vector_type(4)));
+
+// Transposing LDS read.  The 16 lanes of a group each name an 8-byte chunk (4 elements);
+// group lane j must point at row k0 + j/4, columns n0 + 4*(j%4); lane i of the group then
+// receives the four elements (k0 .. k0+3, column n0 + i).
+__device__ __forceinline__ uint2 lds_read_tr(const uint16_t* p) {
+  const short4v_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PF_LDS16(short4v_t))(uintptr_t)p);
+  return __builtin_bit_cast(uint2, r);
+}
+
+// A operand X^T[row = hd index][k = token] for the 16-token chunk starting at `t0` of a
+// natural [token][LD] tile, hd rows o32 .. o32+31, with the token permutation of pack8():
+// element i of the lane <-> token t0 + 8*(i/4) + 4*(lane/32) + (i%4)
+template <int LD>
+__device__ __forceinline__ uint4 frag_tr(const uint16_t* s, int t0, int o32, int lane) {
+  const int g = lane >> 4, j = lane & 15;
+  const uint16_t* p = s + (t0 + 4 * (g >> 1) + (j >> 2)) * LD + o32 + 16 * (g & 1) + 4 * (j & 3);
+  const uint2 lo = lds_read_tr(p), hi = lds_read_tr(p + 8 * LD);
+  return make_uint4(lo.x, lo.y, hi.x, hi.y);
+}
+
+template <int DT>
+__device__ __forceinline__ void unpack8(const uint4& r, float (&v)[8]) {
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    if constexpr (DT == PF_F16) {
+      v[2 * k] = pf_f16_bits_to_f32((uint16_t)(w[k] & 0xffffu));
+      v[2 * k + 1] = pf_f16_bits_to_f32((uint16_t)(w[k] >> 16));
+    } else {
+      v[2 * k] = __uint_as_float(w[k] << 16);
+      v[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+    }
+  }
+}
+
+// Two whole [T][hd] operands of one head -> LDS [rows][HD + 8] each (rows past T and hd
+// chunks past hd are zero); 256 threads, eight 16-byte loads in flight per thread
+template <int HD>
+__device__ __forceinline__ void load_heads(const uint16_t* x, int64_t x_st, const uint16_t* y, int64_t y_st, int T,
+                                           int hd, int rows, uint16_t* sx, uint16_t* sy, int tid) {
+  constexpr int VPR = HD / 8, LD = HD + 8;
+  const int n = rows * VPR;
+  for (int e0 = 0; e0 < n; e0 += 256 * 4) {
+    uint4 vx[4], vy[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = e0 + i * 256 + tid;
+      const int t = e / VPR, c = (e % VPR) * 8;
+      vx[i] = e < n ? load_row8(x, x_st, t, T, c, hd) : make_uint4(0, 0, 0, 0);
+      vy[i] = e < n ? load_row8(y, y_st, t, T, c, hd) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = e0 + i * 256 + tid;
+      if (e < n) {
+        *(uint4*)(sx + (e / VPR) * LD + (e % VPR) * 8) = vx[i];
+        *(uint4*)(sy + (e / VPR) * LD + (e % VPR) * 8) = vy[i];
+      }
+    }
+  }
+}
+
+// forward: workgroup = 128 queries of one (batch, head), wavefront = 32 of them; keys in steps of 32
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_fwd_short_kernel(const AttnArgs a, int rows) {
+  constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
+  extern __shared__ __align__(16) uint16_t smem[];
+  uint16_t* sK = smem;
+  uint16_t* sV = smem + rows * LD;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int q0 = blockIdx.x * 128 + wave * 32;
+  const int qi = q0 + (lane & 31);
+  const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;
+
+  uint4 qf[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) qf[c] = load_row8(Q, a.q_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
+  load_heads<HD>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
+                 sV, tid);
+  __syncthreads();
+  if (q0 >= a.Tq) return;   // this wavefront has no query row (no barrier follows)
+
+  float16_t oacc[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[o][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const int k_end = a.causal ? min(a.Tk, min(q0 + 31, a.Tq - 1) + shift + 1) : a.Tk;
+  for (int k0 = 0; k0 < k_end; k0 += 32) {
+    float16_t s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const uint4 kf = *(const uint4*)(sK + (k0 + (lane & 31)) * LD + c * 16 + (lane >> 5) * 8);
+      s = M32<DT>::run(kf, qf[c], s);
+    }
+    const bool masked = (k0 + 32 > a.Tk) || (a.causal && k0 + 31 > q0 + shift);
+    float mx = m;
+    if (masked) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kj = k0 + acc_row(r, lane);
+        const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
+        s[r] = ok ? s[r] : -INFINITY;
+        mx = fmaxf(mx, s[r]);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const bool dead = (mx == -INFINITY);
+    const float moff = dead ? 0.f : -mx * sc;
+    const float alpha = dead ? 1.f : __builtin_amdgcn_exp2f((m - mx) * sc);
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = __builtin_amdgcn_exp2f(fmaf(s[r], sc, moff));
+      s[r] = p;
+      psum += p;
+    }
+    l = l * alpha + psum;
+    m = mx;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int o = 0; o < NO; ++o)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[o][r] *= alpha;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint4 pf = pack8<DT>(s, 8 * j);
+#pragma unroll
+      for (int o = 0; o < NO; ++o) oacc[o] = M32<DT>::run(frag_tr<LD>(sV, k0 + 16 * j, o * 32, lane), pf, oacc[o]);
+    }
+  }
+  l += __shfl_xor(l, 32, 64);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  if (qi < a.Tq) {
+    uint16_t* O = a.out + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd)
+          *(uint2*)(O + h0) = make_uint2(M32<DT>::pack(oacc[o][4 * g] * inv, oacc[o][4 * g + 1] * inv),
+                                         M32<DT>::pack(oacc[o][4 * g + 2] * inv, oacc[o][4 * g + 3] * inv));
+      }
+    if ((lane >> 5) == 0) a.lse[((int64_t)bh) * a.Tq + qi] = (l > 0.f) ? (m * sc + log2f(l)) / LOG2E : -INFINITY;
+  }
+}
+
+// dQ (and delta = rowsum(dO * O), which the dK/dV kernel launched after this one reads)
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_dq_short_kernel(const AttnArgs a, float* delta_out, int rows) {
+  constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
+  extern __shared__ __align__(16) uint16_t smem[];
+  uint16_t* sK = smem;
+  uint16_t* sV = smem + rows * LD;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int q0 = blockIdx.x * 128 + wave * 32;
+  const int qi = q0 + (lane & 31);
+  const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t* DO = a.d_o + b * a.do_sb + h * a.do_sh;
+  const uint16_t* OO = a.o + b * a.o_sb + h * a.o_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;
+
+  uint4 qf[NC], dof[NC];
+  float dlt = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int h0 = c * 16 + (lane >> 5) * 8;
+    qf[c] = load_row8(Q, a.q_st, qi, a.Tq, h0, a.hd);
+    dof[c] = load_row8(DO, a.do_st, qi, a.Tq, h0, a.hd);
+    const uint4 of = load_row8(OO, a.o_st, qi, a.Tq, h0, a.hd);
+    float x[8], y[8];
+    unpack8<DT>(dof[c], x);
+    unpack8<DT>(of, y);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) dlt += x[k] * y[k];
+  }
+  dlt += __shfl_xor(dlt, 32, 64);
+  const bool qok = qi < a.Tq;
+  if (qok && (lane >> 5) == 0) delta_out[(int64_t)bh * a.Tq + qi] = dlt;
+  const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
+  load_heads<HD>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
+                 sV, tid);
+  __syncthreads();
+  if (q0 >= a.Tq) return;
+
+  float16_t acc[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[o][r] = 0.f;
+  const int k_end = a.causal ? min(a.Tk, min(q0 + 31, a.Tq - 1) + shift + 1) : a.Tk;
+  for (int k0 = 0; k0 < k_end; k0 += 32) {
+    float16_t s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int off = (k0 + (lane & 31)) * LD + c * 16 + (lane >> 5) * 8;
+      s = M32<DT>::run(*(const uint4*)(sK + off), qf[c], s);
+      dp = M32<DT>::run(*(const uint4*)(sV + off), dof[c], dp);
+    }
+    const bool masked = (k0 + 32 > a.Tk) || (a.causal && k0 + 31 > q0 + shift);
+    if (masked) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kj = k0 + acc_row(r, lane);
+        const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
+        const float p = ok ? __builtin_amdgcn_exp2f(s[r] * sc - lse2) : 0.f;
+        s[r] = p * (dp[r] - dlt);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(s[r] * sc - lse2) * (dp[r] - dlt);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint4 dsf = pack8<DT>(s, 8 * j);
+#pragma unroll
+      for (int o = 0; o < NO; ++o) acc[o] = M32<DT>::run(frag_tr<LD>(sK, k0 + 16 * j, o * 32, lane), dsf, acc[o]);
+    }
+  }
+  if (qok) {
+    uint16_t* DQ = a.dq + b * a.dq_sb + h * a.dq_sh + (int64_t)qi * a.dq_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd)
+          *(uint2*)(DQ + h0) = make_uint2(M32<DT>::pack(acc[o][4 * g] * a.scale, acc[o][4 * g + 1] * a.scale),
+                                          M32<DT>::pack(acc[o][4 * g + 2] * a.scale, acc[o][4 * g + 3] * a.scale));
+      }
+  }
+}
+
+// dK/dV: workgroup = 128 keys, wavefront = 32 of them; queries in steps of 32
+template <int DT, int HD>
+__global__ __launch_bounds__(256) void attn_dkv_short_kernel(const AttnArgs a, int rows) {
+  constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
+  extern __shared__ __align__(16) uint16_t smem[];
+  uint16_t* sQ = smem;
+  uint16_t* sDO = smem + rows * LD;
+  float* sLse = (float*)(smem + 2 * rows * LD);
+  float* sDelta = sLse + rows;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const int kw0 = blockIdx.x * 128 + wave * 32;
+  const int kj = kw0 + (lane & 31);
+  const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;
+  const bool kok = kj < a.Tk;
+
+  uint4 kf[NC], vf[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    kf[c] = load_row8(K, a.k_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
+    vf[c] = load_row8(V, a.v_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
+  }
+  for (int i = tid; i < rows; i += 256) {
+    // rows past the end: Q and dO rows are zero, lse = +inf makes their P exactly zero
+    sLse[i] = i < a.Tq ? a.lse[(int64_t)bh * a.Tq + i] * LOG2E : INFINITY;
+    sDelta[i] = i < a.Tq ? a.delta[(int64_t)bh * a.Tq + i] : 0.f;
+  }
+  load_heads<HD>(a.q + b * a.q_sb + h * a.q_sh, a.q_st, a.d_o + b * a.do_sb + h * a.do_sh, a.do_st, a.Tq, a.hd, rows,
+                 sQ, sDO, tid);
+  __syncthreads();
+  if (kw0 >= a.Tk) return;
+
+  float16_t dk[NO], dv[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[o][r] = dv[o][r] = 0.f;
+  int q_begin = 0;
+  if (a.causal) q_begin = max(0, kw0 - shift) / 32 * 32;   // queries i with i + shift >= kw0 see this wavefront's keys
+  for (int q0 = q_begin; q0 < a.Tq; q0 += 32) {
+    const bool masked = a.causal && (kw0 + 31 > q0 + shift);
+    float16_t s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int off = (q0 + (lane & 31)) * LD + c * 16 + (lane >> 5) * 8;
+      s = M32<DT>::run(*(const uint4*)(sQ + off), kf[c], s);
+      dp = M32<DT>::run(*(const uint4*)(sDO + off), vf[c], dp);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int ql = q0 + acc_row(r, lane);
+      float p = __builtin_amdgcn_exp2f(s[r] * sc - sLse[ql]);
+      if (masked && kj > ql + shift) p = 0.f;
+      s[r] = p;
+      dp[r] = p * (dp[r] - sDelta[ql]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint4 pf = pack8<DT>(s, 8 * j);
+      const uint4 dsf = pack8<DT>(dp, 8 * j);
+#pragma unroll
+      for (int o = 0; o < NO; ++o) {
+        dv[o] = M32<DT>::run(frag_tr<LD>(sDO, q0 + 16 * j, o * 32, lane), pf, dv[o]);
+        dk[o] = M32<DT>::run(frag_tr<LD>(sQ, q0 + 16 * j, o * 32, lane), dsf, dk[o]);
+      }
+    }
+  }
+  if (kok) {
+    uint16_t* DK = a.dk + b * a.dk_sb + h * a.dk_sh + (int64_t)kj * a.dk_st;
+    uint16_t* DV = a.dv + b * a.dv_sb + h * a.dv_sh + (int64_t)kj * a.dv_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd) {
+          *(uint2*)(DK + h0) = make_uint2(M32<DT>::pack(dk[o][4 * g] * a.scale, dk[o][4 * g + 1] * a.scale),
+                                          M32<DT>::pack(dk[o][4 * g + 2] * a.scale, dk[o][4 * g + 3] * a.scale));
+          *(uint2*)(DV + h0) = make_uint2(M32<DT>::pack(dv[o][4 * g], dv[o][4 * g + 1]),
+                                          M32<DT>::pack(dv[o][4 * g + 2], dv[o][4 * g + 3]));
+        }
+      }
+  }
+}
+
 bool strides_ok(const void* p, int64_t sb, int64_t sh, int64_t st) {
   return pf_aligned(p, 16) && sb % 8 == 0 && sh % 8 == 0 && st % 8 == 0;
 }
@@ -545,6 +897,40 @@ AttnArgs make_args(const pf_attn_desc* d) {
 
 }  // namespace
 
+// Launch of a short-sequence kernel with `lds` bytes of dynamic LDS (above 64 KB the kernel is
+// opted in once per instantiation and device).
+template <typename K, typename... Args>
+int launch_short(K kern, dim3 grid, size_t lds, hipStream_t st, Args... args) {
+  if (lds > 64 * 1024) {
+    static std::mutex mu;
+    static bool raised[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!raised[dev]) {
+      const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) {
+        pf_set_error("pf_attention: cannot raise dynamic LDS: %s", hipGetErrorString(e));
+        return PF_ERR_HIP;
+      }
+      raised[dev] = true;
+    }
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, args...);
+  return PF_OK;
+}
+
+#define PF_ATTN_SHORT(KERNEL, rc, grid, lds, st, dt, hd, ...)                                            \
+  do {                                                                                                 \
+    if (dt == PF_F16) {                                                                                \
+      if (hd <= 64) rc = launch_short(KERNEL<PF_F16, 64>, grid, (lds)(64), st, __VA_ARGS__);            \
+      else rc = launch_short(KERNEL<PF_F16, 96>, grid, (lds)(96), st, __VA_ARGS__);                     \
+    } else {                                                                                           \
+      if (hd <= 64) rc = launch_short(KERNEL<PF_BF16, 64>, grid, (lds)(64), st, __VA_ARGS__);           \
+      else rc = launch_short(KERNEL<PF_BF16, 96>, grid, (lds)(96), st, __VA_ARGS__);                    \
+    }                                                                                                  \
+  } while (0)
+
 #define PF_ATTN_DISPATCH(KERNEL, grid, st, a, dt, hd)                                          \
   do {                                                                                         \
     if (dt == PF_F16) {                                                                        \
@@ -563,7 +949,14 @@ extern "C" int pf_attention_fwd(const pf_attn_desc* d, void* stream) {
              "pf_attention_fwd: bad output operand");
   AttnArgs a = make_args(d);
   const dim3 grid((unsigned)((d->Tq + 127) / 128), (unsigned)(d->B * d->H));
-  PF_ATTN_DISPATCH(attn_fwd_kernel, grid, (hipStream_t)stream, a, d->dtype, d->hd);
+  if (d->Tq <= SHORT_T && d->Tk <= SHORT_T) {
+    const int rows = (d->Tk + 31) / 32 * 32;
+    auto lds = [rows](int HD) { return (size_t)2 * rows * (HD + 8) * 2; };
+    PF_ATTN_SHORT(attn_fwd_short_kernel, rc, grid, lds, (hipStream_t)stream, d->dtype, d->hd, a, rows);
+    if (rc != PF_OK) return rc;
+  } else {
+    PF_ATTN_DISPATCH(attn_fwd_kernel, grid, (hipStream_t)stream, a, d->dtype, d->hd);
+  }
   PF_CHECK_LAUNCH("pf_attention_fwd");
   return PF_OK;
 }
@@ -582,10 +975,22 @@ extern "C" int pf_attention_bwd(const pf_attn_desc* d, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   AttnArgs ad = a;
   if (d->dtype == PF_BF16) ad.causal |= 0x100;  // dtype flag for the delta kernel
-  const int64_t rows = (int64_t)d->B * d->H * d->Tq;
-  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, ad, d->delta);
   const dim3 gq((unsigned)((d->Tq + 127) / 128), (unsigned)(d->B * d->H));
   const dim3 gk((unsigned)((d->Tk + 127) / 128), (unsigned)(d->B * d->H));
+  if (d->Tq <= SHORT_T && d->Tk <= SHORT_T) {
+    // dQ first: it also leaves delta = rowsum(dO * O) for the dK/dV kernel
+    const int rows_k = (d->Tk + 31) / 32 * 32, rows_q = (d->Tq + 31) / 32 * 32;
+    auto lds_q = [rows_k](int HD) { return (size_t)2 * rows_k * (HD + 8) * 2; };
+    auto lds_k = [rows_q](int HD) { return (size_t)2 * rows_q * (HD + 8) * 2 + (size_t)rows_q * 8; };
+    PF_ATTN_SHORT(attn_dq_short_kernel, rc, gq, lds_q, st, d->dtype, d->hd, a, d->delta, rows_k);
+    if (rc != PF_OK) return rc;
+    PF_ATTN_SHORT(attn_dkv_short_kernel, rc, gk, lds_k, st, d->dtype, d->hd, a, rows_q);
+    if (rc != PF_OK) return rc;
+    PF_CHECK_LAUNCH("pf_attention_bwd");
+    return PF_OK;
+  }
+  const int64_t rows = (int64_t)d->B * d->H * d->Tq;
+  hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, ad, d->delta);
   PF_ATTN_DISPATCH(attn_dkv_kernel, gk, st, a, d->dtype, d->hd);
   PF_ATTN_DISPATCH(attn_dq_kernel, gq, st, a, d->dtype, d->hd);
   PF_CHECK_LAUNCH("pf_attention_bwd");

@@ -134,14 +134,24 @@ template <int W, int NV>
 __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt, const void* x, int x_dt,
                                                        const float* gamma, const float* mean, const float* rstd,
                                                        const void* dx_add, int add_dt, void* dx, int dx_dt,
-                                                       float* ws, int64_t rows, int64_t d, int rms, int want_wgrad) {
+                                                       float* ws, int64_t rows, int64_t d, int rms, int want_wgrad,
+                                                       void* dx_lp, int lp_dt, int want_colsum) {
+  // dx_lp: optional second copy of dx in a 16-bit dtype (what the next matrix product reads);
+  // want_colsum: also leave the column sums of that copy's values (the bias gradient of the
+  // layer that produced x) as a third partial row.  Partial rows per block: [dgamma, dbeta]
+  // or, with want_colsum, [dgamma, dbeta, colsum].
   __shared__ float red[4][64 * W];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float pg[NV][W], pb[NV][W];
+  constexpr int NS = (NV * W <= 32) ? NV : 1;   // column sums only exist on the register-cached variants
+  float pg[NV][W], pb[NV][W], ps[NS][W];
 #pragma unroll
   for (int i = 0; i < NV; ++i)
 #pragma unroll
     for (int k = 0; k < W; ++k) pg[i][k] = pb[i][k] = 0.f;
+#pragma unroll
+  for (int i = 0; i < NS; ++i)
+#pragma unroll
+    for (int k = 0; k < W; ++k) ps[i][k] = 0.f;
 
   constexpr bool CACHE = (NV * W <= 32);   // keep the row's dy and x in registers between the two passes
   for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < rows; row += (int64_t)gridDim.x * 4) {
@@ -220,20 +230,31 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
           }
         }
         st_vec<W>(dx, base + c, dx_dt, o);
+        if (dx_lp) {
+          st_vec<W>(dx_lp, base + c, lp_dt, o);
+          if constexpr (NS == NV) {
+            if (want_colsum) {
+#pragma unroll
+              for (int k = 0; k < W; ++k) ps[i][k] += pf_round_to(lp_dt, o[k]);
+            }
+          }
+        }
       }
     }
   }
-  if (!want_wgrad) return;  // uniform over the block
+  if (!want_wgrad && !want_colsum) return;  // uniform over the block
   // reduce the 4 wavefronts through LDS, then one partial row per block:
-  // ws layout [gridDim.x][2][d]
-  float* wrow = ws + (int64_t)blockIdx.x * 2 * d;
+  // ws layout [gridDim.x][2 or 3][d]
+  const int nrows = want_colsum ? 3 : 2;
+  float* wrow = ws + (int64_t)blockIdx.x * nrows * d;
 #pragma unroll
-  for (int which = 0; which < 2; ++which) {
+  for (int which = 0; which < 3; ++which) {
+    if (which < 2 ? !want_wgrad : !want_colsum) continue;   // uniform over the block
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       __syncthreads();
 #pragma unroll
-      for (int k = 0; k < W; ++k) red[wave][lane * W + k] = which ? pb[i][k] : pg[i][k];
+      for (int k = 0; k < W; ++k) red[wave][lane * W + k] = which == 0 ? pg[i][k] : (which == 1 ? pb[i][k] : ps[i < NS ? i : 0][k]);
       __syncthreads();
       if (wave == 0) {
         const int64_t c = ((int64_t)lane + i * 64) * W;
@@ -465,20 +486,25 @@ int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, voi
 
 int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* gamma, const float* mean,
              const float* rstd, const void* dx_add, int add_dt, void* dx, int dx_dt, float* dgamma, float* dbeta,
-             float* ws, int64_t rows, int64_t d, int rms, int defer, hipStream_t st, const char* name) {
+             float* ws, int64_t rows, int64_t d, int rms, int defer, hipStream_t st, const char* name,
+             void* dx_lp = nullptr, int lp_dt = PF_F16, int want_colsum = 0) {
   PF_REQUIRE(rows >= 0 && d > 0, "%s: bad shape", name);
   if (rows == 0) return PF_OK;
   PF_REQUIRE(dy && x && gamma && rstd && dx, "%s: null pointer", name);
   PF_REQUIRE(rms || mean, "%s: mean required", name);
   PF_REQUIRE(pf_is_float_dtype(dy_dt) && pf_is_float_dtype(x_dt) && pf_is_float_dtype(dx_dt), "%s: bad dtype", name);
   const int want = (dgamma || dbeta || defer) ? 1 : 0;
-  if (want) PF_REQUIRE(ws, "%s: workspace required for parameter gradients", name);
+  if (want || want_colsum) PF_REQUIRE(ws, "%s: workspace required for parameter gradients", name);
   const int blocks = norm_bwd_blocks(rows);
   const bool v = vec_ok(dy, dy_dt, d) && vec_ok(x, x_dt, d) && vec_ok(dx, dx_dt, d) && vec_ok(gamma, PF_F32, d) &&
-                 vec_ok(dx_add, dx_add ? add_dt : PF_F32, d);
+                 vec_ok(dx_add, dx_add ? add_dt : PF_F32, d) && vec_ok(dx_lp, lp_dt, d);
+  if (want_colsum && !(v && d <= 64 * 8 * 4)) {
+    pf_set_error("%s: the fused column sum needs 16-byte aligned operands and d <= 2048", name);
+    return PF_ERR_UNSUPPORTED;
+  }
 #define PF_NB(W, NV)                                                                                          \
   hipLaunchKernelGGL((norm_bwd_kernel<W, NV>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, mean, \
-                     rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want)
+                     rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want, dx_lp, lp_dt, want_colsum)
   if (v) {
     if (d <= 64 * 8 * 2) PF_NB(8, 2);
     else if (d <= 64 * 8 * 4) PF_NB(8, 4);
@@ -525,6 +551,17 @@ __global__ __launch_bounds__(256) void colreduce_finalize_batch_kernel(const pf_
     for (int q = 0; q < 8; ++q) t += red[q][cl];
     it.acc[c] += t;
   }
+}
+
+extern "C" int pf_norm_bwd_fused(const pf_norm_bwd_desc* n, void* stream) {
+  PF_REQUIRE(n != nullptr, "pf_norm_bwd_fused: null descriptor");
+  PF_REQUIRE(!n->dx_lp || n->dx_lp_dtype == PF_F16 || n->dx_lp_dtype == PF_BF16,
+             "pf_norm_bwd_fused: the second copy of dx is fp16 or bf16");
+  PF_REQUIRE(!n->want_colsum || n->dx_lp, "pf_norm_bwd_fused: column sums are taken over the 16-bit copy");
+  return norm_bwd(n->dy, n->dy_dtype, n->x, n->x_dtype, n->gamma, n->mean, n->rstd, n->dx_add, n->add_dtype, n->dx,
+                  n->dx_dtype, nullptr, nullptr, n->workspace, n->rows, n->d, n->mean == nullptr ? 1 : 0,
+                  n->want_wgrad ? 1 : 0, (hipStream_t)stream, "pf_norm_bwd_fused", n->dx_lp, n->dx_lp_dtype,
+                  n->want_colsum ? 1 : 0);
 }
 
 extern "C" int pf_norm_bwd_partials(int64_t rows) { return norm_bwd_blocks(rows < 1 ? 1 : rows); }

@@ -258,9 +258,15 @@ class StageProgram:
         for launch in self.fwd:
             launch(stream)
 
-    def run_backward(self, stream):
+    def run_backward(self, stream, side=None, issue=None):
+        """`side`/`issue`: a second stream and the kernel table's fork/join issue loop for the
+        launches marked `side` (weight and bias gradients); without them everything runs in
+        list order on `stream`."""
         if self.bwd_graph is not None:
             self.bwd_graph(stream)
+            return
+        if side and issue is not None:
+            issue(self.bwd, stream, side)
             return
         for launch in self.bwd:
             launch(stream)
@@ -283,25 +289,70 @@ class BwdCtx:
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
         self._transposed = {}  # (data_ptr, rows, cols, ld) -> transposed copy made earlier in this job
+        self._side_params = set()   # parameters whose gradient a side launch of this job writes
+        self._join_next = False
+        # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
+        # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
+        self._lp = {}
 
     def emit(self, launch):
+        if self._join_next:
+            launch.after_side = True
+            self._join_next = False
+        self.out.append(launch)
+
+    def param_grad(self, param):
+        """fp32 gradient accumulator of `param` for a launch on the main stream: if a side launch
+        of this job has written it (a parameter used twice, e.g. tied embeddings), the next
+        launch waits for the side stream first."""
+        if id(param) in self._side_params:
+            self._join_next = True
+        return self.L.params.grad(param)
+
+    def emit_side(self, launch, param=None):
+        """A launch whose results nothing later in this job reads, except the batched reduction
+        at its end: parameter-gradient work, which only the optimizer consumes.  The executor may
+        run it on a second stream beside the input-gradient chain.  Its inputs (the finished
+        gradient of a forward value, saved activations, job-private temporaries) are never
+        written again within the job, and all such launches share one stream, so two writers of
+        one parameter gradient (tied weights) keep their order."""
+        launch.side = True
+        if param is not None:
+            self._side_params.add(id(param))
         self.out.append(launch)
 
     def transposed(self, t, rows, cols, ld):
-        """[cols, rows] copy of the 16-bit matrix t (made once per job and matrix: several products
-        that reduce over the same token rows share it)."""
+        """[cols, rows] copy of the 16-bit matrix t (made once per job and matrix: several
+        weight-gradient products that reduce over the same token rows share it)."""
         key = (t.data_ptr(), rows, cols, ld)
         tt = self._transposed.get(key)
         if tt is None:
             tt = self.temp((cols, rows), t.dtype)
-            self.emit(self.k.transpose_cast(t, ld, tt, rows, rows, cols))
+            self.emit_side(self.k.transpose_cast(t, ld, tt, rows, rows, cols))
             self._transposed[key] = tt
         return tt
 
+    def register_lp(self, full, copy, colsum=None):
+        """`copy` holds the values of the fp32 gradient `full` in the compute dtype; `colsum`:
+        (ws, offset, n_partials, stride) of partial rows whose sum is copy's column sum."""
+        self._lp[full.data_ptr()] = (full.untyped_storage().data_ptr(), copy, colsum)
+
+    def _written(self, t):
+        """Gradient buffer t is about to be written: side copies of anything in its storage are stale."""
+        if self._lp and t is not None:
+            st = t.untyped_storage().data_ptr()
+            for key in [k for k, v in self._lp.items() if v[0] == st]:
+                del self._lp[key]
+
     def colsum_into(self, x, rows, cols, ld, acc):
         """acc[c] += sum_r x[r, c] (bias gradient), reduction finished at the end of the job."""
+        for _, copy, cs in self._lp.values():
+            if cs is not None and copy.data_ptr() == x.data_ptr() and copy.numel() == rows * cols and ld == cols:
+                ws, off, nb, stride = cs     # the kernel that produced x already summed its columns
+                self.reduces.append((ws, off, nb, stride, cols, acc))
+                return
         ws = self.temp((self.k.colreduce_workspace(rows, cols),), torch.float32)
-        self.emit(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
+        self.emit_side(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
         self.reduces.append((ws, 0, self.k.colsum_partials(rows), cols, cols, acc))
 
     def new_like(self, like, private=False):
@@ -327,7 +378,8 @@ class BwdCtx:
     def _own_base_grad(self, val, zero_fill):
         """Make sure `val` (kind base) has a private, writable gradient buffer."""
         if val.param is not None:
-            return self.L.params.grad(val.param)
+            return self.param_grad(val.param)
+        self._written(val.grad)
         if val.grad is None:
             val.grad = self.new_like(val.buf, val.boundary)
             val.grad_shared = False
@@ -355,10 +407,15 @@ class BwdCtx:
     def grad_target(self, val):
         """-> (dst, prev): write the NEW TOTAL gradient of `val` into dst; prev is the
         total so far (None: nothing yet; `prev is dst`: accumulate in place)."""
+        dst, prev = self._grad_target(val)
+        self._written(dst)
+        return dst, prev
+
+    def _grad_target(self, val):
         if not val.req_grad:
             raise RuntimeError("gradient requested for a value that does not require one: %r" % val)
         if val.kind == "view":
-            dst_b, prev_b = self.grad_target(val.base)
+            dst_b, prev_b = self._grad_target(val.base)
             self._pending[id(val)] = dst_b
             return val.view_fn(dst_b), (None if prev_b is None else val.view_fn(prev_b))
         if val.kind == "part":
@@ -370,7 +427,7 @@ class BwdCtx:
                 return region, region
             return region, None
         if val.param is not None:
-            g = self.L.params.grad(val.param)  # AccumulateGrad: always += into the fp32 accumulator
+            g = self.param_grad(val.param)  # AccumulateGrad: always += into the fp32 accumulator
             return g, g
         if val.grad is None:
             return self.new_like(val.buf, val.boundary), None
@@ -451,6 +508,9 @@ class BwdCtx:
         """t as a row-major matrix of `dtype` (cast / compact into a temp when needed)."""
         if t.dtype == dtype and as_matrix(t) is not None:
             return t
+        hit = self._lp.get(t.data_ptr())
+        if hit is not None and hit[1].dtype == dtype and hit[1].numel() == t.numel() and t.is_contiguous():
+            return hit[1].view(t.shape)
         tmp = self.temp(t.shape, dtype)
         self.copy(t, tmp)
         return tmp
@@ -537,7 +597,9 @@ class Lowerer:
         for fn in reversed(prog.backward_fns):
             fn(B)
         if B.reduces:
-            prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
+            fin = self.kernels.colreduce_finalize_batch(B.reduces)
+            fin.after_side = True    # reads the partial sums the side launches leave
+            prog.bwd.append(fin)
         prog.input_grads = []
         for v in prog.inputs:
             if isinstance(v, Val) and v.req_grad and v.param is None:
@@ -691,6 +753,10 @@ def lower_linear(L, node):
     L.emit(L.kernels.gemm(xm, w_cd, out, **kw))
     req = x.req_grad or w.req_grad or (b is not None and b.req_grad) or (res is not None and res.req_grad)
     outv = Val(out, req_grad=req, name=out_node.name)
+    if L.mixed and out_dtype == torch.float32 and act == ACT_NONE:
+        # backward reads this value's gradient as a 16-bit matrix (and sums its columns for the
+        # bias): whoever produces that gradient may write it in that form as well
+        outv.lp_grad = dict(colsum=b is not None and b.req_grad and b.param is not None, cols=N)
     if act != ACT_NONE:
         outv.preact = (act, h)
     if out_node is not node:
@@ -721,10 +787,11 @@ def lower_linear(L, node):
                 # transposes cost what the faster product saves
                 dy_t = B.transposed(dy, M, N, ld_dy)
                 x_t = B.transposed(xm, M, K, lda)
-                B.emit(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1))
+                B.emit_side(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1),
+                            w.param)
             else:
-                B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
-                                b_trans=1, beta=1))
+                B.emit_side(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K,
+                                     a_trans=1, b_trans=1, beta=1), w.param)
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:
@@ -817,17 +884,31 @@ def lower_layer_norm(L, node, rms=False):
                 raise Unsupported("normalisation backward into a non-contiguous gradient")
         else:
             dst, prev = B.temp(x.shape, x.dtype), None
-        if rms:
-            B.emit(B.k.rmsnorm_bwd(g, x.buf, g32, rstd, prev, dst, None, ws, rows, d, defer=1 if want else 0))
-        else:
-            B.emit(B.k.layernorm_bwd(g, x.buf, g32, mean, rstd, prev, dst, None, None, ws, rows, d,
-                                     defer=1 if want else 0))
-        if want:
+        lp_info = getattr(x, "lp_grad", None)
+        if (lp_info is not None and x.req_grad and L.mixed and dst.dtype == torch.float32 and d % 8 == 0
+                and lp_info["cols"] == d and hasattr(B.k, "norm_bwd_fused")):
+            # the layer before x reads this gradient as a 16-bit matrix and sums its columns for
+            # its bias: written here, while the values are in registers
+            want_cs = bool(lp_info["colsum"]) and d <= 2048
+            stride = (3 if want_cs else 2) * d
             nb = B.k.norm_bwd_partials(rows)
+            ws = B.temp((nb * stride,), torch.float32) if (want or want_cs) else None
+            lp = B.temp(x.shape, L.cd)
+            B.emit(B.k.norm_bwd_fused(g, x.buf, g32, mean, rstd, prev, dst, lp, ws, rows, d, want, want_cs))
+            B.register_lp(dst, lp, (ws, 2 * d, nb, stride) if want_cs else None)
+        else:
+            stride = 2 * d
+            nb = B.k.norm_bwd_partials(rows) if want else 0
+            if rms:
+                B.emit(B.k.rmsnorm_bwd(g, x.buf, g32, rstd, prev, dst, None, ws, rows, d, defer=1 if want else 0))
+            else:
+                B.emit(B.k.layernorm_bwd(g, x.buf, g32, mean, rstd, prev, dst, None, None, ws, rows, d,
+                                         defer=1 if want else 0))
+        if want:
             if dgamma is not None:
-                B.reduces.append((ws, 0, nb, 2 * d, d, dgamma))
+                B.reduces.append((ws, 0, nb, stride, d, dgamma))
             if dbeta is not None:
-                B.reduces.append((ws, d, nb, 2 * d, d, dbeta))
+                B.reduces.append((ws, d, nb, stride, d, dbeta))
         if x.req_grad:
             B.commit(x, dst)
 
@@ -1028,7 +1109,7 @@ def lower_conv2d(L, node):
         dy = B.matrix_in(gm_, cd)
         _, _, ld_dy = as_matrix(dy)
         if w.req_grad and w.param is not None:
-            B.emit(B.k.gemm(dy, cols, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
+            B.emit(B.k.gemm(dy, cols, B.param_grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
                             b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
@@ -1106,7 +1187,7 @@ def _lower_conv_same(L, x, w, b, k):
             return
         dy = _grad_nhwc(B, g, cd).reshape(M, O)
         if w.req_grad and w.param is not None:
-            wg = L.params.grad(w.param)
+            wg = B.param_grad(w.param)
             if k == 1:
                 B.emit(B.k.gemm(dy, cols, wg, M=O, N=Kc, K=M, lda=O, ldb=Kc, ldc=Kc, a_trans=1, b_trans=1, beta=1))
             else:
@@ -1646,7 +1727,7 @@ def lower_embedding(L, node):
         if g is None or table.param is None:
             return
         gc = g if g.is_contiguous() else _compact(B, g)
-        B.emit(B.k.embedding_bwd(gc, ids.buf, L.params.grad(table.param), n, dim, vocab, padding_idx))
+        B.emit(B.k.embedding_bwd(gc, ids.buf, B.param_grad(table.param), n, dim, vocab, padding_idx))
 
     if table.req_grad:
         L.add_backward(bwd)

@@ -71,7 +71,7 @@ class Val:
     """A tensor value of a stage program."""
 
     __slots__ = ("buf", "req_grad", "kind", "base", "view_fn", "param", "grad", "grad_shared", "written",
-                 "partial_only", "tiled", "name", "preact", "grad_is_preact", "pending_act", "boundary")
+                 "partial_only", "tiled", "name", "preact", "grad_is_preact", "pending_act", "boundary", "lp_grad")
 
     def __init__(self, buf, req_grad=False, kind="base", base=None, view_fn=None, param=None, name=""):
         self.buf = buf
@@ -88,6 +88,7 @@ class Val:
         self.name = name
         self.preact = None        # (act, pre-activation buffer) when this value is act(linear(...)) fused in a GEMM
         self.grad_is_preact = False
+        self.lp_grad = None       # dict(colsum, cols) when backward reads this value's gradient as a 16-bit matrix
         self.boundary = False     # stage input produced by another stage: its gradient outlives the backward job
         self.pending_act = None   # (act, source value) when this is the not-yet-applied gate of a gated MLP
 

@@ -61,6 +61,15 @@ class GemmDesc(Structure):
     ]
 
 
+class NormBwdDesc(Structure):
+    """Mirror of `pf_norm_bwd_desc` in include/pfeife_hip.h."""
+
+    _fields_ = ([(n, c_void_p) for n in ("dy", "x", "gamma", "mean", "rstd", "dx_add", "dx", "dx_lp", "workspace")]
+                + [("rows", c_int64), ("d", c_int64)]
+                + [(n, c_int32) for n in ("dy_dtype", "x_dtype", "add_dtype", "dx_dtype", "dx_lp_dtype", "want_wgrad",
+                                          "want_colsum", "reserved")])
+
+
 class AttnDesc(Structure):
     """Mirror of `pf_attn_desc` in include/pfeife_hip.h."""
 
@@ -79,11 +88,13 @@ _SIGNATURES = {
     "pf_graph_capture_begin": [_P],
     "pf_graph_capture_end": [_P, POINTER(c_void_p)],
     "pf_graph_launch": [_P, _P],
+    "pf_stream_order_after": [_P, _P],
     "pf_graph_destroy": [_P],
     "pf_gemm": [POINTER(GemmDesc), _P],
     "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
     "pf_attention_fwd": [POINTER(AttnDesc), _P],
     "pf_attention_bwd": [POINTER(AttnDesc), _P],
+    "pf_norm_bwd_fused": [POINTER(NormBwdDesc), _P],
     "pf_layernorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _F, _P],
     "pf_layernorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _L, _L, _I, _P],
     "pf_rmsnorm_fwd": [_P, _I, _P, _P, _I, _P, _L, _L, _F, _P],
@@ -223,16 +234,46 @@ class HipKernels:
     def run(self, name, *a, **kw):
         getattr(self, name)(*a, **kw)(current_stream_ptr())
 
-    def capture(self, launches, stream):
+    def issue(self, launches, stream, side=None):
+        """Issue prepared launches on `stream`.  Launches marked `side` (their results are read by
+        nothing later in the list except launches marked `after_side`) go to the stream `side`,
+        each ordered after the main-stream work issued before it; the main stream is ordered after
+        the side stream before an `after_side` launch and at the end of the list."""
+        if not side:
+            for launch in launches:
+                launch(stream)
+            return
+        order = self.lib.pf_stream_order_after
+        forked = False      # side already waits for everything issued on the main stream so far
+        dirty = False       # the side stream has work the main stream has not waited for
+        for launch in launches:
+            if getattr(launch, "side", False):
+                if not forked:
+                    if order(stream, side) != 0:
+                        raise RuntimeError("fork: %s" % self.lib.pf_last_error().decode())
+                    forked = True
+                launch(side)
+                dirty = True
+                continue
+            if dirty and getattr(launch, "after_side", False):
+                if order(side, stream) != 0:
+                    raise RuntimeError("join: %s" % self.lib.pf_last_error().decode())
+                dirty = False
+            launch(stream)
+            forked = False
+        if dirty and order(side, stream) != 0:
+            raise RuntimeError("join: %s" % self.lib.pf_last_error().decode())
+
+    def capture(self, launches, stream, side=None):
         """Record `launches` (prepared launches) into a hipGraph on `stream`; returns a replay
-        callable `fn(stream)` that issues the whole list with one host call."""
+        callable `fn(stream)` that issues the whole list with one host call.  With `side`, the
+        launches marked for the side stream become a parallel branch of the graph."""
         lib = self.lib
         rc = lib.pf_graph_capture_begin(stream)
         if rc != 0:
             raise RuntimeError("graph capture: %s" % lib.pf_last_error().decode())
         try:
-            for launch in launches:
-                launch(stream)
+            self.issue(launches, stream, side)
         finally:
             handle = c_void_p()
             rc = lib.pf_graph_capture_end(stream, byref(handle))
@@ -332,6 +373,19 @@ class HipKernels:
                 _ptr(dx), _dt(dx), _ptr(dgamma), _ptr(dbeta), _ptr(ws), rows, d, int(defer))
         return self._prep("pf_layernorm_bwd", args, (dy, x, gamma, mean, rstd, dx_add, dx, dgamma, dbeta, ws),
                           rows * d * (_es(dy) + _es(x) + _es(dx) + _es(dx_add)))
+
+    def norm_bwd_fused(self, dy, x, gamma, mean, rstd, dx_add, dx, dx_lp, ws, rows, d, want_wgrad, want_colsum):
+        """Layer/RMS-norm backward (mean None: RMS) that also writes a 16-bit copy of dx and, with
+        want_colsum, its column sums; partial rows [dgamma | dbeta | colsum] go to ws."""
+        n = NormBwdDesc()
+        n.dy, n.x, n.gamma, n.mean, n.rstd = _ptr(dy), _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd)
+        n.dx_add, n.dx, n.dx_lp, n.workspace = _ptr(dx_add), _ptr(dx), _ptr(dx_lp), _ptr(ws)
+        n.rows, n.d = rows, d
+        n.dy_dtype, n.x_dtype, n.add_dtype, n.dx_dtype = _dt(dy), _dt(x), _dt(dx_add), _dt(dx)
+        n.dx_lp_dtype = _dt(dx_lp)
+        n.want_wgrad, n.want_colsum = int(bool(want_wgrad)), int(bool(want_colsum))
+        return self._prep("pf_norm_bwd_fused", (byref(n),), (n, dy, x, gamma, mean, rstd, dx_add, dx, dx_lp, ws),
+                          rows * d * (_es(dy) + _es(x) + _es(dx) + _es(dx_add) + _es(dx_lp)))
 
     def groupnorm_workspace(self, B, C, groups):
         return int(self.lib.pf_groupnorm_workspace(B, C, groups))

@@ -186,6 +186,44 @@ def test_layernorm_many_rows_param_grads(hip, oracle):
     close(r["dbeta"], 1e-4, 2e-2)
 
 
+@pytest.mark.parametrize("lpdt", [F16, BF16])
+@pytest.mark.parametrize("rows,d,rms,want_cs", [(3152, 1024, False, True), (37, 2048, True, True), (9, 100, False, False),
+                                                (300, 4096, False, False), (5, 1408, True, True)])
+def test_norm_backward_with_16bit_copy_and_column_sums(hip, oracle, lpdt, rows, d, rms, want_cs):
+    """pf_norm_bwd_fused: dx as pf_layernorm_bwd / pf_rmsnorm_bwd give it (bit-exact), its 16-bit copy
+    (bit-exact rounding of dx), and partial rows that reduce to dgamma, dbeta and the copy's column sums."""
+    x, dy, add = rnd((rows, d), F32, 1) + 0.5, rnd((rows, d), lpdt, 2), rnd((rows, d), F32, 3)
+    gamma = rnd((d,), F32, 4) + 1
+    mean = None if rms else x.mean(1)
+    rstd = 1 / torch.sqrt((x * x).mean(1) + 1e-6) if rms else 1 / torch.sqrt(x.var(1, unbiased=False) + 1e-5)
+    nb = hip.norm_bwd_partials(rows)
+    stride = (3 if want_cs else 2) * d
+    dev = lambda t: None if t is None else t.cuda()
+    dx, lp, ws = torch.zeros(rows, d).cuda(), torch.zeros(rows, d, dtype=lpdt).cuda(), torch.zeros(nb * stride).cuda()
+    hip.run("norm_bwd_fused", dev(dy), dev(x), dev(gamma), dev(mean), dev(rstd), dev(add), dx, lp, ws, rows, d, True,
+            want_cs)
+    dx0, dg0, db0 = torch.zeros(rows, d).cuda(), torch.zeros(d).cuda(), torch.zeros(d).cuda()
+    ws0 = torch.zeros(hip.colreduce_workspace(rows, d)).cuda()
+    if rms:
+        hip.run("rmsnorm_bwd", dev(dy), dev(x), dev(gamma), dev(rstd), dev(add), dx0, dg0, ws0, rows, d)
+    else:
+        hip.run("layernorm_bwd", dev(dy), dev(x), dev(gamma), dev(mean), dev(rstd), dev(add), dx0, dg0, db0, ws0, rows, d)
+    torch.cuda.synchronize()
+    assert torch.equal(dx, dx0)
+    assert torch.equal(lp, dx0.to(lpdt))
+    part = ws.view(nb, stride).cpu()
+    torch.testing.assert_close(part[:, :d].sum(0), dg0.cpu(), rtol=1e-5, atol=1e-5 * rows ** 0.5)
+    if not rms:
+        torch.testing.assert_close(part[:, d:2 * d].sum(0), db0.cpu(), rtol=1e-5, atol=1e-5 * rows ** 0.5)
+    if want_cs:
+        torch.testing.assert_close(part[:, 2 * d:].sum(0), lp.float().sum(0).cpu(), rtol=1e-5, atol=1e-5 * rows ** 0.5)
+    # and against the oracle (dx within the fp32 tolerance of the other norm tests)
+    odx, olp, ows = torch.zeros(rows, d), torch.zeros(rows, d, dtype=lpdt), torch.zeros(3 * d)
+    oracle.run("norm_bwd_fused", dy, x, gamma, mean, rstd, add, odx, olp, ows, rows, d, True, want_cs)
+    close((dx.cpu(), odx), *TOL[F32])
+    close((lp.cpu(), olp), *TOL[lpdt])
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16, F32])
 def test_colsum(hip, oracle, dtype):
     for rows, cols, ld in [(3152, 1024, 1024), (77, 1000, 1000), (5, 13, 16), (4096, 96, 104)]:
@@ -441,6 +479,9 @@ def test_deferred_reductions_match_immediate(hip):
     dict(B=1, H=2, Tq=300, Tk=300, hd=64, causal=1, packed=False),   # ragged causal over several tiles
     dict(B=2, H=2, Tq=64, Tk=77, hd=64, causal=0, packed=False),     # cross attention (77 context tokens)
     dict(B=1, H=1, Tq=5, Tk=3, hd=8, causal=0, packed=False),        # tiny
+    dict(B=2, H=2, Tq=100, Tk=130, hd=64, causal=1, packed=False),   # short causal, more keys than queries
+    dict(B=1, H=3, Tq=200, Tk=40, hd=88, causal=0, packed=False),    # short, several query blocks, few keys
+    dict(B=1, H=2, Tq=320, Tk=290, hd=64, causal=0, packed=False),   # beyond the whole-head-in-LDS kernels
 ])
 def test_fused_attention(hip, oracle, dtype, case):
     B, H, Tq, Tk, hd = case["B"], case["H"], case["Tq"], case["Tk"], case["hd"]

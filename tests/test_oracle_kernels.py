@@ -102,6 +102,15 @@ def test_norms_match_torch_and_autograd(oracle, rms):
         torch.testing.assert_close(db - 3.0, beta.grad)
     torch.testing.assert_close(dx, x.grad + add)
     torch.testing.assert_close(dg - 2.0, gamma.grad)
+    # fused form: same dx, plus its fp16 copy, the copy's column sums and the parameter partials
+    dx2, lp, ws = torch.zeros(rows, d), torch.zeros(rows, d, dtype=torch.float16), torch.zeros(3 * d)
+    oracle.run("norm_bwd_fused", dy, x.detach(), gamma.detach(), None if rms else mean, rstd, add, dx2, lp, ws,
+               rows=rows, d=d, want_wgrad=True, want_colsum=True)
+    assert torch.equal(dx2, dx) and torch.equal(lp, dx.to(torch.float16))
+    torch.testing.assert_close(ws[:d], gamma.grad)
+    if not rms:
+        torch.testing.assert_close(ws[d:2 * d], beta.grad)
+    torch.testing.assert_close(ws[2 * d:], (x.grad + add).to(torch.float16).float().sum(0))
 
 
 def test_softmax_backward_matches_autograd(oracle):
