@@ -57,13 +57,6 @@ int pf_graph_capture_begin(void* stream);
 int pf_graph_capture_end(void* stream, void** graph_exec_out);
 int pf_graph_launch(void* graph_exec, void* stream);
 int pf_graph_destroy(void* graph_exec);
-/* Orders stream `to` after everything issued on stream `from` so far (event record + wait).
- * A job forks launches that nothing later in the job reads (weight and bias gradients, which
- * only the optimizer consumes; torch.autograd orders them the same way only by accident of
- * its queue, pfeife/mp/worker.py:1585-1587) onto a side stream and joins it at the end of the
- * job, so that they fill the compute units the input-gradient chain leaves idle.  Inside a
- * capture the fork and join become graph edges.  Both streams at the default priority. */
-int pf_stream_order_after(void* from, void* to);
 
 /* ---- dense contractions (MFMA) -------------------------------------------
  * One descriptor covers every matrix product a stage executes:

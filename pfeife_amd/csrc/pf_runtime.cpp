@@ -79,28 +79,6 @@ extern "C" int pf_graph_capture_end(void* stream, void** graph_exec_out) {
   return PF_OK;
 }
 
-// Orders `to` after everything issued on `from` so far (an event recorded on `from`, waited on
-// by `to`): the fork and the join of a side stream.  Under stream capture this only adds graph
-// edges, and `to` joins the capture of `from`.  Events come from a ring: an event may be
-// recorded again as soon as its wait has been issued.
-extern "C" int pf_stream_order_after(void* from, void* to) {
-  PF_REQUIRE(from != nullptr && to != nullptr && from != to, "pf_stream_order_after: needs two created streams");
-  constexpr int RING = 256;
-  static thread_local hipEvent_t ring[RING] = {};
-  static thread_local int next = 0;
-  hipEvent_t& ev = ring[next];
-  next = (next + 1) % RING;
-  hipError_t e = hipSuccess;
-  if (ev == nullptr) e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
-  if (e == hipSuccess) e = hipEventRecord(ev, (hipStream_t)from);
-  if (e == hipSuccess) e = hipStreamWaitEvent((hipStream_t)to, ev, 0);
-  if (e != hipSuccess) {
-    pf_set_error("pf_stream_order_after: %s", hipGetErrorString(e));
-    return PF_ERR_HIP;
-  }
-  return PF_OK;
-}
-
 extern "C" int pf_graph_launch(void* graph_exec, void* stream) {
   PF_REQUIRE(graph_exec != nullptr, "pf_graph_launch: null graph");
   hipError_t e = hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream);

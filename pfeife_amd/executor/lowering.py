@@ -258,15 +258,9 @@ class StageProgram:
         for launch in self.fwd:
             launch(stream)
 
-    def run_backward(self, stream, side=None, issue=None):
-        """`side`/`issue`: a second stream and the kernel table's fork/join issue loop for the
-        launches marked `side` (weight and bias gradients); without them everything runs in
-        list order on `stream`."""
+    def run_backward(self, stream):
         if self.bwd_graph is not None:
             self.bwd_graph(stream)
-            return
-        if side and issue is not None:
-            issue(self.bwd, stream, side)
             return
         for launch in self.bwd:
             launch(stream)
@@ -289,36 +283,11 @@ class BwdCtx:
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
         self._transposed = {}  # (data_ptr, rows, cols, ld) -> transposed copy made earlier in this job
-        self._side_params = set()   # parameters whose gradient a side launch of this job writes
-        self._join_next = False
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
         self._lp = {}
 
     def emit(self, launch):
-        if self._join_next:
-            launch.after_side = True
-            self._join_next = False
-        self.out.append(launch)
-
-    def param_grad(self, param):
-        """fp32 gradient accumulator of `param` for a launch on the main stream: if a side launch
-        of this job has written it (a parameter used twice, e.g. tied embeddings), the next
-        launch waits for the side stream first."""
-        if id(param) in self._side_params:
-            self._join_next = True
-        return self.L.params.grad(param)
-
-    def emit_side(self, launch, param=None):
-        """A launch whose results nothing later in this job reads, except the batched reduction
-        at its end: parameter-gradient work, which only the optimizer consumes.  The executor may
-        run it on a second stream beside the input-gradient chain.  Its inputs (the finished
-        gradient of a forward value, saved activations, job-private temporaries) are never
-        written again within the job, and all such launches share one stream, so two writers of
-        one parameter gradient (tied weights) keep their order."""
-        launch.side = True
-        if param is not None:
-            self._side_params.add(id(param))
         self.out.append(launch)
 
     def transposed(self, t, rows, cols, ld):
@@ -328,7 +297,7 @@ class BwdCtx:
         tt = self._transposed.get(key)
         if tt is None:
             tt = self.temp((cols, rows), t.dtype)
-            self.emit_side(self.k.transpose_cast(t, ld, tt, rows, rows, cols))
+            self.emit(self.k.transpose_cast(t, ld, tt, rows, rows, cols))
             self._transposed[key] = tt
         return tt
 
@@ -352,7 +321,7 @@ class BwdCtx:
                 self.reduces.append((ws, off, nb, stride, cols, acc))
                 return
         ws = self.temp((self.k.colreduce_workspace(rows, cols),), torch.float32)
-        self.emit_side(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
+        self.emit(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
         self.reduces.append((ws, 0, self.k.colsum_partials(rows), cols, cols, acc))
 
     def new_like(self, like, private=False):
@@ -378,7 +347,7 @@ class BwdCtx:
     def _own_base_grad(self, val, zero_fill):
         """Make sure `val` (kind base) has a private, writable gradient buffer."""
         if val.param is not None:
-            return self.param_grad(val.param)
+            return self.L.params.grad(val.param)
         self._written(val.grad)
         if val.grad is None:
             val.grad = self.new_like(val.buf, val.boundary)
@@ -427,7 +396,7 @@ class BwdCtx:
                 return region, region
             return region, None
         if val.param is not None:
-            g = self.param_grad(val.param)  # AccumulateGrad: always += into the fp32 accumulator
+            g = self.L.params.grad(val.param)  # AccumulateGrad: always += into the fp32 accumulator
             return g, g
         if val.grad is None:
             return self.new_like(val.buf, val.boundary), None
@@ -597,9 +566,7 @@ class Lowerer:
         for fn in reversed(prog.backward_fns):
             fn(B)
         if B.reduces:
-            fin = self.kernels.colreduce_finalize_batch(B.reduces)
-            fin.after_side = True    # reads the partial sums the side launches leave
-            prog.bwd.append(fin)
+            prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
         prog.input_grads = []
         for v in prog.inputs:
             if isinstance(v, Val) and v.req_grad and v.param is None:
@@ -787,11 +754,10 @@ def lower_linear(L, node):
                 # transposes cost what the faster product saves
                 dy_t = B.transposed(dy, M, N, ld_dy)
                 x_t = B.transposed(xm, M, K, lda)
-                B.emit_side(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1),
-                            w.param)
+                B.emit(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1))
             else:
-                B.emit_side(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K,
-                                     a_trans=1, b_trans=1, beta=1), w.param)
+                B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
+                                b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:
@@ -1109,7 +1075,7 @@ def lower_conv2d(L, node):
         dy = B.matrix_in(gm_, cd)
         _, _, ld_dy = as_matrix(dy)
         if w.req_grad and w.param is not None:
-            B.emit(B.k.gemm(dy, cols, B.param_grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
+            B.emit(B.k.gemm(dy, cols, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=K, ldc=K, a_trans=1,
                             b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
@@ -1187,7 +1153,7 @@ def _lower_conv_same(L, x, w, b, k):
             return
         dy = _grad_nhwc(B, g, cd).reshape(M, O)
         if w.req_grad and w.param is not None:
-            wg = B.param_grad(w.param)
+            wg = L.params.grad(w.param)
             if k == 1:
                 B.emit(B.k.gemm(dy, cols, wg, M=O, N=Kc, K=M, lda=O, ldb=Kc, ldc=Kc, a_trans=1, b_trans=1, beta=1))
             else:
@@ -1727,7 +1693,7 @@ def lower_embedding(L, node):
         if g is None or table.param is None:
             return
         gc = g if g.is_contiguous() else _compact(B, g)
-        B.emit(B.k.embedding_bwd(gc, ids.buf, B.param_grad(table.param), n, dim, vocab, padding_idx))
+        B.emit(B.k.embedding_bwd(gc, ids.buf, L.params.grad(table.param), n, dim, vocab, padding_idx))
 
     if table.req_grad:
         L.add_backward(bwd)

@@ -65,6 +65,61 @@ class PartitionGraph:
         self.placeholder_names: List[str] = []
         self.static_placeholder: List[bool] = []
 
+    # -- summary (the reference prints its PipeGraph the same way, pfeife/graph/pipe_graph.py:53-54,
+    # :113-120, :145-154: one line per stage, one per stage-to-stage edge) --------------------------------
+    def edges(self):
+        """[(src stage, dst stage, bytes, [(value name, shape, dtype)])] for every pair of stages that
+        exchange activations, in stage order."""
+        out = {}
+        for idx in sorted(self.nodes):
+            st = self.nodes[idx]
+            for name, meta in zip(st.outputs, st.output_shapes):
+                for dst in sorted(d for d in st.output_map.get(name, ()) if d >= 0):
+                    e = out.setdefault((idx, dst), [0, []])
+                    if meta is not None:
+                        e[0] += meta.bytes
+                        e[1].append((name, tuple(meta.size), meta.dtype))
+        return [(a, b, w, vals) for (a, b), (w, vals) in sorted(out.items())]
+
+    def stage_summary(self, idx):
+        """dict(weight, node_len, recv, send, inputs, outputs) of one stage: bytes of the module
+        state it reads, number of compute nodes, bytes received from / sent to other stages."""
+        st = self.nodes[idx]
+        weight = recv = 0
+        for meta, gi, src in zip(st.input_shapes, st.input_placeholder, st.input_source):
+            if meta is None:
+                continue
+            if src is not None:
+                recv += meta.bytes
+            elif gi >= 0 and gi < len(self.static_placeholder) and self.static_placeholder[gi]:
+                weight += meta.bytes
+        send = sum(meta.bytes for name, meta in zip(st.outputs, st.output_shapes)
+                   if meta is not None and any(d >= 0 for d in st.output_map.get(name, ())))
+        n = len(compute_nodes(st.graph_module)) if st.graph_module is not None else 0
+        return dict(weight=weight, node_len=n, recv=recv, send=send)
+
+    def to_str(self):
+        from ..utils import fmem
+
+        lines = []
+        edges = self.edges()
+        lines.append("GRAPH: %d nodes / %d edges" % (len(self.nodes), len(edges)))
+        lines.append("==== nodes ====")
+        for idx in sorted(self.nodes):
+            st = self.nodes[idx]
+            s = self.stage_summary(idx)
+            lines.append("Node [%d/%d] (weight: %s, node len: %d, recv weight: %s, send weight: %s)"
+                         % (idx, st.rank, fmem(s["weight"]), s["node_len"], fmem(s["recv"]), fmem(s["send"])))
+        lines.append("==== edges ====")
+        for a, b, w, vals in edges:
+            shapes = ", ".join("%s %s %s" % (n, list(sz), str(dt).replace("torch.", "")) for n, sz, dt in vals)
+            lines.append("Edge (%d -> %d) (weight: %s, device: %d -> %d, values: %s)"
+                         % (a, b, fmem(w), self.nodes[a].rank, self.nodes[b].rank, shapes))
+        return "\n".join(lines)
+
+    def print_graph(self):
+        print(self.to_str())
+
 
 def compute_nodes(gm: fx.GraphModule):
     return [n for n in gm.graph.nodes if n.op not in ("placeholder", "output", "get_attr")]

@@ -88,7 +88,6 @@ _SIGNATURES = {
     "pf_graph_capture_begin": [_P],
     "pf_graph_capture_end": [_P, POINTER(c_void_p)],
     "pf_graph_launch": [_P, _P],
-    "pf_stream_order_after": [_P, _P],
     "pf_graph_destroy": [_P],
     "pf_gemm": [POINTER(GemmDesc), _P],
     "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
@@ -234,46 +233,16 @@ class HipKernels:
     def run(self, name, *a, **kw):
         getattr(self, name)(*a, **kw)(current_stream_ptr())
 
-    def issue(self, launches, stream, side=None):
-        """Issue prepared launches on `stream`.  Launches marked `side` (their results are read by
-        nothing later in the list except launches marked `after_side`) go to the stream `side`,
-        each ordered after the main-stream work issued before it; the main stream is ordered after
-        the side stream before an `after_side` launch and at the end of the list."""
-        if not side:
-            for launch in launches:
-                launch(stream)
-            return
-        order = self.lib.pf_stream_order_after
-        forked = False      # side already waits for everything issued on the main stream so far
-        dirty = False       # the side stream has work the main stream has not waited for
-        for launch in launches:
-            if getattr(launch, "side", False):
-                if not forked:
-                    if order(stream, side) != 0:
-                        raise RuntimeError("fork: %s" % self.lib.pf_last_error().decode())
-                    forked = True
-                launch(side)
-                dirty = True
-                continue
-            if dirty and getattr(launch, "after_side", False):
-                if order(side, stream) != 0:
-                    raise RuntimeError("join: %s" % self.lib.pf_last_error().decode())
-                dirty = False
-            launch(stream)
-            forked = False
-        if dirty and order(side, stream) != 0:
-            raise RuntimeError("join: %s" % self.lib.pf_last_error().decode())
-
-    def capture(self, launches, stream, side=None):
+    def capture(self, launches, stream):
         """Record `launches` (prepared launches) into a hipGraph on `stream`; returns a replay
-        callable `fn(stream)` that issues the whole list with one host call.  With `side`, the
-        launches marked for the side stream become a parallel branch of the graph."""
+        callable `fn(stream)` that issues the whole list with one host call."""
         lib = self.lib
         rc = lib.pf_graph_capture_begin(stream)
         if rc != 0:
             raise RuntimeError("graph capture: %s" % lib.pf_last_error().decode())
         try:
-            self.issue(launches, stream, side)
+            for launch in launches:
+                launch(stream)
         finally:
             handle = c_void_p()
             rc = lib.pf_graph_capture_end(stream, byref(handle))

@@ -277,6 +277,7 @@ class PartialModule(nn.Module):
         live = list(args)
         self.partition_graph = partition_by_split_points(self.gm, live, option.split_points, option.device_cnt)
         if option.print_graph:
+            self.partition_graph.print_graph()
             for idx, st in self.partition_graph.nodes.items():
                 print("================ PARTITION GRAPH %d: %d nodes ================"
                       % (idx, len(st.graph_module.graph.nodes)))

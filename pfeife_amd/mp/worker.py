@@ -62,12 +62,6 @@ class StageWorker:
         self.stream_obj = torch.cuda.Stream(self.device) if self.device.type == "cuda" else None
         self.use_graphs = (bool(getattr(kernels, "supports_graphs", False)) and self.stream_obj is not None
                            and os.environ.get("PFEIFE_NO_GRAPH", "0") != "1")
-        # second stream (default priority) for the weight- and bias-gradient launches of a backward
-        # job, which nothing else in the job reads: they run beside the input-gradient chain
-        self.side_obj = None
-        if (self.stream_obj is not None and hasattr(kernels, "issue")
-                and os.environ.get("PFEIFE_NO_SIDE_STREAM", "0") != "1"):
-            self.side_obj = torch.cuda.Stream(self.device)
         self.graphs_ready = False
         self.steps_done = 0
         self.begin_graph = None
@@ -250,9 +244,6 @@ class StageWorker:
     def stream(self):
         return self.stream_obj.cuda_stream if self.stream_obj is not None else None
 
-    def side_stream(self):
-        return self.side_obj.cuda_stream if self.side_obj is not None else None
-
     def capture_graphs(self):
         """Record every job's launch list (and the per-step zero/refresh list) into hipGraphs.
         Called after one complete eager step, when every program exists and every kernel has
@@ -263,8 +254,7 @@ class StageWorker:
                 if prog.fwd_graph is None and prog.fwd:
                     prog.fwd_graph = self.kernels.capture(prog.fwd, s)
                 if prog.bwd_graph is None and prog.bwd:
-                    prog.bwd_graph = (self.kernels.capture(prog.bwd, s, self.side_stream()) if self.side_obj is not None
-                                      else self.kernels.capture(prog.bwd, s))
+                    prog.bwd_graph = self.kernels.capture(prog.bwd, s)
         pre = self.params.zero_launches() + self.params.refresh_launches()
         self._drop_begin_graph()
         self.begin_graph = self.kernels.capture(pre, s) if pre else None
@@ -341,7 +331,7 @@ class StageWorker:
         if is_fwd:
             prog.run_forward(self.stream())
         else:
-            prog.run_backward(self.stream(), self.side_stream(), getattr(self.kernels, "issue", None))
+            prog.run_backward(self.stream())
 
     def init_optimizer(self, optimizer):
         if optimizer is not None:

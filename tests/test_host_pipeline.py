@@ -289,3 +289,42 @@ def test_failed_step_releases_parked_micro_batches():
         fail[0] = None
         again = [float(v) for v in runner.step(x, y)]
         assert again == good, mode
+
+
+def test_print_graph_lists_stages_and_edges(capsys):
+    """print_graph=True prints the stage summary in the reference's layout (pfeife/graph/pipe_graph.py:145-154):
+    a header, one line per stage, one per stage-to-stage edge with the boundary shapes and bytes."""
+    from pfeife_amd.mp import partial_compiler
+
+    torch.manual_seed(0)
+    model = VisionTransformer(CFG)
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=["blocks.1", "blocks.2", "blocks.3"],
+                        optimizer=dict(type="sgd", lr=0.0), print_graph=True)
+    runner = make_runner(option)
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+
+    def fn(x, y):
+        loss = crit(cmodel(x).float(), y)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    runner.step(torch.randn(4, 3, 32, 32, generator=g), torch.randint(0, 10, (4,), generator=g))
+    out = capsys.readouterr().out
+    assert "GRAPH: 4 nodes / 3 edges" in out
+    assert "==== nodes ====" in out and "==== edges ====" in out
+    pg = runner.worker.part_graph
+    for idx in range(4):
+        assert "Node [%d/%d] (weight: " % (idx, idx % 2) in out
+    # micro-batch 2 x (4 patches + cls) x dim floats cross every boundary
+    tokens = (CFG.image_size // CFG.patch_size) ** 2 + 1
+    edges = pg.edges()
+    assert [(a, b) for a, b, _, _ in edges] == [(0, 1), (1, 2), (2, 3)]
+    for a, b, w, vals in edges:
+        assert w == 2 * tokens * CFG.dim * 4 and vals[0][1] == (2, tokens, CFG.dim)
+        assert "Edge (%d -> %d) (weight: " % (a, b) in out
+    # the parameters are split over the stages without overlap
+    total = sum(pg.stage_summary(i)["weight"] for i in range(4))
+    assert total == sum(p.numel() * 4 for p in model.parameters())

@@ -252,3 +252,90 @@ def test_streaming(oracle):
     acc = torch.ones(6)
     oracle.run("colsum_accumulate", x, rows=4, cols=6, ld=6, acc=acc, ws=None)
     torch.testing.assert_close(acc, 1 + x.sum(0))
+
+
+@pytest.mark.parametrize("Tq,Tk,causal", [(9, 9, 1), (7, 12, 0), (5, 5, 0), (4, 10, 1)])
+def test_fused_attention_matches_sdpa_and_its_autograd(oracle, Tq, Tk, causal):
+    """attention_fwd / attention_bwd against F.scaled_dot_product_attention and autograd in fp32 (where
+    the oracle's 16-bit roundings of P and dS are the identity).  Causal with Tq != Tk: the oracle's
+    (and the kernels') bottom-right alignment, written here as an explicit mask."""
+    B, H, hd = 2, 3, 8
+    q, k, v = (rnd((B, H, T, hd), i + 1).requires_grad_() for i, T in enumerate((Tq, Tk, Tk)))
+    d_o = rnd((B, H, Tq, hd), 4)
+    mask = torch.ones(Tq, Tk, dtype=torch.bool).tril(Tk - Tq) if causal else None
+    ref = F.scaled_dot_product_attention(q, k, v, attn_mask=mask, scale=0.3)
+    ref.backward(d_o)
+    o, lse, delta = torch.zeros(B, H, Tq, hd), torch.zeros(B, H, Tq), torch.zeros(B, H, Tq)
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    oracle.run("attention_fwd", qd, kd, vd, o, lse, 0.3, causal)
+    oracle.run("attention_bwd", qd, kd, vd, o, d_o, lse, delta, dq, dk, dv, 0.3, causal)
+    torch.testing.assert_close(o, ref.detach())
+    s = torch.matmul(qd, kd.transpose(-1, -2)) * 0.3
+    if causal:
+        s = s.masked_fill(~mask, float("-inf"))
+    torch.testing.assert_close(lse, torch.logsumexp(s, -1))
+    torch.testing.assert_close(delta, (d_o * ref.detach()).sum(-1))
+    torch.testing.assert_close(dq, q.grad)
+    torch.testing.assert_close(dk, k.grad)
+    torch.testing.assert_close(dv, v.grad)
+    if causal and Tq == Tk:   # the square case is also what is_causal=True means
+        torch.testing.assert_close(o, F.scaled_dot_product_attention(qd, kd, vd, is_causal=True, scale=0.3))
+
+
+def test_groupnorm_matches_torch_and_autograd(oracle):
+    """groupnorm_fwd / groupnorm_bwd work on channels-last [B, HW, C] activations; F.group_norm on the
+    [B, C, HW] view is the reference, autograd gives dx, dgamma, dbeta."""
+    B, HW, C, G = 3, 10, 12, 4
+    x = (rnd((B, HW, C), 1) * 2 + 0.3).requires_grad_()
+    gamma, beta = (rnd((C,), 2) + 1).requires_grad_(), rnd((C,), 3).requires_grad_()
+    ref = F.group_norm(x.permute(0, 2, 1), G, gamma, beta, 1e-5).permute(0, 2, 1)
+    y, mean, rstd = torch.zeros(B, HW, C), torch.zeros(B * G), torch.zeros(B * G)
+    oracle.run("groupnorm_fwd", x.detach(), gamma.detach(), beta.detach(), y, mean, rstd, B=B, HW=HW, C=C, groups=G,
+               eps=1e-5)
+    torch.testing.assert_close(y, ref.detach())
+    xg = x.detach().reshape(B, HW, G, C // G)
+    torch.testing.assert_close(mean.view(B, G), xg.mean(dim=(1, 3)))
+    torch.testing.assert_close(rstd.view(B, G), 1 / torch.sqrt(xg.var(dim=(1, 3), unbiased=False) + 1e-5))
+    dy = rnd((B, HW, C), 4)
+    ref.backward(dy)
+    dx, dg, db = torch.zeros(B, HW, C), torch.full((C,), 2.0), torch.full((C,), 3.0)
+    ws = torch.zeros(oracle.groupnorm_workspace(B, C, G))
+    oracle.run("groupnorm_bwd", dy, x.detach(), gamma.detach(), mean, rstd, dx, dg, db, ws, B=B, HW=HW, C=C, groups=G)
+    torch.testing.assert_close(dx, x.grad)
+    torch.testing.assert_close(dg - 2.0, gamma.grad)
+    torch.testing.assert_close(db - 3.0, beta.grad)
+    # deferred form: per-batch partial rows [B][2][C] that sum to the same parameter gradients
+    oracle.run("groupnorm_bwd", dy, x.detach(), gamma.detach(), mean, rstd, dx, None, None, ws, B=B, HW=HW, C=C,
+               groups=G, defer=1)
+    part = ws[:B * 2 * C].view(B, 2, C)
+    torch.testing.assert_close(part[:, 0].sum(0), gamma.grad)
+    torch.testing.assert_close(part[:, 1].sum(0), beta.grad)
+
+
+def test_transpose_cast_copy_strided_and_column_sums(oracle):
+    src = torch.arange(5 * 8, dtype=torch.float32).view(5, 8) / 3
+    dst = torch.zeros(6, 8, dtype=torch.float16)          # [cols=6][rows=5], row stride 8
+    oracle.run("transpose_cast", src, 8, dst, 8, rows=5, cols=6)
+    assert torch.equal(dst[:, :5], src[:, :6].t().to(torch.float16)) and torch.all(dst[:, 5:] == 0)
+    # copy_strided: a permuted view into a padded destination, then accumulated once more
+    a = rnd((2, 3, 4), 1)
+    out = torch.zeros(4, 3, 2 + 1)
+    sizes, ss, ds = (4, 3, 2), (1, 4, 12), (9, 3, 1)      # out[k, j, i] = a[i, j, k]
+    oracle.run("copy_strided", a, ss, out, ds, sizes)
+    assert torch.equal(out[:, :, :2], a.permute(2, 1, 0)) and torch.all(out[:, :, 2] == 0)
+    oracle.run("copy_strided", a, ss, out, ds, sizes, accumulate=1)
+    assert torch.equal(out[:, :, :2], 2 * a.permute(2, 1, 0))
+    ids = torch.arange(6).view(2, 3)
+    iout = torch.zeros(3, 2, dtype=torch.int64)
+    oracle.run("copy_strided", ids, (1, 3), iout, (2, 1), (3, 2))
+    assert torch.equal(iout, ids.t())
+    # column sums: immediate and deferred through the batched finish
+    x = rnd((7, 6), 2).to(torch.float16)
+    acc = torch.full((4,), 1.5)
+    oracle.run("colsum_accumulate", x, 7, 4, 6, acc, None)
+    torch.testing.assert_close(acc - 1.5, x[:, :4].float().sum(0))
+    ws, acc2 = torch.zeros(8), torch.zeros(4)
+    oracle.run("colsum_accumulate", x, 7, 4, 6, None, ws, defer=1)
+    oracle.run("colreduce_finalize_batch", [(ws, 0, oracle.colsum_partials(7), 4, 4, acc2)])
+    torch.testing.assert_close(acc2, x[:, :4].float().sum(0))
