@@ -250,7 +250,7 @@ def hbm_kernel_rates(runner, reps=3):
 
 def cpu_baseline(name):
     """The oracle's restatement of the reference's stage execution on the host
-    cores, fp32, on a bounded sample of the workload (2 micro-batches)."""
+    cores, fp32, on a bounded sample of the workload (about 10-20 s of CPU work in all)."""
     import torch
     import torch.nn as nn
     import torch.nn.functional as F
@@ -271,7 +271,7 @@ def cpu_baseline(name):
         cfg = getattr(vit, cfg_name)
         model = vit.VisionTransformer(cfg)
         stages = vit.split_stages(model, int(splits[0].split(".")[1]))
-        mb = 4
+        mb, cnt = 8, 4     # the workload's four micro-batches at half their size
         x = torch.randn(mb * cnt, cfg.channels, cfg.image_size, cfg.image_size, generator=g)
         y = torch.randint(0, cfg.num_classes, (mb * cnt,), generator=g)
         loss_fn = nn.CrossEntropyLoss()
