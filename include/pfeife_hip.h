@@ -333,6 +333,20 @@ typedef struct pf_cast_item {
   int32_t src_dtype, dst_dtype, vec, reserved;
 } pf_cast_item;
 int pf_cast_batch(const pf_cast_item* items_dev, int n_items, int64_t max_n, void* stream);
+/* Both 16-bit shadows of many fp32 weight matrices in one launch (`items_dev` in DEVICE memory):
+ * plain[r*cols + c] = transposed[c*rows + r] = (dtype) src[r*cols + c]; either destination may
+ * be NULL.  Every matrix is contiguous with rows % 4 == 0 and cols % 4 == 0, src 16-byte and
+ * the destinations 8-byte aligned (the caller checks; other matrices go through pf_cast_batch /
+ * pf_transpose_cast).  max_tiles = max over items of ceil(rows/64) * ceil(cols/64).  The master
+ * is read once instead of once per shadow (autocast re-casts the weight at every use). */
+typedef struct pf_shadow_item {
+  const float* src;
+  void* plain;
+  void* transposed;
+  int64_t rows, cols;
+  int32_t dtype, reserved;
+} pf_shadow_item;
+int pf_shadow_batch(const pf_shadow_item* items_dev, int n_items, int64_t max_tiles, void* stream);
 /* dst[c*ld_dst + r] = src[r*ld_src + c] with dtype conversion: the transposed 16-bit
  * shadow of a weight matrix, made once per optimiser step, lets the input-gradient
  * product dx = dy W read W with its reduction dimension contiguous. */

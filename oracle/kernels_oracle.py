@@ -444,6 +444,20 @@ class OracleKernels:
 
         return launch
 
+    @staticmethod
+    def shadow_batch_ok(src, plain, transposed):
+        return src.dim() == 2 and src.is_contiguous()
+
+    def shadow_batch(self, items):
+        def launch(stream=None):
+            for src, plain, tr in items:
+                if plain is not None:
+                    plain.copy_(src.to(plain.dtype))
+                if tr is not None:
+                    tr.copy_(src.t().to(tr.dtype))
+
+        return launch
+
     def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
         def launch(stream=None):
             _rows(dst, cols, rows, ld_dst).copy_(_rows(src, rows, cols, ld_src).t().to(dst.dtype))

@@ -270,6 +270,49 @@ __global__ __launch_bounds__(256) void cast_batch_kernel(const pf_cast_item* ite
     pf_store_from_f32(it.dst, i, it.dst_dtype, pf_load_as_f32(it.src, i, it.src_dtype));
 }
 
+// ---- both 16-bit shadows of every weight matrix in one launch -------------------------------
+// Block (x, y) converts the 64x64 tile x of item y: the fp32 master is read once (float4 per
+// lane, 256-byte runs), the plain shadow is written from registers (8 bytes per lane), the
+// transposed shadow through a 16-bit LDS tile (8 bytes per lane, 128-byte runs).
+__global__ __launch_bounds__(256) void shadow_batch_kernel(const pf_shadow_item* items) {
+  __shared__ uint16_t tile[64][64 + 2];
+  const pf_shadow_item it = items[blockIdx.y];
+  const int64_t tiles_c = (it.cols + 63) / 64, tiles_r = (it.rows + 63) / 64;
+  if ((int64_t)blockIdx.x >= tiles_c * tiles_r) return;   // uniform over the block
+  const int64_t r0 = ((int64_t)blockIdx.x / tiles_c) * 64, c0 = ((int64_t)blockIdx.x % tiles_c) * 64;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  const bool bf = it.dtype == PF_BF16;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int lr = ty + 16 * i;
+    const int64_t r = r0 + lr, c = c0 + tx * 4;
+    uint16_t h[4] = {0, 0, 0, 0};
+    if (r < it.rows && c < it.cols) {       // rows and cols are multiples of 4
+      const float4 v = *(const float4*)(it.src + r * it.cols + c);
+      const float f[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) h[k] = bf ? pf_f32_to_bf16_bits(f[k]) : pf_f32_to_f16_bits(f[k]);
+      if (it.plain)
+        *(uint2*)((uint16_t*)it.plain + r * it.cols + c) =
+            make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) tile[lr][tx * 4 + k] = h[k];
+  }
+  __syncthreads();
+  if (!it.transposed) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int lc = ty + 16 * i;             // source column = row of the transposed shadow
+    const int64_t c = c0 + lc, r = r0 + tx * 4;
+    if (c < it.cols && r < it.rows) {
+      const uint32_t lo = (uint32_t)tile[tx * 4][lc] | ((uint32_t)tile[tx * 4 + 1][lc] << 16);
+      const uint32_t hi = (uint32_t)tile[tx * 4 + 2][lc] | ((uint32_t)tile[tx * 4 + 3][lc] << 16);
+      *(uint2*)((uint16_t*)it.transposed + c * it.rows + r) = make_uint2(lo, hi);
+    }
+  }
+}
+
 // ---- multi-tensor Adam / AdamW ---------------------------------------------------------
 // One launch updates every parameter of a param group.  Items live in device memory;
 // block y walks item y in a grid-stride loop.  The arithmetic follows torch.optim.Adam's
@@ -689,6 +732,16 @@ int adam_launch(const pf_adam_item* items_dev, int n_items, int64_t max_n, doubl
   return PF_OK;
 }
 }  // namespace
+
+extern "C" int pf_shadow_batch(const pf_shadow_item* items_dev, int n_items, int64_t max_tiles, void* stream) {
+  PF_REQUIRE(n_items >= 0 && max_tiles >= 0, "pf_shadow_batch: bad arguments");
+  if (n_items == 0 || max_tiles == 0) return PF_OK;
+  PF_REQUIRE(items_dev != nullptr && n_items <= 65535 && max_tiles < (1ll << 31), "pf_shadow_batch: bad item list");
+  hipLaunchKernelGGL(shadow_batch_kernel, dim3((unsigned)max_tiles, (unsigned)n_items), dim3(256), 0,
+                     (hipStream_t)stream, items_dev);
+  PF_CHECK_LAUNCH("pf_shadow_batch");
+  return PF_OK;
+}
 
 extern "C" int pf_cast_batch(const pf_cast_item* items_dev, int n_items, int64_t max_n, void* stream) {
   PF_REQUIRE(n_items >= 0 && max_n >= 0, "pf_cast_batch: bad arguments");

@@ -49,6 +49,7 @@ class ParamStore:
         self.params = []       # parameters that receive gradients, in first-use order
         self._keep = []
         self.cast_pairs = []   # (fp32 master, 16-bit shadow): refreshed by ONE batched launch per step
+        self.shadow_t_pairs = []   # (fp32 master, transposed 16-bit shadow) of weight matrices
         self._arena = None     # current block of the gradient arena
         self._arena_used = 0
         self.arena_block = 64 * 1024 * 1024   # fp32 elements per arena block (256 MiB)
@@ -72,10 +73,32 @@ class ParamStore:
         return sh
 
     def refresh_launches(self):
-        """Launches that bring every shadow up to date with its master (once per step)."""
+        """Launches that bring every shadow up to date with its master (once per step): weight
+        matrices get their plain and transposed shadows from one read of the master, in one
+        launch for all of them; the remaining casts share a second launch."""
         out = list(self.refresh)
-        if self.cast_pairs:
-            out.insert(0, self.kernels.cast_batch(list(self.cast_pairs)))
+        pairs = list(self.cast_pairs)
+        t_of = {src.data_ptr(): (src, sh) for src, sh in self.shadow_t_pairs}
+        batch = getattr(self.kernels, "shadow_batch", None)
+        duals, rest = [], []
+        for src, sh in pairs:
+            hit = t_of.get(src.data_ptr())
+            if (batch is not None and hit is not None and hit[1].dtype == sh.dtype
+                    and self.kernels.shadow_batch_ok(src, sh, hit[1])):
+                duals.append((src, sh, hit[1]))
+                del t_of[src.data_ptr()]
+            else:
+                rest.append((src, sh))
+        for src, sh in t_of.values():           # transposed shadow only (or not batchable)
+            if batch is not None and self.kernels.shadow_batch_ok(src, None, sh):
+                duals.append((src, None, sh))
+            else:
+                rows, cols = src.shape
+                out.append(self.kernels.transpose_cast(src, cols, sh, rows, rows, cols))
+        if duals:
+            out.insert(0, batch(duals))
+        if rest:
+            out.insert(0, self.kernels.cast_batch(rest))
         return out
 
     def _arena_alloc(self, shape, device):
@@ -158,7 +181,7 @@ class ParamStore:
             src = tensor.detach()
             if not src.is_contiguous():
                 raise Unsupported("non-contiguous parameter %s" % (tuple(tensor.shape),))
-            self.refresh.append(self.kernels.transpose_cast(src, cols, sh, rows, rows, cols))
+            self.shadow_t_pairs.append((src, sh))
             self._shadow[key] = sh
             self._keep.append(tensor)
         return sh

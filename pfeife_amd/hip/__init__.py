@@ -119,6 +119,7 @@ _SIGNATURES = {
     "pf_groupnorm_fwd": [_P, _I, _P, _P, _P, _I, _P, _P, _L, _L, _L, _I, _F, _P],
     "pf_groupnorm_bwd": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _L, _L, _L, _I, _I, _P],
     "pf_cast": [_P, _I, _P, _I, _L, _P],
+    "pf_shadow_batch": [_P, _I, _L, _P],
     "pf_cast_batch": [_P, _I, _L, _P],
     "pf_transpose_cast": [_P, _I, _L, _P, _I, _L, _L, _L, _P],
     "pf_fill": [_P, _I, _F, _L, _P],
@@ -472,6 +473,29 @@ class HipKernels:
         table = torch.tensor(rows, dtype=torch.int64).to(pairs[0][1].device)
         args = (table.data_ptr(), len(rows), max(r[2] for r in rows))
         return self._prep("pf_cast_batch", args, (table, pairs))
+
+    @staticmethod
+    def shadow_batch_ok(src, plain, transposed):
+        """Can pf_shadow_batch make these shadows of the contiguous fp32 matrix `src`?"""
+        if src.dim() != 2 or src.dtype != torch.float32 or not src.is_contiguous():
+            return False
+        if src.shape[0] % 4 or src.shape[1] % 4 or src.data_ptr() % 16:
+            return False
+        return all(t is None or (t.is_contiguous() and t.data_ptr() % 8 == 0 and t.dtype in (torch.float16, torch.bfloat16))
+                   for t in (plain, transposed))
+
+    def shadow_batch(self, items):
+        """One launch writing the plain and/or transposed 16-bit shadow of every (src, plain, transposed)."""
+        rows = []
+        for src, plain, tr in items:
+            r, c = src.shape
+            dt = dtype_code((plain if plain is not None else tr).dtype)
+            rows.append([src.data_ptr(), 0 if plain is None else plain.data_ptr(), 0 if tr is None else tr.data_ptr(),
+                         r, c, dt])
+        table = torch.tensor(rows, dtype=torch.int64).to(items[0][0].device)
+        tiles = max(((r[3] + 63) // 64) * ((r[4] + 63) // 64) for r in rows)
+        nbytes = sum(r[3] * r[4] * (4 + 2 * (r[1] != 0) + 2 * (r[2] != 0)) for r in rows)
+        return self._prep("pf_shadow_batch", (table.data_ptr(), len(rows), tiles), (table, items), nbytes)
 
     def transpose_cast(self, src, ld_src, dst, ld_dst, rows, cols):
         args = (_ptr(src), _dt(src), ld_src, _ptr(dst), _dt(dst), ld_dst, rows, cols)

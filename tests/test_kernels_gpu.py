@@ -622,3 +622,27 @@ def test_adam_step_scaled_skips_on_overflow_and_counts_steps_on_device(hip):
     torch.cuda.synchronize()
     for a, b in zip(got, ref):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_shadow_batch_bit_exact(hip, dtype):
+    """pf_shadow_batch: plain and transposed 16-bit shadows of several fp32 matrices in one launch,
+    bit-identical to torch's cast (and to its transpose), for tile-ragged shapes and for items with
+    only one of the two destinations."""
+    shapes = [(1024, 4096), (200, 72), (64, 64), (4, 1000), (260, 4)]
+    items, keep = [], []
+    for i, (r, c) in enumerate(shapes):
+        src = rnd((r, c), F32, 10 + i, 3.0).cuda()
+        plain = None if i == 3 else torch.zeros(r, c, dtype=dtype, device="cuda")
+        tr = None if i == 4 else torch.zeros(c, r, dtype=dtype, device="cuda")
+        assert hip.shadow_batch_ok(src, plain, tr)
+        items.append((src, plain, tr))
+    hip.shadow_batch(items)(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for src, plain, tr in items:
+        if plain is not None:
+            assert torch.equal(plain, src.to(dtype))
+        if tr is not None:
+            assert torch.equal(tr, src.t().contiguous().to(dtype))
+    assert not hip.shadow_batch_ok(torch.zeros(6, 8, device="cuda"), None, None)          # rows % 4
+    assert not hip.shadow_batch_ok(torch.zeros(8, 8, device="cuda").t(), None, None)      # not contiguous
