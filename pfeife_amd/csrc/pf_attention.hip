@@ -12,8 +12,8 @@
 //   dK/dV kernel        : tile = S[q][kv],   column = key row     (workgroup = 128 keys)
 //
 // Operands whose MFMA reduction index is NOT their contiguous dimension (V in forward,
-// K in dQ, Q and dO in dK/dV) are transposed in registers (8x8 blocks) on their way
-// into LDS, like the GEMM's transposing loader.
+// K in dQ, Q and dO in dK/dV) stay in their natural [token][hd] layout in LDS and are read
+// with the transposing LDS read (ds_read_b64_tr_b16); no transposed copy exists anywhere.
 //
 // Q, K, V, O and their gradients are [B, H, T, hd] tensors addressed with element
 // strides (batch, head, token) and unit stride along hd, so heads can live inside a
@@ -91,42 +91,26 @@ template <int HD> struct Tile {
   }
 };
 
-// LDS natural tile [KT][HD + 8] -> LDS transposed tile [HD][KT + 8] (element (h, t)):
-// 8x8 blocks transposed in registers, no global traffic
-template <int HD>
-__device__ __forceinline__ void transpose_tile(const uint16_t* nat, uint16_t* tr, int tid) {
-  constexpr int NLD = HD + 8, TLD = KT + 8, TB = KT / 8, HB = HD / 8;
-  for (int b = tid; b < TB * HB; b += 256) {
-    const int hb = b % HB, tb = b / HB;   // consecutive threads: adjacent 16-byte chunks of the same 8 token rows
-    uint32_t in[8][4];
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-      const uint4 x = *(const uint4*)(nat + (tb * 8 + r) * NLD + hb * 8);
-      in[r][0] = x.x; in[r][1] = x.y; in[r][2] = x.z; in[r][3] = x.w;
-    }
-#pragma unroll
-    for (int J = 0; J < 4; ++J) {
-      uint32_t lo[4], hi[4];
-#pragma unroll
-      for (int I = 0; I < 4; ++I) {
-        const uint32_t a = in[2 * I][J], c = in[2 * I + 1][J];
-        lo[I] = (a & 0xffffu) | (c << 16);
-        hi[I] = (a >> 16) | (c & 0xffff0000u);
-      }
-      *(uint4*)(tr + (hb * 8 + 2 * J) * TLD + tb * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
-      *(uint4*)(tr + (hb * 8 + 2 * J + 1) * TLD + tb * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
-    }
-  }
+#define PF_LDS16(T) __attribute__((address_space(3))) T*
+typedef short short4v_t __attribute__((ext_vector_type(4)));
+
+// Transposing LDS read.  The 16 lanes of a group each name an 8-byte chunk (4 elements);
+// group lane j must point at row k0 + j/4, columns n0 + 4*(j%4); lane i of the group then
+// receives the four elements (k0 .. k0+3, column n0 + i).
+__device__ __forceinline__ uint2 lds_read_tr(const uint16_t* p) {
+  const short4v_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PF_LDS16(short4v_t))(uintptr_t)p);
+  return __builtin_bit_cast(uint2, r);
 }
 
-// A operand read from a transposed tile for the reduction chunk [16*j, 16*j+16) of the
-// tile's token axis, with the index permutation that matches pack8(): element i of the
-// lane <-> token 16*j + 8*(i/4) + 4*(lane/32) + (i%4)
+// A operand X^T[row = hd index][k = token] for the 16-token chunk starting at `t0` of a
+// natural [token][LD] tile, hd rows o32 .. o32+31, with the token permutation of pack8():
+// element i of the lane <-> token t0 + 8*(i/4) + 4*(lane/32) + (i%4)
 template <int LD>
-__device__ __forceinline__ uint4 frag_transposed(const uint16_t* s, int row, int j, int lane) {
-  const uint16_t* p = s + row * LD + 16 * j + 4 * (lane >> 5);
-  const uint2 a = *(const uint2*)p, b = *(const uint2*)(p + 8);
-  return make_uint4(a.x, a.y, b.x, b.y);
+__device__ __forceinline__ uint4 frag_tr(const uint16_t* s, int t0, int o32, int lane) {
+  const int g = lane >> 4, j = lane & 15;
+  const uint16_t* p = s + (t0 + 4 * (g >> 1) + (j >> 2)) * LD + o32 + 16 * (g & 1) + 4 * (j & 3);
+  const uint2 lo = lds_read_tr(p), hi = lds_read_tr(p + 8 * LD);
+  return make_uint4(lo.x, lo.y, hi.x, hi.y);
 }
 
 // ---------------------------------------------------------------------------------
@@ -134,10 +118,9 @@ __device__ __forceinline__ uint4 frag_transposed(const uint16_t* s, int row, int
 // ---------------------------------------------------------------------------------
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
-  constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8, VLD = KT + 8;
+  constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8;
   __shared__ __align__(16) uint16_t sK[KT * KLD];
   __shared__ __align__(16) uint16_t sV[KT * KLD];
-  __shared__ __align__(16) uint16_t sVt[HD * VLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   const int q0 = blockIdx.x * 128 + wave * 32;
@@ -171,8 +154,6 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     __syncthreads();                     // previous tile's LDS reads are done
     tk.store(sK, tid);
     tv.store(sV, tid);
-    __syncthreads();
-    transpose_tile<HD>(sV, sVt, tid);
     if (k0 + KT < k_end) {               // next tile's global loads fly during this tile's math
       tk.load(K, a.k_st, k0 + KT, a.Tk, a.hd, tid);
       tv.load(V, a.v_st, k0 + KT, a.Tk, a.hd, tid);
@@ -234,8 +215,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
       const uint4 pf = pack8<DT>(s[j >> 1], 8 * (j & 1));
 #pragma unroll
       for (int o = 0; o < NO; ++o) {
-        const uint4 vf = frag_transposed<VLD>(sVt, o * 32 + (lane & 31), j, lane);
-        oacc[o] = M32<DT>::run(vf, pf, oacc[o]);
+        oacc[o] = M32<DT>::run(frag_tr<KLD>(sV, 16 * j, o * 32, lane), pf, oacc[o]);
       }
     }
   }
@@ -289,10 +269,9 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a, float
 // ---------------------------------------------------------------------------------
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
-  constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8, TLD = KT + 8;
+  constexpr int NC = HD / 16, NO = HD / 32, KLD = HD + 8;
   __shared__ __align__(16) uint16_t sK[KT * KLD];
   __shared__ __align__(16) uint16_t sV[KT * KLD];
-  __shared__ __align__(16) uint16_t sKt[HD * TLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   const int q0 = blockIdx.x * 128 + wave * 32;
@@ -333,8 +312,6 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
     __syncthreads();
     tk.store(sK, tid);
     tv.store(sV, tid);
-    __syncthreads();
-    transpose_tile<HD>(sK, sKt, tid);
     if (k0 + KT < k_end) {
       tk.load(K, a.k_st, k0 + KT, a.Tk, a.hd, tid);
       tv.load(V, a.v_st, k0 + KT, a.Tk, a.hd, tid);
@@ -370,8 +347,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
       const uint4 dsf = pack8<DT>(s[j >> 1], 8 * (j & 1));
 #pragma unroll
       for (int o = 0; o < NO; ++o) {
-        const uint4 kf = frag_transposed<TLD>(sKt, o * 32 + (lane & 31), j, lane);
-        acc[o] = M32<DT>::run(kf, dsf, acc[o]);
+        acc[o] = M32<DT>::run(frag_tr<KLD>(sK, 16 * j, o * 32, lane), dsf, acc[o]);
       }
     }
   }
@@ -395,11 +371,9 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
 // ---------------------------------------------------------------------------------
 template <int DT, int HD>
 __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
-  constexpr int NC = HD / 16, NO = HD / 32, QLD = HD + 8, TLD = KT + 8;
+  constexpr int NC = HD / 16, NO = HD / 32, QLD = HD + 8;
   __shared__ __align__(16) uint16_t sQ[KT * QLD];
   __shared__ __align__(16) uint16_t sDO[KT * QLD];
-  __shared__ __align__(16) uint16_t sQt[HD * TLD];
-  __shared__ __align__(16) uint16_t sDOt[HD * TLD];
   __shared__ float sLse[KT], sDelta[KT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
@@ -451,9 +425,6 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
       sLse[tid] = r_lse;
       sDelta[tid] = r_dlt;
     }
-    __syncthreads();
-    transpose_tile<HD>(sQ, sQt, tid);
-    transpose_tile<HD>(sDO, sDOt, tid);
     if (q0 + KT < a.Tq) prefetch(q0 + KT);
     __syncthreads();
     // causal: the tile needs element masks only where it crosses the diagonal
@@ -484,9 +455,8 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
       const uint4 dsf = pack8<DT>(dp[j >> 1], 8 * (j & 1));
 #pragma unroll
       for (int o = 0; o < NO; ++o) {
-        const int row = o * 32 + (lane & 31);
-        dv[o] = M32<DT>::run(frag_transposed<TLD>(sDOt, row, j, lane), pf, dv[o]);
-        dk[o] = M32<DT>::run(frag_transposed<TLD>(sQt, row, j, lane), dsf, dk[o]);
+        dv[o] = M32<DT>::run(frag_tr<QLD>(sDO, 16 * j, o * 32, lane), pf, dv[o]);
+        dk[o] = M32<DT>::run(frag_tr<QLD>(sQ, 16 * j, o * 32, lane), dsf, dk[o]);
       }
     }
   }
@@ -518,28 +488,6 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
 // so no transposed copy is made.
 // =================================================================================
 constexpr int SHORT_T = 288;   // 2 operands x 288 rows x (96 + 8) x 2 bytes = 117 KB of the 160 KB
-#define PF_LDS16(T) __attribute__((address_space(3))) T*
-typedef short short4v_t __attribute__((ext_vector_type(4)));
-
-// Transposing LDS read.  The 16 lanes of a group each name an 8-byte chunk (4 elements);
-// group lane j must point at row k0 + j/4, columns n0 + 4*(j%4); lane i of the group then
-// receives the four elements (k0 .. k0+3, column n0 + i).
-__device__ __forceinline__ uint2 lds_read_tr(const uint16_t* p) {
-  const short4v_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PF_LDS16(short4v_t))(uintptr_t)p);
-  return __builtin_bit_cast(uint2, r);
-}
-
-// A operand X^T[row = hd index][k = token] for the 16-token chunk starting at `t0` of a
-// natural [token][LD] tile, hd rows o32 .. o32+31, with the token permutation of pack8():
-// element i of the lane <-> token t0 + 8*(i/4) + 4*(lane/32) + (i%4)
-template <int LD>
-__device__ __forceinline__ uint4 frag_tr(const uint16_t* s, int t0, int o32, int lane) {
-  const int g = lane >> 4, j = lane & 15;
-  const uint16_t* p = s + (t0 + 4 * (g >> 1) + (j >> 2)) * LD + o32 + 16 * (g & 1) + 4 * (j & 3);
-  const uint2 lo = lds_read_tr(p), hi = lds_read_tr(p + 8 * LD);
-  return make_uint4(lo.x, lo.y, hi.x, hi.y);
-}
-
 template <int DT>
 __device__ __forceinline__ void unpack8(const uint4& r, float (&v)[8]) {
   const uint32_t w[4] = {r.x, r.y, r.z, r.w};

@@ -565,6 +565,41 @@ extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* sr
   return PF_OK;
 }
 
+namespace {
+// 16-bit rotary embedding, one thread per 8 consecutive pair indices: two 16-byte loads, two
+// 16-byte stores, 8 cos / sin values each (requires D/2 % 8 == 0 and 16-byte aligned rows)
+template <int DT>
+__global__ __launch_bounds__(EW_BLOCK) void rope_vec_kernel(const uint16_t* x, uint16_t* y, const float* cos_t,
+                                                            const float* sin_t, int64_t tab_ld, int64_t B, int64_t T,
+                                                            int64_t H, int64_t D, int64_t xsb, int64_t xst, int64_t xsh,
+                                                            int64_t ysb, int64_t yst, int64_t ysh, int inverse) {
+  const int64_t half = D / 2, hv = half / 8;
+  const int64_t total = B * T * H * hv;
+  const int64_t gsz = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gsz) {
+    const int64_t i = (idx % hv) * 8;
+    int64_t r = idx / hv;
+    const int64_t h = r % H;
+    r /= H;
+    const int64_t t = r % T, b = r / T;
+    const int64_t xo = b * xsb + t * xst + h * xsh + i, yo = b * ysb + t * yst + h * ysh + i;
+    float x1[8], x2[8], c[8], sn[8], o1[8], o2[8];
+    Vec8<DT>::load(x, xo, x1);
+    Vec8<DT>::load(x, xo + half, x2);
+    Vec8<PF_F32>::load(cos_t, t * tab_ld + i, c);
+    Vec8<PF_F32>::load(sin_t, t * tab_ld + i, sn);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float s = inverse ? -sn[k] : sn[k];
+      o1[k] = x1[k] * c[k] - x2[k] * s;
+      o2[k] = x2[k] * c[k] + x1[k] * s;
+    }
+    Vec8<DT>::store(y, yo, o1);
+    Vec8<DT>::store(y, yo + half, o2);
+  }
+}
+}  // namespace
+
 extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, const float* sin_t, int64_t tab_ld,
                        int64_t B, int64_t T, int64_t H, int64_t D, int64_t x_sb, int64_t x_st, int64_t x_sh,
                        int64_t y_sb, int64_t y_st, int64_t y_sh, int inverse, void* stream) {
@@ -573,6 +608,20 @@ extern "C" int pf_rope(const void* x, void* y, int dtype, const float* cos_t, co
   const int64_t total = B * T * H * (D / 2);
   if (total == 0) return PF_OK;
   PF_REQUIRE(x && y && cos_t && sin_t, "pf_rope: null pointer");
+  const bool vec = dtype != PF_F32 && (D / 2) % 8 == 0 && tab_ld % 4 == 0 && al16(x) && al16(y) && al16(cos_t) &&
+                   al16(sin_t) && x_sb % 8 == 0 && x_st % 8 == 0 && x_sh % 8 == 0 && y_sb % 8 == 0 && y_st % 8 == 0 &&
+                   y_sh % 8 == 0;
+  if (vec) {
+    const dim3 grid = ew_grid(total / 8);
+    if (dtype == PF_F16)
+      hipLaunchKernelGGL(rope_vec_kernel<PF_F16>, grid, dim3(EW_BLOCK), 0, (hipStream_t)stream, (const uint16_t*)x,
+                         (uint16_t*)y, cos_t, sin_t, tab_ld, B, T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
+    else
+      hipLaunchKernelGGL(rope_vec_kernel<PF_BF16>, grid, dim3(EW_BLOCK), 0, (hipStream_t)stream, (const uint16_t*)x,
+                         (uint16_t*)y, cos_t, sin_t, tab_ld, B, T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
+    PF_CHECK_LAUNCH("pf_rope");
+    return PF_OK;
+  }
   hipLaunchKernelGGL(rope_kernel, ew_grid(total), dim3(EW_BLOCK), 0, (hipStream_t)stream, x, y, dtype, cos_t, sin_t,
                      tab_ld, B, T, H, D, x_sb, x_st, x_sh, y_sb, y_st, y_sh, inverse);
   PF_CHECK_LAUNCH("pf_rope");

@@ -305,24 +305,12 @@ class BwdCtx:
         self._seq = 0
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
-        self._transposed = {}  # (data_ptr, rows, cols, ld) -> transposed copy made earlier in this job
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
         self._lp = {}
 
     def emit(self, launch):
         self.out.append(launch)
-
-    def transposed(self, t, rows, cols, ld):
-        """[cols, rows] copy of the 16-bit matrix t (made once per job and matrix: several
-        weight-gradient products that reduce over the same token rows share it)."""
-        key = (t.data_ptr(), rows, cols, ld)
-        tt = self._transposed.get(key)
-        if tt is None:
-            tt = self.temp((cols, rows), t.dtype)
-            self.emit(self.k.transpose_cast(t, ld, tt, rows, rows, cols))
-            self._transposed[key] = tt
-        return tt
 
     def register_lp(self, full, copy, colsum=None):
         """`copy` holds the values of the fp32 gradient `full` in the compute dtype; `colsum`:
@@ -517,7 +505,6 @@ class Lowerer:
         self.device = torch.device(device)
         self.cd = compute_dtype or torch.float32
         self.mixed = self.cd != torch.float32
-        self.dw_transpose_min_elems = 8 * 1024 * 1024
         self.params = params or ParamStore(kernels, self.device)
         self.pool = pool or BufferPool(self.device)
         self._ws = None
@@ -769,18 +756,10 @@ def lower_linear(L, node):
             dy = B.matrix_in(g, cd)
         _, _, ld_dy = as_matrix(dy)
         if w.req_grad and w.param is not None:
-            if L.mixed and M % 8 == 0 and M >= 1024 and N * K >= L.dw_transpose_min_elems:
-                # dW = dY^T X reduces over the token rows: with both operands copied transposed
-                # (cheap, HBM-bound) it runs on the row-row MFMA path.  Measured: for weight
-                # matrices of >= 8M elements (enough 128x128 tiles for two workgroups per CU) that
-                # path is ~1.8x the rate of the transposing loaders; for smaller ones the two
-                # transposes cost what the faster product saves
-                dy_t = B.transposed(dy, M, N, ld_dy)
-                x_t = B.transposed(xm, M, K, lda)
-                B.emit(B.k.gemm(dy_t, x_t, L.params.grad(w.param), M=N, N=K, K=M, lda=M, ldb=M, ldc=K, beta=1))
-            else:
-                B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
-                                b_trans=1, beta=1))
+            # dW = dY^T X reduces over the token rows, the strided dimension of both operands: the
+            # GEMM reads them with transposing LDS reads (no transposed copies in memory)
+            B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
+                            b_trans=1, beta=1))
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:

@@ -369,6 +369,14 @@ def test_copy_strided_and_rope(hip, oracle, dtype):
     back = both(hip, oracle, "rope", dict(x=r["y"][1], y=torch.zeros_like(y), cos_t=cos_t, sin_t=sin_t), ["y"], B=Bq,
                 T=T, H=H, D=D, xs=(T * H * D, H * D, D), ys=(T * H * D, H * D, D), inverse=1)
     close((back["y"][0], qkv.view(Bq, T, 3, H, D)[:, :, 0].contiguous()), TOL[dtype][0] * 3, TOL[dtype][1] * 3)
+    # a head dim whose half is no multiple of 8 takes the element-wise kernel
+    D2 = 24
+    x2 = rnd((Bq, T, H, D2), dtype, 5)
+    ang2 = torch.arange(T).float()[:, None] * (1.0 / (10000 ** (torch.arange(0, D2, 2).float() / D2)))[None, :]
+    r = both(hip, oracle, "rope", dict(x=x2, y=torch.zeros_like(x2), cos_t=ang2.cos().contiguous(),
+                                       sin_t=ang2.sin().contiguous()), ["y"], B=Bq, T=T, H=H, D=D2,
+             xs=(T * H * D2, H * D2, D2), ys=(T * H * D2, H * D2, D2), inverse=0)
+    close(r["y"], *TOL[dtype])
 
 
 def test_split_merge_bit_exact(hip, oracle):

@@ -384,29 +384,6 @@ def test_unet_stage_sdxl_style(mixed):
     _check_grads(model, ref, mixed)
 
 
-@pytest.mark.parametrize("mixed", ["fp16", "bf16"])
-def test_many_token_rows_take_the_transposed_weight_gradient_path(mixed, monkeypatch):
-    """With >= 1024 token rows per micro-batch, weight gradients of large matrices are computed
-    from transposed copies of dY and X (row-row MFMA path); same parity bar as every other
-    configuration.  (The size threshold is lowered so that this small model takes the path.)"""
-    from pfeife_amd.bench_models.vit import ViTConfig
-    from pfeife_amd.executor import lowering
-
-    orig = lowering.Lowerer.__init__
-
-    def patched(self, *a, **kw):
-        orig(self, *a, **kw)
-        self.dw_transpose_min_elems = 0
-
-    monkeypatch.setattr(lowering.Lowerer, "__init__", patched)
-
-    cfg = ViTConfig(image_size=32, patch_size=16, dim=128, depth=2, heads=2, mlp_dim=256, num_classes=16)
-    m, r, l, rl, runner = _run_vit(cfg, 512, 2, "blocks.1", mixed)   # 256 images x 5 tokens = 1280 rows
-    _check(m, r, l, rl, mixed)
-    kernels = [getattr(x, "kernel", "") for p in runner.worker.mbs[0].stage_programs.values() for x in p.bwd]
-    assert "pf_transpose_cast" in kernels
-
-
 @pytest.mark.parametrize("opt_type,wd", [("adam", 0.0), ("adam", 0.01), ("adamw", 0.05)])
 def test_fused_adam_matches_torch_optimizer(opt_type, wd):
     """Three training steps with the fused multi-tensor Adam launch against the same steps
