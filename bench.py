@@ -154,7 +154,7 @@ def gemm_roofline(runner, mixed, workload, reps=3):
     record of the instantiation that takes the most time plus an all-GEMM summary."""
     groups = {}
     for launch in _step_launches(runner):
-        if getattr(launch, "kernel", "") == "pf_gemm":
+        if getattr(launch, "kernel", "") in ("pf_gemm", "pf_gemm_grouped"):
             g = groups.setdefault(launch.variant, dict(launches=[], flops=0.0))
             g["launches"].append(launch)
             g["flops"] += launch.flops

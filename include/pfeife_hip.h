@@ -134,6 +134,13 @@ typedef struct pf_gemm_desc {
 } pf_gemm_desc;
 
 int pf_gemm(const pf_gemm_desc* desc, void* stream);
+/* n products in as few launches as possible.  Runs of consecutive descriptors that are weight
+ * gradients (a_trans = b_trans = 1, 16-bit operands, fp32 C with beta = 1, no epilogue operands,
+ * no batch) and resolve to the same kernel instantiation share ONE launch (up to 4 per launch):
+ * dW of a 1024x1024 weight covers only 64 of the 256 CUs on its own.  Everything else is issued
+ * as by pf_gemm, in order.  The products of one call must not depend on each other's results.
+ * torch.autograd issues the same products one by one (pfeife/mp/worker.py:1585-1587). */
+int pf_gemm_grouped(const pf_gemm_desc* descs, int n, void* stream);
 /* Name of the kernel instantiation pf_gemm would launch for `desc`, spelled the
  * way a profiler prints it, e.g. "gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 0>"
  * (dtype, tile M, tile N, stage depth, wavefront grid, stages, a_trans, b_trans, epilogue

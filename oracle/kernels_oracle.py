@@ -84,6 +84,19 @@ class OracleKernels:
         return 1
 
     # -- dense contractions ----------------------------------------------------
+    GEMM_GROUP_MAX = 4
+
+    @staticmethod
+    def gemm_groupable(launch):
+        return False      # the oracle runs every product on its own
+
+    def gemm_group(self, launches):
+        def launch(stream=None):
+            for l in launches:
+                l(stream)
+
+        return launch
+
     def gemm(self, a, b, c, M, N, K, lda, ldb, ldc, a_trans=0, b_trans=0, batch=(1, 1), sa=(0, 0), sb=(0, 0),
              sc=(0, 0), alpha=1.0, beta=0, bias=None, round_mid=0, aux_out=None, ld_aux_out=0, act=0, dact=0,
              aux_in=None, ld_aux_in=0, residual=None, ld_res=0):

@@ -18,6 +18,8 @@
 // direct-to-LDS kernels, one translation unit per operand dtype
 int pf_gemm_x_f16(const pf_gemm_desc& d, int tile, hipStream_t st);
 int pf_gemm_x_bf16(const pf_gemm_desc& d, int tile, hipStream_t st);
+int pf_gemm_xgroup_f16(const pf_gemm_desc* d, int n, int tile, hipStream_t st);
+int pf_gemm_xgroup_bf16(const pf_gemm_desc* d, int n, int tile, hipStream_t st);
 
 namespace {
 
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, ((BM * BN > 128 * 128 || (AT && BT)
   using SB = Stage<BN, BK, NT, BT>;
   extern __shared__ __align__(16) uint16_t smem[];
 
-  const int t = gemm_tile_id(g.tiles_m * g.tiles_n, g.per_xcd);
+  const int t = gemm_tile_id((int)blockIdx.x, g.tiles_m * g.tiles_n, g.per_xcd);
   if (t < 0) return;
   int tm, tn;
   gemm_tile_rc(t, g.tiles_m, g.tiles_n, tm, tn);
@@ -315,7 +317,7 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const pf_gemm_desc p, const
   __shared__ float sA[TK][TB + PAD];
   __shared__ float sB[TK][TB + PAD];
 
-  const int t = gemm_tile_id(g.tiles_m * g.tiles_n, g.per_xcd);
+  const int t = gemm_tile_id((int)blockIdx.x, g.tiles_m * g.tiles_n, g.per_xcd);
   if (t < 0) return;
   int tm, tn;
   gemm_tile_rc(t, g.tiles_m, g.tiles_n, tm, tn);
@@ -554,6 +556,58 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
   }
   if (d.in_dtype == PF_F16) return dispatch16<PF_F16>(d, st);
   return dispatch16<PF_BF16>(d, st);
+}
+
+// Checks shared by pf_gemm and pf_gemm_grouped for one 16-bit descriptor that is to run on the
+// direct-to-LDS weight-gradient kernel as part of a group.
+namespace {
+bool groupable(const pf_gemm_desc& d, int& variant) {
+  if (d.in_dtype != PF_F16 && d.in_dtype != PF_BF16) return false;
+  if (!(d.a_trans && d.b_trans) || d.c_dtype != PF_F32 || d.beta != 1 || d.alpha != 1.f) return false;
+  if (d.batch1 > 1 || d.batch2 > 1 || d.bias || d.residual || d.aux_in || d.aux_out || d.act || d.dact) return false;
+  if (d.M <= 0 || d.N <= 0 || d.K <= 0 || !d.A || !d.B || !d.C) return false;
+  if (!pf_aligned(d.A, 16) || !pf_aligned(d.B, 16) || d.lda % 8 || d.ldb % 8 || d.lda < d.M || d.ldb < d.N ||
+      d.ldc < d.N)
+    return false;
+  const int64_t a_bytes = (d.K + 256) * d.lda * 2, b_bytes = (d.K + 256) * d.ldb * 2;
+  if (a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31)) return false;
+  variant = resolve_variant(d);
+  if (variant != V_X256 && variant != V_X256x128 && variant != V_X128) return false;
+  if (!x_supports(d, variant)) return false;
+  return epi_class(d, epi_vec_ok(d)) == EC_ACC32;
+}
+}  // namespace
+
+extern "C" int pf_gemm_grouped(const pf_gemm_desc* descs, int n, void* stream) {
+  PF_REQUIRE(n >= 0 && (n == 0 || descs != nullptr), "pf_gemm_grouped: bad arguments");
+  int i = 0;
+  while (i < n) {
+    // longest run (up to the kernel's group size) of problems that share one instantiation
+    int v0 = 0, run = 0;
+    if (groupable(descs[i], v0)) {
+      run = 1;
+      int v = 0;
+      while (i + run < n && run < 4 && descs[i + run].in_dtype == descs[i].in_dtype && groupable(descs[i + run], v) &&
+             v == v0)
+        ++run;
+    }
+    if (run >= 2) {
+      pf_gemm_desc d[4];
+      for (int k = 0; k < run; ++k) {
+        d[k] = descs[i + k];
+        d[k].batch1 = d[k].batch2 = 1;
+      }
+      const int rc = descs[i].in_dtype == PF_F16 ? pf_gemm_xgroup_f16(d, run, v0, (hipStream_t)stream)
+                                                 : pf_gemm_xgroup_bf16(d, run, v0, (hipStream_t)stream);
+      if (rc != PF_OK) return rc;
+      i += run;
+    } else {
+      const int rc = pf_gemm(&descs[i], stream);
+      if (rc != PF_OK) return rc;
+      ++i;
+    }
+  }
+  return PF_OK;
 }
 
 extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {

@@ -98,8 +98,7 @@ __device__ __forceinline__ void epilogue_vec8(const Epi& e, int64_t c_base, int6
 // XCD-aware tile id: consecutive workgroup ids are dealt round-robin to the 8
 // XCDs, so give each XCD a contiguous range of tiles (its L2 then sees a compact
 // set of A rows / B columns). Returns -1 for the padding workgroups.
-__device__ __forceinline__ int gemm_tile_id(int tiles, int per_xcd) {
-  const int pid = blockIdx.x;
+__device__ __forceinline__ int gemm_tile_id(int pid, int tiles, int per_xcd) {
   const int t = (pid & 7) * per_xcd + (pid >> 3);
   return t < tiles ? t : -1;
 }

@@ -168,9 +168,10 @@ template <int DT> __device__ __forceinline__ v4i_t pack16(const float8_t& v) {
   return o;
 }
 
+// `pid`: index of this workgroup among the workgroups of its problem (the launch may hold several
+// problems, see gemm16x_group_kernel)
 template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
-__global__ __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 1024 && 64 * WGM * WGN <= 256) ? 2 : 1) void gemm16x_kernel(
-    const pf_gemm_desc p, const GemmGrid g) {
+__device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGrid& g, const int pid) {
   constexpr int NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 10
   constexpr int NFA = AT ? TM : KK, NFB = BT ? TN : KK;
   extern __shared__ __align__(16) uint16_t smem[];
 
-  const int t = gemm_tile_id(g.tiles_m * g.tiles_n, g.per_xcd);
+  const int t = gemm_tile_id(pid, g.tiles_m * g.tiles_n, g.per_xcd);
   if (t < 0) return;
   int tm, tn;
   gemm_tile_rc(t, g.tiles_m, g.tiles_n, tm, tn);
@@ -533,6 +534,33 @@ __global__ __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 10
   __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 
+#define PF_X_BOUNDS __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 1024 && 64 * WGM * WGN <= 256) ? 2 : 1)
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
+__global__ PF_X_BOUNDS void gemm16x_kernel(const pf_gemm_desc p, const GemmGrid g) {
+  gemm16x_body<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>(p, g, (int)blockIdx.x);
+}
+
+// Several independent problems of the same kind in one launch: problem i owns the workgroups
+// [start[i], start[i+1]).  Weight-gradient products are independent of everything that follows
+// them in a backward job; small ones (64 tiles for a 1024x1024 weight) are launched together so
+// that they fill the 256 CUs.
+constexpr int GEMM_GROUP_MAX = 4;
+struct GemmGroup {
+  pf_gemm_desc p[GEMM_GROUP_MAX];
+  GemmGrid g[GEMM_GROUP_MAX];
+  int start[GEMM_GROUP_MAX];
+  int n;
+};
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
+__global__ PF_X_BOUNDS void gemm16x_group_kernel(const GemmGroup ga) {
+  int i = 0;
+#pragma unroll
+  for (int k = 1; k < GEMM_GROUP_MAX; ++k)
+    if (k < ga.n && (int)blockIdx.x >= ga.start[k]) i = k;
+  i = __builtin_amdgcn_readfirstlane(i);
+  gemm16x_body<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>(ga.p[i], ga.g[i], (int)blockIdx.x - ga.start[i]);
+}
+
 template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
 int launch16x_t(const pf_gemm_desc& d, const GemmGrid& g, hipStream_t st) {
   constexpr int NT = 64 * WGM * WGN;
@@ -603,6 +631,66 @@ int launch16x(const pf_gemm_desc& d, hipStream_t st) {
 #undef PF_X
   pf_set_error("pf_gemm: tile %dx%d has no variant for a_trans=%d b_trans=%d", BM, BN, d.a_trans, d.b_trans);
   return PF_ERR_INVALID;
+}
+
+// Several weight-gradient products (both operands reduction-strided, fp32 C accumulated) in one
+// launch; the caller has checked that they all take tile BMxBN and the EC_ACC32 epilogue.
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST>
+int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
+  if constexpr ((BM == 128 || BM == 256) && (BN == 128 || BN == 256)) {
+    constexpr int NT = 64 * WGM * WGN;
+    constexpr size_t lds_main = (size_t)ST * (BM + BN) * BK * 2;
+    constexpr size_t lds_fast = (size_t)(WGM * WGN) * (16 * (BN / WGN + 8) * 4 + 2 * (16 / (64 / (BN / WGN / 8))) * 2 * 1024);
+    constexpr size_t lds = lds_main > lds_fast ? lds_main : lds_fast;
+    GemmGroup ga;
+    int blocks = 0;
+    for (int i = 0; i < n; ++i) {
+      ga.p[i] = d[i];
+      ga.g[i].tiles_m = (int)((d[i].M + BM - 1) / BM);
+      ga.g[i].tiles_n = (int)((d[i].N + BN - 1) / BN);
+      ga.g[i].per_xcd = (int)(((int64_t)ga.g[i].tiles_m * ga.g[i].tiles_n + 7) / 8);
+      ga.g[i].vec_epi = epi_vec_ok(d[i]);
+      ga.start[i] = blocks;          // a multiple of 8: the workgroup -> XCD dealing stays aligned
+      blocks += ga.g[i].per_xcd * 8;
+    }
+    for (int i = n; i < GEMM_GROUP_MAX; ++i) {
+      ga.p[i] = d[0];
+      ga.g[i] = ga.g[0];
+      ga.start[i] = blocks;
+    }
+    ga.n = n;
+    auto kern = gemm16x_group_kernel<DT, BM, BN, BK, WGM, WGN, ST, true, true, EC_ACC32>;
+    if (lds > 64 * 1024) {
+      static std::mutex mu;
+      static bool raised[64] = {};
+      int dev = 0;
+      if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+      std::lock_guard<std::mutex> lock(mu);
+      if (!raised[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) {
+          pf_set_error("pf_gemm_grouped: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
+          return PF_ERR_HIP;
+        }
+        raised[dev] = true;
+      }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks, 1, 1), dim3(NT), lds, st, ga);
+    PF_CHECK_LAUNCH("pf_gemm_grouped");
+    return PF_OK;
+  }
+  pf_set_error("pf_gemm_grouped: tile %dx%d has no transposed variant", BM, BN);
+  return PF_ERR_INVALID;
+}
+
+template <int DT>
+int gemm_x_group_launch(const pf_gemm_desc* d, int n, int tile, hipStream_t st) {
+  switch (tile) {
+    case PF_XT_256x256: return launch16x_group<DT, 256, 256, 32, 2, 2, 5>(d, n, st);
+    case PF_XT_256x128: return launch16x_group<DT, 256, 128, 64, 2, 2, 3>(d, n, st);
+    case PF_XT_128x128: return launch16x_group<DT, 128, 128, 64, 2, 2, 3>(d, n, st);
+    default: pf_set_error("pf_gemm_grouped: unknown direct-to-LDS tile %d", tile); return PF_ERR_INVALID;
+  }
 }
 
 // tile: one of the PF_XT_* shapes (see pf_gemm_x_tiles)

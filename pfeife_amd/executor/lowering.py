@@ -305,12 +305,53 @@ class BwdCtx:
         self._seq = 0
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
+        self._dw = []       # held-back weight-gradient products: (launch, accumulator, tiles)
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
         self._lp = {}
 
     def emit(self, launch):
         self.out.append(launch)
+
+    # -- weight-gradient products that share a launch ---------------------------------------------
+    FULL_GRID = 256     # workgroups that fill the device (one tile per CU)
+
+    @staticmethod
+    def _tiles(launch):
+        bm, bn = (int(x) for x in launch.variant.split("<")[1].split(",")[1:3])
+        return ((launch.desc.M + bm - 1) // bm) * ((launch.desc.N + bn - 1) // bn)
+
+    def emit_dw(self, launch, grad):
+        """A weight-gradient product: only the optimizer reads its result, and its inputs (a
+        finished gradient, a saved activation) are not written again within the job, so it may
+        be held back and issued together with later ones.  Products too small to give every CU a
+        tile are collected until they fill the device (ViT-L: dW of the 1024x1024 attention
+        projection, 64 tiles, rides with dW of the qkv projection, 192 tiles)."""
+        groupable = getattr(self.k, "gemm_groupable", None)
+        if groupable is None or not groupable(launch):
+            self.emit(launch)
+            return
+        tiles = self._tiles(launch)
+        if any(g.data_ptr() == grad.data_ptr() for _, g, _ in self._dw):
+            self.flush_dw()          # two products into one accumulator keep their order
+        if tiles >= self.FULL_GRID:
+            self.emit(launch)
+            return
+        held = sum(t for _, _, t in self._dw)
+        if self._dw and (self._dw[0][0].variant != launch.variant or held + tiles > self.FULL_GRID
+                         or len(self._dw) == self.k.GEMM_GROUP_MAX):
+            self.flush_dw()
+            held = 0
+        self._dw.append((launch, grad, tiles))
+        if held + tiles >= self.FULL_GRID - 32:
+            self.flush_dw()
+
+    def flush_dw(self):
+        if len(self._dw) == 1:
+            self.emit(self._dw[0][0])
+        elif self._dw:
+            self.emit(self.k.gemm_group([l for l, _, _ in self._dw]))
+        self._dw = []
 
     def register_lp(self, full, copy, colsum=None):
         """`copy` holds the values of the fp32 gradient `full` in the compute dtype; `colsum`:
@@ -575,6 +616,7 @@ class Lowerer:
                 B.contribute(v, g)
         for fn in reversed(prog.backward_fns):
             fn(B)
+        B.flush_dw()
         if B.reduces:
             prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
         prog.input_grads = []
@@ -758,8 +800,8 @@ def lower_linear(L, node):
         if w.req_grad and w.param is not None:
             # dW = dY^T X reduces over the token rows, the strided dimension of both operands: the
             # GEMM reads them with transposing LDS reads (no transposed copies in memory)
-            B.emit(B.k.gemm(dy, xm, L.params.grad(w.param), M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1,
-                            b_trans=1, beta=1))
+            wg = L.params.grad(w.param)
+            B.emit_dw(B.k.gemm(dy, xm, wg, M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1, b_trans=1, beta=1), wg)
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:

@@ -90,6 +90,7 @@ _SIGNATURES = {
     "pf_graph_launch": [_P, _P],
     "pf_graph_destroy": [_P],
     "pf_gemm": [POINTER(GemmDesc), _P],
+    "pf_gemm_grouped": [POINTER(GemmDesc), _I, _P],
     "pf_gemm_variant": [POINTER(GemmDesc), ctypes.c_char_p, _I],
     "pf_attention_fwd": [POINTER(AttnDesc), _P],
     "pf_attention_bwd": [POINTER(AttnDesc), _P],
@@ -302,6 +303,30 @@ class HipKernels:
         self.lib.pf_gemm_variant(byref(d), name, 128)
         launch.variant = name.value.decode()
         launch.flops = 2.0 * M * N * K * batch[0] * batch[1]
+        launch.desc = d
+        return launch
+
+    GEMM_GROUP_MAX = 4
+
+    @staticmethod
+    def gemm_groupable(launch):
+        """A weight-gradient product on the direct-to-LDS kernel (fp32 C accumulated): launches of
+        this kind with the same `variant` may share one launch (pf_gemm_grouped)."""
+        v = getattr(launch, "variant", "")
+        return v.startswith("gemm16x_kernel<") and v.endswith("true, true, 4>")
+
+    def gemm_group(self, launches):
+        """One launch for 2..GEMM_GROUP_MAX independent `gemm_groupable` products of the same variant."""
+        n = len(launches)
+        if not (2 <= n <= self.GEMM_GROUP_MAX) or len({l.variant for l in launches}) != 1 \
+                or not all(self.gemm_groupable(l) for l in launches):
+            raise RuntimeError("gemm_group: needs 2..%d groupable launches of one variant" % self.GEMM_GROUP_MAX)
+        arr = (GemmDesc * n)()
+        for i, l in enumerate(launches):
+            ctypes.memmove(ctypes.byref(arr[i]), ctypes.byref(l.desc), ctypes.sizeof(GemmDesc))
+        launch = self._prep("pf_gemm_grouped", (arr, n), (arr, launches))
+        launch.variant = launches[0].variant.replace("gemm16x_kernel<", "gemm16x_group_kernel<")
+        launch.flops = sum(l.flops for l in launches)
         return launch
 
     # -- fused attention -----------------------------------------------------------

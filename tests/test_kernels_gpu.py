@@ -654,3 +654,48 @@ def test_shadow_batch_bit_exact(hip, dtype):
             assert torch.equal(tr, src.t().contiguous().to(dtype))
     assert not hip.shadow_batch_ok(torch.zeros(6, 8, device="cuda"), None, None)          # rows % 4
     assert not hip.shadow_batch_ok(torch.zeros(8, 8, device="cuda").t(), None, None)      # not contiguous
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_gemm_grouped_weight_gradients_bit_exact(hip, dtype):
+    """pf_gemm_grouped: several weight-gradient products (dY^T X accumulated into fp32) in one launch
+    give bit-identical results to the same products launched one by one (same kernel, same tiles);
+    products of different instantiations in one call fall back to separate launches, in order."""
+    torch.manual_seed(0)
+    K = 1576   # token rows: not a multiple of the reduction tile
+    shapes = [(1024, 1024), (1024, 3072), (256, 512), (384, 1024)]
+    probs = []
+    for i, (M, N) in enumerate(shapes):
+        dy = rnd((K, M), dtype, 20 + i).cuda()
+        x = rnd((K, N), dtype, 30 + i).cuda()
+        c0 = rnd((M, N), F32, 40 + i).cuda()
+        probs.append((dy, x, c0))
+    singles, groups = [], []
+    for dy, x, c0 in probs:
+        M, N = dy.shape[1], x.shape[1]
+        c1, c2 = c0.clone(), c0.clone()
+        singles.append((hip.gemm(dy, x, c1, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1), c1))
+        groups.append((hip.gemm(dy, x, c2, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1), c2))
+    s = torch.cuda.current_stream().cuda_stream
+    for l, _ in singles:
+        l(s)
+    by_variant = {}
+    for l, c in groups:      # the 256x512 problem runs on the register-staged kernel: not groupable
+        by_variant.setdefault(l.variant if hip.gemm_groupable(l) else "single %d" % len(by_variant), []).append(l)
+    grouped = 0
+    for v, ls in by_variant.items():
+        if len(ls) >= 2:
+            g = hip.gemm_group(ls)
+            assert g.variant.startswith("gemm16x_group_kernel<") and g.flops == sum(l.flops for l in ls)
+            g(s)
+            grouped += 1
+        else:
+            ls[0](s)
+    assert grouped >= 1
+    torch.cuda.synchronize()
+    for (_, c1), (_, c2), (dy, x, c0) in zip(singles, groups, probs):
+        assert torch.equal(c1, c2)
+        ref = c0.double() + dy.double().t() @ x.double()
+        torch.testing.assert_close(c1.double(), ref, rtol=2e-3, atol=2e-2)
+    with pytest.raises(RuntimeError):
+        hip.gemm_group([groups[0][0]])
