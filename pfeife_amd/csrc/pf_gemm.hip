@@ -423,7 +423,7 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
 // Variant ids (pf_gemm_desc.variant; 0 = automatic):
 //   1..3   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128
 //   11..14 register-staged kernel: 128x128 by 8 wavefronts, 128x128, 128x64, 64x64 by 4
-enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
+enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_X192x256 = 4, V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
 
 // Register-staged tiles: 128x128 with two workgroups resident per CU is the largest that keeps
 // accumulators, two sets of staging registers and fragments in the register file; smaller tiles
@@ -444,7 +444,8 @@ int choose_staged(const pf_gemm_desc& d) {
 // reduction-contiguous or both reduction-strided; a ragged reduction tail is zero-filled by the
 // hardware range check only in the second case (whole k-rows fall outside the operand).
 bool x_supports(const pf_gemm_desc& d, int xt) {
-  const int bk = xt == PF_XT_256x256 ? 32 : 64;
+  const int bk = (xt == PF_XT_256x256 || xt == PF_XT_192x256) ? 32 : 64;
+  if (xt == PF_XT_192x256 && d.a_trans) return false;   // no reduction-strided 192-row tile
   if (d.a_trans != d.b_trans) return false;
   if (!d.a_trans && d.K % bk != 0) return false;
   return d.K >= bk;
@@ -479,7 +480,7 @@ template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
   const int v = resolve_variant(d);
   switch (v) {
-    case V_X256: case V_X256x128: case V_X128: {
+    case V_X256: case V_X256x128: case V_X128: case V_X192x256: {
       const int xt = v;   // variant ids 1..5 are the PF_XT_* tile ids
       if (!x_supports(d, xt)) {
         pf_set_error("pf_gemm: variant %d needs both operands stored alike and (unless transposed) K a multiple of the stage depth", v);
@@ -623,8 +624,9 @@ extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   const char* bt = d.b_trans ? "true" : "false";
   const int v = resolve_variant(d);
   switch (v) {
-    case V_X256: case V_X256x128: case V_X128: {
-      static const char* shapes[PF_XT_COUNT] = {"", "256, 256, 32, 2, 2, 5", "256, 128, 64, 2, 2, 3", "128, 128, 64, 2, 2, 3"};
+    case V_X256: case V_X256x128: case V_X128: case V_X192x256: {
+      static const char* shapes[PF_XT_COUNT] = {"", "256, 256, 32, 2, 2, 5", "256, 128, 64, 2, 2, 3", "128, 128, 64, 2, 2, 3",
+                                                "192, 256, 32, 2, 2, 5"};
       int ec = epi_class(d, epi_vec_ok(d));
       if (d.a_trans && ec != EC_ACC32 && ec != EC_STORE32) ec = EC_GENERIC;
       snprintf(out, (size_t)cap, "gemm16x_kernel<%d, %s, %s, %s, %d>", d.in_dtype, shapes[v], at, bt, ec);

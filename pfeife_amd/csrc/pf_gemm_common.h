@@ -173,7 +173,7 @@ __device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t b
 // Tile shapes of the direct-to-LDS kernel (BM x BN; reduction depth per stage, stages):
 //   256x256 (32 deep, 5 stages): one 128x128 block per wavefront, the least operand traffic per FLOP
 //   256x128 (64 deep, 3 stages), 128x128 (64 deep, 3 stages): more workgroups for smaller outputs
-enum { PF_XT_256x256 = 1, PF_XT_256x128 = 2, PF_XT_128x128 = 3, PF_XT_COUNT = 4 };
+enum { PF_XT_256x256 = 1, PF_XT_256x128 = 2, PF_XT_128x128 = 3, PF_XT_192x256 = 4, PF_XT_COUNT = 5 };
 
 // Epilogue classes with straight-line code (which operands exist, and their dtypes, fixed at
 // compile time).  Everything else takes EC_GENERIC: one rolled loop with runtime switches.

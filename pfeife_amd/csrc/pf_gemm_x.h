@@ -700,6 +700,7 @@ int gemm_x_launch(const pf_gemm_desc& d, int tile, hipStream_t st) {
     case PF_XT_256x256: return launch16x<DT, 256, 256, 32, 2, 2, 5>(d, st);
     case PF_XT_256x128: return launch16x<DT, 256, 128, 64, 2, 2, 3>(d, st);
     case PF_XT_128x128: return launch16x<DT, 128, 128, 64, 2, 2, 3>(d, st);
+    case PF_XT_192x256: return launch16x<DT, 192, 256, 32, 2, 2, 5>(d, st);
     default: pf_set_error("pf_gemm: unknown direct-to-LDS tile %d", tile); return PF_ERR_INVALID;
   }
 }

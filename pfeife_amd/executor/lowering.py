@@ -231,9 +231,13 @@ class BufferPool:
         self._scratch = {}
         self._bwd = {}
         self.bytes = 0
+        # Jobs of different pipeline ranks may run at the same time on streams of their own;
+        # the worker sets `lane` to the rank whose stage is being lowered, and every shared
+        # buffer is shared within a lane only.
+        self.lane = 0
 
     def scratch(self, slot, shape, dtype):
-        key = (slot, tuple(shape), dtype)
+        key = (self.lane, slot, tuple(shape), dtype)
         t = self._scratch.get(key)
         if t is None:
             t = torch.empty(tuple(shape), dtype=dtype, device=self.device)
@@ -242,10 +246,10 @@ class BufferPool:
         return t
 
     def bwd_like(self, seq, like):
-        """Buffer number `seq` of a backward job.  Backward jobs never overlap in
+        """Buffer number `seq` of a backward job.  Backward jobs of one lane never overlap in
         time (one stream, one job at a time) and their temporaries die with the
-        job, so all stages and micro-batches share one set of buffers."""
-        key = (seq, tuple(like.shape), tuple(like.stride()), like.dtype)
+        job, so all stages and micro-batches of a lane share one set of buffers."""
+        key = (self.lane, seq, tuple(like.shape), tuple(like.stride()), like.dtype)
         t = self._bwd.get(key)
         if t is None:
             t = torch.empty_like(like, device=self.device)

@@ -149,6 +149,7 @@ class PartialRunner:
             worker.run_job(stage, mb, is_fwd)
             if is_fwd and worker.last_forward.get(i) == mb:
                 self.finalize_output(mb)
+        worker.end_jobs()
         worker.optimizer_step()
         worker.steps_done += 1
         return self._take_results()
@@ -160,12 +161,14 @@ class PartialRunner:
     def finalize_output(self, batch_idx):
         """Wake micro-batch `batch_idx`: its outputs exist; wait until its exec_fn has
         returned (loss computed, backward hooks fired)."""
+        self.worker.outputs_ready(batch_idx)
         PartialModule._module_queues[batch_idx].put(None)
         ret = self._return_queues[batch_idx].get()
         self._parked.discard(batch_idx)
         if isinstance(ret, _ExecError):
             raise ret.exc
         self.worker.finish_micro_batch(batch_idx)
+        self.worker.loss_grads_ready(batch_idx)
         self.results.append(ret)
 
     def backward_hook(self, batch_idx, output_idx, grad):

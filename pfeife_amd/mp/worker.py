@@ -65,6 +65,13 @@ class StageWorker:
         self.graphs_ready = False
         self.steps_done = 0
         self.begin_graph = None
+        # One stream per pipeline rank ("lane"): the jobs of different ranks are independent by
+        # construction of the schedule (that is what lets the reference run them on different
+        # GPUs), so on one GPU they run side by side and fill the CUs and launch gaps that a
+        # single job's kernels leave idle.  rank -> torch.cuda.Stream; None: everything on stream_obj.
+        self.lanes = None
+        self._job_events = {}
+        self._loss_events = {}
         # dynamic loss scaling: {scale, growth tracker, found_inf, completed steps, 4 scratch} on the device
         self.dyn_scale = option.loss_scale == "dynamic"
         self.scaler_state = None
@@ -111,11 +118,38 @@ class StageWorker:
         self.sched_params = PipeSchedParams(device_cnt, opt.batch_cnt, node_cnt, loop_batch, prefetch)
         self.scheduler = SingleCommScheduler(self.sched_params)
         self.order = serialize_ranks(self.sched_params.rank_works, node_cnt)
+        self._setup_lanes(pg, device_cnt)
         last = {}
         for i, (stage, mb, is_fwd) in enumerate(self.order):
             if is_fwd:
                 last[mb] = i
         self.last_forward = {i: mb for mb, i in last.items()}
+
+    def _setup_lanes(self, pg, device_cnt):
+        """Decide whether the ranks get streams of their own.  They do not when a parameter is
+        read by stages of two ranks (its gradient accumulator would be updated from two streams
+        at once) or when PFEIFE_NO_LANES=1."""
+        self.lanes = None
+        self._job_events = {}
+        self._loss_events = {}
+        if self.stream_obj is None or device_cnt < 2 or os.environ.get("PFEIFE_NO_LANES", "0") == "1":
+            return
+        owner = {}
+        for st in pg.nodes.values():
+            for gi in st.input_placeholder:
+                v = pg.static_vals.get(gi) if gi >= 0 else None
+                if v is None or not v.req_grad:
+                    continue
+                key = v.buf.untyped_storage().data_ptr()
+                if owner.setdefault(key, st.rank) != st.rank:
+                    self.log.info("parameter %s is shared by two pipeline ranks: single-stream execution", v.name)
+                    return
+        main_rank = pg.nodes[max(pg.nodes)].rank   # user code (loss, hooks) follows the last stage
+        self.main_rank = main_rank
+        self.lanes = {r: (self.stream_obj if r == main_rank else torch.cuda.Stream(self.device))
+                      for r in range(device_cnt)}
+        # which stages hand a value to user code / receive a loss gradient from it
+        self._output_stages = sorted({ref[0] for ref in pg.outputs if isinstance(ref[0], int)})
 
     def stage_parameters(self):
         seen, out = set(), []
@@ -169,6 +203,7 @@ class StageWorker:
                         ins.append(bv)
                     else:
                         ins.append(pv)
+            self.pool.lane = st.rank if self.lanes is not None else 0
             prog = L.lower_forward(st, mb, ins)
             slot.stage_programs[sid] = prog
             stage_out[sid] = prog.outputs
@@ -199,7 +234,9 @@ class StageWorker:
             for oi, ref in enumerate(pg.outputs):
                 if ref[0] == sid and oi in slot.loss_grads:
                     out_grads[ref[1]].append(slot.loss_grads[oi])
+            self.pool.lane = st.rank if self.lanes is not None else 0
             L.lower_backward(prog, out_grads)
+        self.pool.lane = 0
         self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
         self.mbs[mb] = slot
         self.graphs_ready = False   # new programs (and possibly new parameters): capture again
@@ -234,6 +271,9 @@ class StageWorker:
         self.graphs_ready = False
         self.static_inputs = {}
         self.part_graph = None
+        self.lanes = None
+        self._job_events = {}
+        self._loss_events = {}
         self.optimizer = None
         self.params = ParamStore(self.kernels, self.device)
         self.pool = BufferPool(self.device)
@@ -276,6 +316,7 @@ class StageWorker:
 
     def begin_step(self):
         s = self.stream()
+        self.end_jobs()   # a step that failed half-way may have left lanes running
         self.params.rebind_grads()
         if self.use_graphs and not self.graphs_ready and self.steps_done >= 1 and len(self.mbs) == self.option.batch_cnt:
             self.capture_graphs()
@@ -288,6 +329,44 @@ class StageWorker:
                 launch(s)
         for slot in self.mbs.values():
             slot.grad_seen.clear()
+        if self.lanes is not None:   # zeroed gradients, fresh shadows and the step's inputs are in place
+            for r, lane in self.lanes.items():
+                if lane is not self.stream_obj:
+                    lane.wait_stream(self.stream_obj)
+
+    # -- lanes -------------------------------------------------------------------------
+    def _event(self, table, key):
+        ev = table.get(key)
+        if ev is None:
+            ev = table[key] = torch.cuda.Event()
+        return ev
+
+    def outputs_ready(self, mb):
+        """User code of micro-batch `mb` is about to read the graph outputs on the main stream."""
+        if self.lanes is None:
+            return
+        pg = self.part_graph
+        for sid in self._output_stages:
+            if self.lanes[pg.nodes[sid].rank] is not self.stream_obj:
+                ev = self._job_events.get((sid, mb, True))
+                if ev is not None:
+                    self.stream_obj.wait_event(ev)
+
+    def loss_grads_ready(self, mb):
+        """The loss gradients of micro-batch `mb` have been written (on the main stream)."""
+        if self.lanes is None:
+            return
+        pg = self.part_graph
+        if any(self.lanes[pg.nodes[sid].rank] is not self.stream_obj for sid in self._output_stages):
+            self._event(self._loss_events, mb).record(self.stream_obj)
+
+    def end_jobs(self):
+        """Every lane's work precedes what follows on the main stream (the optimizer step)."""
+        if self.lanes is None:
+            return
+        for lane in self.lanes.values():
+            if lane is not self.stream_obj:
+                self.stream_obj.wait_stream(lane)
 
     def recv_loss_grad(self, mb, out_idx, grad):
         slot = self.mbs[mb]
@@ -328,10 +407,38 @@ class StageWorker:
 
     def run_job(self, stage, mb, is_fwd):
         prog = self.mbs[mb].stage_programs[stage]
+        if self.lanes is None:
+            if is_fwd:
+                prog.run_forward(self.stream())
+            else:
+                prog.run_backward(self.stream())
+            return
+        # the job goes to its rank's stream, after the jobs of other ranks whose results it reads:
+        # forward after the producers of its inputs, backward after the consumers of its outputs
+        pg = self.part_graph
+        st = pg.nodes[stage]
+        lane = self.lanes[st.rank]
         if is_fwd:
-            prog.run_forward(self.stream())
+            deps = {src[0] for src in st.input_source if src is not None}
         else:
-            prog.run_backward(self.stream())
+            deps = {t.idx for t in pg.nodes.values()
+                    if any(src is not None and src[0] == stage for src in t.input_source)}
+        for other in sorted(deps):
+            if self.lanes[pg.nodes[other].rank] is not lane:
+                ev = self._job_events.get((other, mb, is_fwd))
+                if ev is None:
+                    raise RuntimeError("job order: stage %d of micro-batch %d runs before stage %d (%s)"
+                                       % (stage, mb, other, "forward" if is_fwd else "backward"))
+                lane.wait_event(ev)
+        if not is_fwd and lane is not self.stream_obj and stage in self._output_stages:
+            ev = self._loss_events.get(mb)
+            if ev is not None:
+                lane.wait_event(ev)
+        if is_fwd:
+            prog.run_forward(lane.cuda_stream)
+        else:
+            prog.run_backward(lane.cuda_stream)
+        self._event(self._job_events, (stage, mb, is_fwd)).record(lane)
 
     def init_optimizer(self, optimizer):
         if optimizer is not None:
