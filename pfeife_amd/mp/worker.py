@@ -70,6 +70,7 @@ class StageWorker:
         # GPUs), so on one GPU they run side by side and fill the CUs and launch gaps that a
         # single job's kernels leave idle.  rank -> torch.cuda.Stream; None: everything on stream_obj.
         self.lanes = None
+        self.lane_mode = "0"
         self._job_events = {}
         self._loss_events = {}
         # dynamic loss scaling: {scale, growth tracker, found_inf, completed steps, 4 scratch} on the device
@@ -125,14 +126,28 @@ class StageWorker:
                 last[mb] = i
         self.last_forward = {i: mb for mb, i in last.items()}
 
+    def _lane_key(self, stage, is_fwd):
+        rank = self.part_graph.nodes[stage].rank
+        return (rank, is_fwd) if self.lane_mode == "rankdir" else (rank, False)
+
     def _setup_lanes(self, pg, device_cnt):
-        """Decide whether the ranks get streams of their own.  They do not when a parameter is
-        read by stages of two ranks (its gradient accumulator would be updated from two streams
-        at once) or when PFEIFE_NO_LANES=1."""
+        """Decide which jobs get streams of their own.  PFEIFE_LANES = "rank": one stream per
+        pipeline rank; "rankdir" (default): per rank one for its forward and one for its backward
+        jobs (forward jobs read parameters only, so they may run ahead of the rank's backward jobs;
+        backward jobs of a rank stay in schedule order on one stream, which fixes the order in
+        which micro-batches are summed into a parameter's gradient); "0": a single stream.
+        A single stream is also used when a parameter is read by stages of two ranks (its
+        gradient accumulator would be updated from two streams at once)."""
         self.lanes = None
         self._job_events = {}
         self._loss_events = {}
-        if self.stream_obj is None or device_cnt < 2 or os.environ.get("PFEIFE_NO_LANES", "0") == "1":
+        mode = os.environ.get("PFEIFE_LANES", "rankdir")
+        if os.environ.get("PFEIFE_NO_LANES", "0") == "1":
+            mode = "0"
+        if mode not in ("0", "rank", "rankdir"):
+            raise RuntimeError("PFEIFE_LANES must be 0, rank or rankdir, not %r" % mode)
+        self.lane_mode = mode
+        if self.stream_obj is None or mode == "0" or (device_cnt < 2 and mode == "rank"):
             return
         owner = {}
         for st in pg.nodes.values():
@@ -144,10 +159,11 @@ class StageWorker:
                 if owner.setdefault(key, st.rank) != st.rank:
                     self.log.info("parameter %s is shared by two pipeline ranks: single-stream execution", v.name)
                     return
-        main_rank = pg.nodes[max(pg.nodes)].rank   # user code (loss, hooks) follows the last stage
-        self.main_rank = main_rank
-        self.lanes = {r: (self.stream_obj if r == main_rank else torch.cuda.Stream(self.device))
-                      for r in range(device_cnt)}
+        # user code (loss, hooks) and the optimizer run on stream_obj, which is also the lane of
+        # the last stage's backward jobs: they read the loss gradients user code writes
+        main_key = self._lane_key(max(pg.nodes), False)
+        keys = sorted({self._lane_key(sid, d) for sid in pg.nodes for d in (True, False)})
+        self.lanes = {k: (self.stream_obj if k == main_key else torch.cuda.Stream(self.device)) for k in keys}
         # which stages hand a value to user code / receive a loss gradient from it
         self._output_stages = sorted({ref[0] for ref in pg.outputs if isinstance(ref[0], int)})
 
@@ -203,7 +219,7 @@ class StageWorker:
                         ins.append(bv)
                     else:
                         ins.append(pv)
-            self.pool.lane = st.rank if self.lanes is not None else 0
+            self.pool.lane = self._lane_key(sid, True) if self.lanes is not None else 0
             prog = L.lower_forward(st, mb, ins)
             slot.stage_programs[sid] = prog
             stage_out[sid] = prog.outputs
@@ -234,7 +250,7 @@ class StageWorker:
             for oi, ref in enumerate(pg.outputs):
                 if ref[0] == sid and oi in slot.loss_grads:
                     out_grads[ref[1]].append(slot.loss_grads[oi])
-            self.pool.lane = st.rank if self.lanes is not None else 0
+            self.pool.lane = self._lane_key(sid, False) if self.lanes is not None else 0
             L.lower_backward(prog, out_grads)
         self.pool.lane = 0
         self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
@@ -330,7 +346,7 @@ class StageWorker:
         for slot in self.mbs.values():
             slot.grad_seen.clear()
         if self.lanes is not None:   # zeroed gradients, fresh shadows and the step's inputs are in place
-            for r, lane in self.lanes.items():
+            for lane in self.lanes.values():
                 if lane is not self.stream_obj:
                     lane.wait_stream(self.stream_obj)
 
@@ -345,9 +361,8 @@ class StageWorker:
         """User code of micro-batch `mb` is about to read the graph outputs on the main stream."""
         if self.lanes is None:
             return
-        pg = self.part_graph
         for sid in self._output_stages:
-            if self.lanes[pg.nodes[sid].rank] is not self.stream_obj:
+            if self.lanes[self._lane_key(sid, True)] is not self.stream_obj:
                 ev = self._job_events.get((sid, mb, True))
                 if ev is not None:
                     self.stream_obj.wait_event(ev)
@@ -356,8 +371,7 @@ class StageWorker:
         """The loss gradients of micro-batch `mb` have been written (on the main stream)."""
         if self.lanes is None:
             return
-        pg = self.part_graph
-        if any(self.lanes[pg.nodes[sid].rank] is not self.stream_obj for sid in self._output_stages):
+        if any(self.lanes[self._lane_key(sid, False)] is not self.stream_obj for sid in self._output_stages):
             self._event(self._loss_events, mb).record(self.stream_obj)
 
     def end_jobs(self):
@@ -417,15 +431,16 @@ class StageWorker:
         # forward after the producers of its inputs, backward after the consumers of its outputs
         pg = self.part_graph
         st = pg.nodes[stage]
-        lane = self.lanes[st.rank]
+        lane = self.lanes[self._lane_key(stage, is_fwd)]
         if is_fwd:
-            deps = {src[0] for src in st.input_source if src is not None}
+            deps = {(src[0], True) for src in st.input_source if src is not None}
         else:
-            deps = {t.idx for t in pg.nodes.values()
+            deps = {(t.idx, False) for t in pg.nodes.values()
                     if any(src is not None and src[0] == stage for src in t.input_source)}
-        for other in sorted(deps):
-            if self.lanes[pg.nodes[other].rank] is not lane:
-                ev = self._job_events.get((other, mb, is_fwd))
+            deps.add((stage, True))    # its own forward (which followed the producers of its inputs)
+        for other, d in sorted(deps):
+            if self.lanes[self._lane_key(other, d)] is not lane:
+                ev = self._job_events.get((other, mb, d))
                 if ev is None:
                     raise RuntimeError("job order: stage %d of micro-batch %d runs before stage %d (%s)"
                                        % (stage, mb, other, "forward" if is_fwd else "backward"))
