@@ -19,6 +19,7 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"fp16": 2500.0, "bf16": 2500.0, "fp32": 157.3}
 PEAK_HBM_GBS = 8000.0
+AUTO_SPLIT = False   # --auto-split: split_points=None, the planner picks the stage boundaries
 
 
 def log(*a):
@@ -68,8 +69,14 @@ def build_workload(name, device):
         model = llama.LlamaForCausalLM(cfg)
         inputs = (torch.randint(0, cfg.vocab, (batch, cfg.max_seq), generator=g),)
     initialize_pfeife()
-    option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
-                        split_points=splits or None, mixed_precision=mixed, optimizer=dict(type="adam", lr=1e-5))
+    if AUTO_SPLIT and splits:
+        # same stage count, boundaries chosen by the auto-partitioner from a profile on this GPU
+        option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
+                            split_points=None, loop_cnt=(len(splits) + 1) // device_cnt, mixed_precision=mixed,
+                            optimizer=dict(type="adam", lr=1e-5))
+    else:
+        option = PipeOption(device_cnt=device_cnt, batch_cnt=batch_cnt, batch_size=batch // batch_cnt,
+                            split_points=splits or None, mixed_precision=mixed, optimizer=dict(type="adam", lr=1e-5))
     runner = PartialRunner(option)
     model.to(device)
     cmodel = torch.compile(model, backend=partial_compiler)
@@ -385,12 +392,17 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
                100 * r["frac"], PEAK_HBM_GBS, "" if r["on_path"] else "  [off-path micro-benchmark]"))
     flops_step = model_flops_per_step(info)
     cfg = info["cfg"]
+    plan = getattr(w, "plan", None)
+    used = getattr(w.part_graph, "nodes", {})
+    splits_txt = ("%s (compute-node indices chosen by the auto-partitioner, expected %.1f ms/step for one rank per GPU)"
+                  % (plan.split_points, plan.expect_ms)) if plan is not None else str(info["splits"])
+    lanes = "%d streams (%s)" % (len(w.lanes), w.lane_mode) if w.lanes else "one stream"
     res = dict(value=value, ms=ms, host_ms=host_ms, roof=roof, hbm=rates, info=info, loss_scaling=scaling,
                model_tflops=None if flops_step is None else round(flops_step / (ms * 1e-3) / 1e12, 2),
                workload="%s: %s micro-batch %d x %d, %d stages split at %s, schedule drawn for %d ranks, "
-                        "all stages on one GPU, Adam" % (
+                        "all stages on one GPU on %s, Adam" % (
                             name, type(cfg).__name__, info["batch"] // info["batch_cnt"], info["batch_cnt"],
-                            len(info["splits"]) + 1, info["splits"], info["device_cnt"]))
+                            len(used), splits_txt, info["device_cnt"], lanes))
     return runner, res
 
 
@@ -424,7 +436,12 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain copy kernel (ew_kernel<Scale>, 256 MiB read + 256 MiB written) three "
                          "times, as the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
+    ap.add_argument("--auto-split", action="store_true",
+                    help="pass split_points=None: the auto-partitioner profiles the model on the GPU and picks "
+                         "the stage boundaries (same stage count as the workload's manual split)")
     args = ap.parse_args()
+    global AUTO_SPLIT
+    AUTO_SPLIT = args.auto_split
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs every pipeline stage on ONE GPU; --gpus %d is not supported "
               "(no collectives, no second device)." % args.gpus, file=sys.stderr)

@@ -277,6 +277,11 @@ class StageProgram:
         self.tile_groups = []   # sibling regions that must all be written for the zero-fill to be skipped
         self.fwd_graph = None   # replay callables once the launch lists have been captured
         self.bwd_graph = None
+        # which launches belong to which graph node (the partitioner's profiler times them):
+        # (node name, first launch, one past the last launch[, forward bytes allocated])
+        self.fwd_ranges = []
+        self.bwd_ranges = []
+        self.backward_nodes = []  # node name per entry of backward_fns
 
     def run_forward(self, stream):
         if self.fwd_graph is not None:
@@ -594,18 +599,22 @@ class Lowerer:
                 outs = list(res) if isinstance(res, (tuple, list)) else [res]
                 prog.outputs = [self.arg(o) for o in outs]
                 continue
+            first, bytes0 = len(prog.fwd), prog.fwd_bytes
+            self.cur_node = node.name
             if node in self.fused:
                 self.env[node] = self.fused[node]
-                continue
-            if node in self.pattern_skip:
-                continue  # interior of a matched multi-node pattern, produced by the pattern's root
-            if node in self.patterns:
-                out = lower_rope(self, node, *self.patterns[node])
+            elif node in self.pattern_skip:
+                pass  # interior of a matched multi-node pattern, produced by the pattern's root
             else:
-                out = self._handler(node)(self, node)
-            self.env[node] = out
-            if isinstance(out, Val) and not out.name:
-                out.name = node.name
+                if node in self.patterns:
+                    out = lower_rope(self, node, *self.patterns[node])
+                else:
+                    out = self._handler(node)(self, node)
+                self.env[node] = out
+                if isinstance(out, Val) and not out.name:
+                    out.name = node.name
+            if node.op != "get_attr":
+                prog.fwd_ranges.append((node.name, first, len(prog.fwd), prog.fwd_bytes - bytes0))
         self.cur = None
         return prog
 
@@ -618,11 +627,16 @@ class Lowerer:
                 continue
             for g in ([gs] if torch.is_tensor(gs) else gs):  # several consumers: fan-out sum
                 B.contribute(v, g)
-        for fn in reversed(prog.backward_fns):
+        for fn, name in zip(reversed(prog.backward_fns), reversed(prog.backward_nodes)):
+            first = len(prog.bwd)
             fn(B)
+            prog.bwd_ranges.append((name, first, len(prog.bwd)))
+        first = len(prog.bwd)
         B.flush_dw()
         if B.reduces:
             prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
+        if prog.bwd_ranges and len(prog.bwd) > first:   # held-back tail: charged to the job's last node
+            prog.bwd_ranges.append((prog.bwd_ranges[-1][0], first, len(prog.bwd)))
         prog.input_grads = []
         for v in prog.inputs:
             if isinstance(v, Val) and v.req_grad and v.param is None:
@@ -647,6 +661,7 @@ class Lowerer:
 
     def add_backward(self, fn):
         self.cur.backward_fns.append(fn)
+        self.cur.backward_nodes.append(getattr(self, "cur_node", ""))
 
     def _handler(self, node):
         if node.op == "call_function":

@@ -278,8 +278,18 @@ class PartialModule(nn.Module):
         ex = self.example_inputs if self.example_inputs is not None else list(args)
         # module state is identified on the real call arguments (they are the live tensors)
         live = list(args)
-        self.partition_graph = partition_by_split_points(self.gm, live, option.split_points, option.device_cnt)
+        points = option.split_points
+        plan = None
+        if self.alias_of is not None:
+            points = self.alias_of.split_points_used      # same pipeline, another micro-batch shape
+        elif points is None and option.device_cnt > 1:
+            plan = worker.plan_split_points(self.gm, live)
+            points = plan.split_points
+        self.split_points_used = points
+        self.partition_graph = partition_by_split_points(self.gm, live, points, option.device_cnt)
         if option.print_graph:
+            if plan is not None:
+                print(plan.describe())
             self.partition_graph.print_graph()
             for idx, st in self.partition_graph.nodes.items():
                 print("================ PARTITION GRAPH %d: %d nodes ================"

@@ -17,7 +17,7 @@ import os
 
 import torch
 
-from ..executor.lowering import BufferPool, Lowerer, ParamStore
+from ..executor.lowering import BufferPool, Lowerer, ParamStore, Unsupported
 from ..executor.values import Val
 from ..option import get_optimizer_cls
 from ..schedule.scheduler import PipeSchedParams, SingleCommScheduler, StepWork, serialize_ranks
@@ -167,6 +167,21 @@ class StageWorker:
         # which stages hand a value to user code / receive a loss gradient from it
         self._output_stages = sorted({ref[0] for ref in pg.outputs if isinstance(ref[0], int)})
 
+    def plan_split_points(self, gm, live_args):
+        """`split_points=None`: profile the captured graph on this device and let the planner pick
+        the stage boundaries (pfeife/schedule/planner.py:667-815 in the reference)."""
+        from ..graph.profile import profile_graph
+        from ..schedule.planner import plan_split
+
+        opt = self.option
+        prof = profile_graph(self.kernels, self.device, opt.mixed_precision, gm, live_args, stream=self.stream())
+        n_nodes = prof.n
+        device_cnt = max(1, min(opt.device_cnt, n_nodes))
+        plan = plan_split(prof, opt, device_cnt)
+        self.plan, self.profile = plan, prof
+        self.log.info("auto-partitioner: %s", plan.describe().replace("\n", "; "))
+        return plan
+
     def stage_parameters(self):
         seen, out = set(), []
         for v in self.static_inputs.values():
@@ -217,6 +232,12 @@ class StageWorker:
                         bv = Val(pv.buf, req_grad=pv.req_grad, name=name)  # same storage: the handoff is a pointer
                         bv.boundary = True
                         ins.append(bv)
+                    elif isinstance(pv, (list, tuple)) and any(isinstance(e, Val) for e in pv):
+                        # its gradient would have to travel back as a tuple as well; the stage
+                        # programs hand over single tensors only
+                        raise Unsupported("the split point in front of stage %d cuts between '%s' (a tuple of "
+                                          "tensors) and its users; move it before the node that makes the tuple "
+                                          "or after the nodes that take it apart" % (sid, name))
                     else:
                         ins.append(pv)
             self.pool.lane = self._lane_key(sid, True) if self.lanes is not None else 0

@@ -191,6 +191,30 @@ def test_integer_split_points_on_device():
     assert all(len(slot.stage_programs) == 2 for slot in runner.worker.mbs.values())
 
 
+@pytest.mark.parametrize("mixed", [None, "fp16"])
+def test_auto_partition_split_points_none(mixed):
+    """split_points=None with two pipeline ranks: the captured graph is profiled on the device
+    (HIP events around each node's launches) and the planner picks the stage boundaries
+    (pfeife/schedule/planner.py:667-815, pfeife/local/graph_bench.py:390-625).  Wherever the
+    boundary falls, the step must equal plain gradient accumulation."""
+    from pfeife_amd.bench_models.vit import ViTConfig
+    from pfeife_amd.schedule.planner import cut_candidates
+
+    cfg = ViTConfig(image_size=64, patch_size=16, dim=128, depth=6, heads=4, mlp_dim=256, num_classes=16)
+    m, r, l, rl, runner = _run_vit(cfg, 8, 4, None, mixed, device_cnt=2, oracle_device="cuda" if mixed else "cpu")
+    _check(m, r, l, rl, mixed)
+    w = runner.worker
+    plan, prof = w.plan, w.profile
+    assert len(w.part_graph.nodes) == w.sched_params.node_cnt == len(plan.split_points) + 1 >= 2
+    assert all(p in cut_candidates(prof) for p in plan.split_points)
+    assert all(t >= 0 for t in prof.fwd_ms + prof.bwd_ms) and sum(prof.fwd_ms) > 0 and sum(prof.bwd_ms) > sum(prof.fwd_ms) * 0.5
+    # the stages are balanced: no stage carries more than its share plus one block of the work
+    total = sum(plan.stage_fwd_ms) + sum(plan.stage_bwd_ms)
+    per_block = total / cfg.depth
+    for f, b in zip(plan.stage_fwd_ms, plan.stage_bwd_ms):
+        assert f + b <= total / len(plan.stage_fwd_ms) + 1.5 * per_block
+
+
 def test_vit_single_stage_and_repeatability():
     from pfeife_amd.bench_models.vit import ViTConfig
 

@@ -1,0 +1,297 @@
+"""Auto-partitioner (split_points=None): the oracle's restatement of the reference's pipeline
+valuation is pinned by closed forms and hand-worked cases; the product's cost model and search
+are checked against it; the whole path runs on the host with the kernel double."""
+import copy
+import random
+
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import planner_oracle as po
+from pfeife_amd.graph.profile import GraphProfile, cut_sizes
+from pfeife_amd.schedule.planner import CostModel, LinkModel, cut_candidates, plan_split, search_points
+from pfeife_amd.schedule.scheduler import PipeSchedParams
+
+
+# ---------------------------------------------------------------------------
+# the oracle itself
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("D,B", [(2, 4), (3, 6), (4, 8), (4, 4)])
+def test_oracle_equal_stages_closed_form(D, B):
+    # one-forward-one-backward over D equal stages: (B + D - 1) slots of (f + b), then the optimizer
+    f, b, o = 1.5, 3.25, 0.5
+    sched = PipeSchedParams(D, B, D, D, 0)
+    ranks = list(range(D))
+    v = po.pipe_value([f] * D, [b] * D, [o] * D, ranks, sched.rank_works, B, po.chain_edges(D, ranks, [0.0] * D))
+    assert v == pytest.approx((B + D - 1) * (f + b) + o)
+
+
+def test_oracle_single_stage_is_the_plain_sum():
+    sched = PipeSchedParams(1, 5, 1, 1, 0)
+    v = po.pipe_value([2.0], [3.0], [0.7], [0], sched.rank_works, 5, [])
+    assert v == pytest.approx(5 * (2.0 + 3.0) + 0.7)
+
+
+def test_oracle_hand_worked_two_unequal_stages_with_transfer():
+    # stage 0: f 1, b 2 (rank 0); stage 1: f 3, b 4 (rank 1); transfer 0.5 each way; B = 2
+    # rank 0: F00 [0,1] F01 [1,2] ; rank 1: F10 starts 1.5 -> 4.5, B10 -> 8.5, F11 -> 11.5, B11 -> 15.5
+    # rank 0: B00 needs B10 + 0.5 = 9 -> 11 ; B01 needs B11 + 0.5 = 16 -> 18 ; + optimizer of rank 0 (0.25)
+    sched = PipeSchedParams(2, 2, 2, 2, 0)
+    assert sched.rank_works[0] == [(0, 0, True), (0, 1, True), (0, 0, False), (0, 1, False)]
+    assert sched.rank_works[1] == [(1, 0, True), (1, 0, False), (1, 1, True), (1, 1, False)]
+    v, dist = po.pipe_value([1.0, 3.0], [2.0, 4.0], [0.25, 0.125], [0, 1], sched.rank_works, 2,
+                            [(0, 1, 0.5)], return_dist=True)
+    assert dist[(1, 0, True)] == pytest.approx(1.5)
+    assert dist[(1, 1, False)] == pytest.approx(11.5)
+    assert dist[(0, 0, False)] == pytest.approx(9.0)
+    assert dist[(0, 1, False)] == pytest.approx(16.0)
+    assert v == pytest.approx(18.25)
+
+
+def test_oracle_peak_memory_hand_trace():
+    # one rank, stage 0 (act 10, temp 14) and stage 1 (act 3, temp 8), weights 100
+    works = [[(0, 0, True), (1, 0, True), (0, 1, True), (1, 0, False), (0, 0, False), (1, 1, True),
+              (1, 1, False), (0, 1, False)]]
+    # cur: 100 ->F0 peak 114, cur 110 ->F1 peak 118, cur 113 ->F0 peak 127, cur 123
+    #      ->B1 peak 123+5=128, cur 120 ->B0 peak 124, cur 110 -> F1 peak 118 ...
+    assert po.peak_memory([100], [10, 3], [14, 8], works) == [128]
+
+
+# ---------------------------------------------------------------------------
+# product cost model against the oracle
+# ---------------------------------------------------------------------------
+def random_profile(rng, n, uniform_cuts=True):
+    p = GraphProfile()
+    for i in range(n):
+        p.names.append("n%d" % i)
+        p.fwd_ms.append(rng.uniform(0.01, 1.0))
+        p.bwd_ms.append(rng.uniform(0.02, 2.0))
+        p.act_bytes.append(rng.randrange(0, 1 << 20))
+        p.param_bytes.append(rng.randrange(0, 1 << 18))
+    p.cut_bytes = [0] + [(1000 if uniform_cuts else rng.randrange(500, 4000)) for _ in range(n - 1)] + [0]
+    p.cut_values = [0] + [1] * (n - 1) + [0]
+    p.temp_bytes = 12345
+    return p
+
+
+def oracle_value(prof, points, sched, link):
+    model = CostModel(prof, link)
+    rows = model.stages(points)
+    S = len(rows)
+    ranks = [s % sched.device_cnt for s in range(S)]
+    send = [0.0] + [link.send_ms(prof.cut_bytes[p]) for p in points]
+    return po.pipe_value([r[0] for r in rows], [r[1] for r in rows], [r[2] for r in rows], ranks,
+                         sched.rank_works, sched.batch_cnt, po.chain_edges(S, ranks, send))
+
+
+@pytest.mark.parametrize("D,B,S,LB,PF", [(2, 4, 2, 2, 0), (2, 8, 4, 2, 0), (3, 6, 6, 3, 0), (4, 8, 4, 4, 1),
+                                         (2, 5, 6, 2, 0), (1, 3, 2, 1, 0)])
+def test_value_and_memory_equal_the_reference_valuation(D, B, S, LB, PF):
+    rng = random.Random(D * 100 + B * 10 + S)
+    sched = PipeSchedParams(D, B, S, LB, PF)
+    for trial in range(5):
+        prof = random_profile(rng, 40, uniform_cuts=False)
+        points = sorted(rng.sample(range(1, 40), S - 1))
+        for link in (LinkModel(), LinkModel(gbs=0.001, latency_ms=0.05)):
+            got = CostModel(prof, link).value(points, sched)
+            assert got == pytest.approx(oracle_value(prof, points, sched, link), rel=1e-12)
+        model = CostModel(prof)
+        idle, peak = model.memory(points, sched)
+        rows = model.stages(points)
+        act = [r[3] for r in rows]
+        temp = [a + prof.temp_bytes for a in act]
+        assert peak == [int(x) for x in po.peak_memory(idle, act, temp, sched.rank_works)]
+
+
+def test_search_finds_the_brute_force_optimum():
+    rng = random.Random(7)
+    for n, D, B, S in [(14, 2, 4, 2), (16, 2, 4, 4), (18, 3, 6, 3)]:
+        prof = random_profile(rng, n)
+        sched = PipeSchedParams(D, B, S, D, 0)
+        model = CostModel(prof)
+        cand = list(range(1, n))
+        want = po.brute_force_points(cand, S - 1, lambda pts: oracle_value(prof, pts, sched, LinkModel()))
+        for limit in (10 ** 9, 0):     # exhaustive, and the beam alone
+            v, pts, _ = search_points(model, sched, cand, exhaustive_limit=limit)
+            assert v == pytest.approx(want[0], rel=1e-9), (n, S, limit, pts, want)
+
+
+def test_beam_is_near_optimal_on_a_larger_graph():
+    rng = random.Random(11)
+    n, D, B, S = 48, 2, 8, 4
+    prof = random_profile(rng, n)
+    sched = PipeSchedParams(D, B, S, D, 0)
+    model = CostModel(prof)
+    cand = list(range(1, n))
+    want = po.brute_force_points(cand, S - 1, lambda pts: model.value(pts, sched))
+    v, pts, evaluated = search_points(model, sched, cand, exhaustive_limit=0)
+    assert v <= want[0] * 1.01
+    assert evaluated < 17296 / 4     # far fewer than the C(47, 3) candidates brute force values
+
+
+def test_memory_budget_rejects_splits():
+    rng = random.Random(3)
+    prof = random_profile(rng, 20)
+    prof.act_bytes = [1 << 20] * 20
+    sched = PipeSchedParams(2, 4, 2, 2, 0)
+    model = CostModel(prof)
+    v_free, pts_free, _ = search_points(model, sched, list(range(1, 20)))
+    _, peak = model.memory(pts_free, sched)
+    tight = [max(peak) - 1] * 2
+    v, pts, _ = search_points(model, sched, list(range(1, 20)), max_mem=tight)
+    if pts is not None and v != float("inf"):
+        _, p2 = model.memory(pts, sched)
+        assert all(a <= b for a, b in zip(p2, tight)) and v >= v_free
+
+
+def test_cut_sizes_on_a_residual_chain():
+    class Net(nn.Module):
+        def forward(self, x):
+            a = x * 2.0          # node 0
+            b = a + 1.0          # node 1
+            c = b * b            # node 2
+            d = c + a            # node 3: `a` crosses the cuts in front of nodes 1, 2, 3
+            return d.sum()       # node 4
+
+    gm = torch.fx.symbolic_trace(Net())
+    x = torch.zeros(4, 8)
+    env = {}
+    for node in gm.graph.nodes:          # example values, as TorchDynamo records them
+        if node.op == "placeholder":
+            env[node] = x
+        elif node.op == "call_function" or node.op == "call_method":
+            args = [env[a] if isinstance(a, torch.fx.Node) else a for a in node.args]
+            env[node] = node.target(*args) if node.op == "call_function" else getattr(args[0], node.target)(*args[1:])
+        if node in env:
+            node.meta["example_value"] = env[node]
+    cb, cc, ok = cut_sizes(gm)
+    assert cc == [0, 1, 2, 2, 1, 0]
+    assert cb == [0, 128, 256, 256, 128, 0]
+    assert ok == [True] * 6
+
+
+def test_a_tuple_may_not_cross_a_stage_boundary():
+    class Net(nn.Module):
+        def forward(self, x):
+            a = x * 2.0                 # node 0
+            parts = a.unbind(0)         # node 1: a tuple
+            b = parts[0] + parts[1]     # nodes 2, 3, 4
+            return b.sum()              # node 5
+
+    gm = torch.fx.symbolic_trace(Net())
+    x = torch.zeros(2, 8)
+    a = x * 2.0
+    vals = {"mul": a, "unbind": a.unbind(0)}
+    for node in gm.graph.nodes:
+        if node.name in vals:
+            node.meta["example_value"] = vals[node.name]
+    _, cc, ok = cut_sizes(gm)
+    assert ok[1] and not ok[2] and not ok[3]      # in front of the getitems the tuple would cross
+    p = GraphProfile()
+    p.names = ["n%d" % i for i in range(6)]
+    p.cut_values, p.cut_bytes, p.cut_ok = cc, [0] * 7, ok
+    assert all(ok[i] for i in cut_candidates(p))
+
+
+def test_cut_candidates_prefer_block_boundaries():
+    p = GraphProfile()
+    p.names = ["n%d" % i for i in range(9)]
+    p.cut_values = [0, 1, 3, 2, 1, 3, 2, 1, 3, 0]
+    p.cut_bytes = [0, 100, 300, 200, 100, 300, 200, 100, 300, 0]
+    assert cut_candidates(p, window=2) == [1, 4, 7]
+    # a cheaper cut far away (the classifier head) does not hide the block boundaries
+    p.cut_values = [0, 2, 3, 2, 4, 3, 2, 3, 1, 0]
+    p.cut_bytes = [0, 200, 300, 200, 400, 300, 200, 300, 10, 0]
+    assert cut_candidates(p, window=1) == [1, 3, 6, 8]
+
+
+# ---------------------------------------------------------------------------
+# end to end on the host: split_points=None
+# ---------------------------------------------------------------------------
+def test_split_points_none_profiles_and_partitions(capsys):
+    from oracle.kernels_oracle import OracleKernels
+    from oracle.stage_oracle import run_unpipelined
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.graph.partition_graph import compute_nodes
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife, net_states, partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=4, heads=4, mlp_dim=128, num_classes=10)
+    torch.manual_seed(0)
+    model = VisionTransformer(cfg)
+    ref = copy.deepcopy(model)
+    torch._dynamo.reset()
+    net_states._reset_state_for_tests()
+    initialize_pfeife(device="cpu")
+    option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=2, split_points=None, loop_cnt=1,
+                        optimizer=dict(type="sgd", lr=0.0), print_graph=True)
+    runner = PartialRunner(option, kernels=OracleKernels("cpu"))
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+
+    def fn(x, y):
+        loss = crit(cmodel(x).float(), y)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(8, 3, 32, 32, generator=g)
+    y = torch.randint(0, 10, (8,), generator=g)
+    losses = runner.step(x, y)
+    worker = runner.worker
+    plan, prof = worker.plan, worker.profile
+    assert len(plan.split_points) == 1 and len(worker.part_graph.nodes) == 2
+    assert prof.n == len(prof.fwd_ms) == len(prof.bwd_ms) and sum(prof.fwd_ms) > 0 and sum(prof.bwd_ms) > 0
+    # the cut is one of the low-traffic positions (a block boundary: only the residual stream crosses)
+    assert plan.split_points[0] in cut_candidates(prof)
+    # every parameter is charged to exactly one node
+    assert sum(prof.param_bytes) == sum(p.numel() * 4 for p in model.parameters())
+    text = capsys.readouterr().out
+    assert "split_points: [%d], expect time:" % plan.split_points[0] in text and "dev 1 - idle mem:" in text
+    # the profiling run leaves no gradient behind, and the step computes what plain accumulation computes
+    want = run_unpipelined(ref, crit, x, y, 4)
+    for a, b in zip(losses, want):
+        assert abs(float(a) - float(b)) <= 1e-5 * abs(float(b))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+
+
+def test_manual_split_between_a_tuple_and_its_users_is_refused():
+    from oracle.kernels_oracle import OracleKernels
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.executor.lowering import Unsupported
+    from pfeife_amd.graph.partition_graph import compute_nodes
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife, net_states, partial_compiler
+    from pfeife_amd.mp.partial.module import PartialModule
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=4, mlp_dim=128, num_classes=10)
+
+    def attempt(points):
+        torch.manual_seed(0)
+        model = VisionTransformer(cfg)
+        torch._dynamo.reset()
+        net_states._reset_state_for_tests()
+        initialize_pfeife(device="cpu")
+        option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=points,
+                            optimizer=dict(type="sgd", lr=0.0))
+        runner = PartialRunner(option, kernels=OracleKernels("cpu"))
+        cmodel = torch.compile(model, backend=partial_compiler)
+
+        def fn(x, y):
+            loss = nn.functional.cross_entropy(cmodel(x).float(), y)
+            loss.backward()
+            return loss.detach()
+
+        runner.set_exec_fn(fn)
+        runner.step(torch.randn(4, 3, 32, 32), torch.randint(0, 10, (4,)))
+        return PartialModule._pp_modules[0].gm
+
+    gm = attempt(["blocks.1"])
+    nodes = compute_nodes(gm)
+    idx = next(i for i, n in enumerate(nodes) if n.op == "call_function" and n.target.__name__ == "getitem"
+               and isinstance(n.args[0], torch.fx.Node) and n.args[0].target == "unbind")
+    with pytest.raises(Unsupported, match="a tuple of tensors"):
+        attempt([idx])
