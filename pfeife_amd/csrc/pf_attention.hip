@@ -113,6 +113,22 @@ __device__ __forceinline__ uint4 frag_tr(const uint16_t* s, int t0, int o32, int
   return make_uint4(lo.x, lo.y, hi.x, hi.y);
 }
 
+// Workgroup -> (row block, batch*head).  The hardware starts workgroups in the order of their
+// linear id (x fastest).  Under a causal mask the blocks of one head differ in work by up to the
+// number of blocks (a query block sweeps the keys up to its diagonal, a key block the queries from
+// its diagonal on): the heaviest blocks of EVERY head are started first, the lightest ones fill the
+// tail.  Without a mask all blocks are alike and neighbours keep sharing a head's operands in L2.
+__device__ __forceinline__ void attn_block(const AttnArgs& a, bool heavy_is_last, int& blk, int& bh) {
+  blk = (int)blockIdx.x;
+  bh = (int)blockIdx.y;
+  if (a.causal) {
+    const int id = (int)(blockIdx.y * gridDim.x + blockIdx.x), nbh = (int)gridDim.y;
+    const int k = id / nbh;
+    bh = id % nbh;
+    blk = heavy_is_last ? (int)gridDim.x - 1 - k : k;
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // forward: one workgroup = 128 queries of one (batch, head); wavefront w owns 32 of them
 // ---------------------------------------------------------------------------------
@@ -122,8 +138,10 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
   __shared__ __align__(16) uint16_t sK[KT * KLD];
   __shared__ __align__(16) uint16_t sV[KT * KLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int q0 = blockIdx.x * 128 + wave * 32;
+  int qb, bh;
+  attn_block(a, true, qb, bh);
+  const int b = bh / a.H, h = bh % a.H;
+  const int q0 = qb * 128 + wave * 32;
   const int qi = q0 + (lane & 31);          // this lane's query row
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
@@ -144,7 +162,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
 
   int k_end = a.Tk;
   if (a.causal) {
-    const int last_q = min(blockIdx.x * 128 + 127, a.Tq - 1);
+    const int last_q = min(qb * 128 + 127, a.Tq - 1);
     k_end = min(a.Tk, last_q + shift + 1);
   }
   Tile<HD> tk, tv;
@@ -273,8 +291,10 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
   __shared__ __align__(16) uint16_t sK[KT * KLD];
   __shared__ __align__(16) uint16_t sV[KT * KLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int q0 = blockIdx.x * 128 + wave * 32;
+  int qb, bh;
+  attn_block(a, true, qb, bh);
+  const int b = bh / a.H, h = bh % a.H;
+  const int q0 = qb * 128 + wave * 32;
   const int qi = q0 + (lane & 31);
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
@@ -302,7 +322,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(const AttnArgs a) {
 
   int k_end = a.Tk;
   if (a.causal) {
-    const int last_q = min(blockIdx.x * 128 + 127, a.Tq - 1);
+    const int last_q = min(qb * 128 + 127, a.Tq - 1);
     k_end = min(a.Tk, last_q + shift + 1);
   }
   Tile<HD> tk, tv;
@@ -376,8 +396,10 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
   __shared__ __align__(16) uint16_t sDO[KT * QLD];
   __shared__ float sLse[KT], sDelta[KT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int kw0 = blockIdx.x * 128 + wave * 32;                // this wavefront's first key row
+  int kb, bh;
+  attn_block(a, false, kb, bh);
+  const int b = bh / a.H, h = bh % a.H;
+  const int kw0 = kb * 128 + wave * 32;                        // this wavefront's first key row
   const int kj = kw0 + (lane & 31);                            // this lane's key row
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
@@ -401,7 +423,7 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(const AttnArgs a) {
 
   int q_begin = 0;
   if (a.causal) {  // queries i with i + shift >= first key of the block see it
-    q_begin = max(0, blockIdx.x * 128 - shift);
+    q_begin = max(0, kb * 128 - shift);
     q_begin = q_begin / KT * KT;
   }
   Tile<HD> tq, tdo;

@@ -421,7 +421,7 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
 }
 
 // Variant ids (pf_gemm_desc.variant; 0 = automatic):
-//   1..3   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128
+//   1..4   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128 / 192x256
 //   11..14 register-staged kernel: 128x128 by 8 wavefronts, 128x128, 128x64, 64x64 by 4
 enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_X192x256 = 4, V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
 
@@ -459,7 +459,8 @@ int choose_variant(const pf_gemm_desc& d) {
   const int64_t nb = d.batch1 * d.batch2;
   if (d.M < 128 || d.N < 128 || d.M * d.N < 128 * 128 * 16) return choose_staged(d);
   struct Cand { int v, xt, bm, bn; double t64, t64_busy; };
-  static const Cand cands[3] = {{V_X256, PF_XT_256x256, 256, 256, 1.45, 1.45},
+  static const Cand cands[4] = {{V_X256, PF_XT_256x256, 256, 256, 1.45, 1.45},
+                                {V_X192x256, PF_XT_192x256, 192, 256, 1.10, 1.10},
                                 {V_X256x128, PF_XT_256x128, 256, 128, 0.85, 0.90},
                                 {V_X128, PF_XT_128x128, 128, 128, 0.50, 0.62}};
   int best = -1;
