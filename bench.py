@@ -201,14 +201,25 @@ def hbm_kernel_rates(runner, reps=3):
             g["launches"].append(launch)
             g["bytes"] += nb
     out = []
+    w = runner.worker
     for name, g in sorted(groups.items()):
         ms = _time_launches(g["launches"], reps)
         n = len(g["launches"])
         gbs = g["bytes"] / (ms * 1e-3) / 1e9
+        # what a launch of this size can reach at all: a plain copy kernel that moves the same number
+        # of bytes (half read, half written), launched the same number of times back to back
+        per = max(1024, int(g["bytes"] / n) // 8)
+        src = torch.ones(per, device="cuda")
+        dst = torch.empty(per, device="cuda")
+        copy = w.kernels.axpby(src, 1.0, None, 0.0, dst, per)
+        copy_ms = _time_launches([copy] * min(n, 64), reps) / min(n, 64)
+        del src, dst
         out.append(dict(kernel=name, on_path=True, launches_per_step=n, ms_per_step=round(ms, 3),
                         avg_launch_us=round(1e3 * ms / n, 2), bytes_per_launch=round(g["bytes"] / n),
-                        achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4)))
-    w = runner.worker
+                        achieved=round(gbs, 1), peak=PEAK_HBM_GBS, unit="GB/s", frac=round(gbs / PEAK_HBM_GBS, 4),
+                        copy_same_bytes_us=round(1e3 * copy_ms, 2),
+                        frac_of_copy=round(copy_ms / (ms / n), 4)))
+
     opt = w.optimizer
     if opt is not None and w._fused_adam_applicable(opt):
         n_par = sum(p.numel() for g in opt.param_groups for p in g["params"] if p.grad is not None)
@@ -387,9 +398,11 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
             % (k, v["launches_per_step"], v["ms_per_step"], v["avg_launch_us"], v["tflops"]))
     rates = hbm_kernel_rates(runner) if hbm else None
     for r in rates or []:
-        log("[bench] %-26s %4d launches/step %8.3f ms/step %8.1f us/launch %7.1f GB/s (%.0f%% of %d)%s"
+        log("[bench] %-26s %4d launches/step %8.3f ms/step %8.1f us/launch %7.1f GB/s (%.0f%% of %d)%s%s"
             % (r["kernel"], r["launches_per_step"], r["ms_per_step"], r["avg_launch_us"], r["achieved"],
-               100 * r["frac"], PEAK_HBM_GBS, "" if r["on_path"] else "  [off-path micro-benchmark]"))
+               100 * r["frac"], PEAK_HBM_GBS, "" if r["on_path"] else "  [off-path micro-benchmark]",
+               "" if "frac_of_copy" not in r else "  copy of the same bytes: %.1f us (kernel at %.0f%% of it)"
+               % (r["copy_same_bytes_us"], 100 * r["frac_of_copy"])))
     flops_step = model_flops_per_step(info)
     cfg = info["cfg"]
     plan = getattr(w, "plan", None)

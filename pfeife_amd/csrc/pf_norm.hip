@@ -357,6 +357,43 @@ __global__ __launch_bounds__(256) void groupnorm_stats_kernel(const void* x, int
   }
 }
 
+// Vectorised statistics (channels per group a multiple of 8, the usual case): a pixel's share of
+// the group is Cg / 8 chunks of 8 consecutive channels; the workgroup's threads stride over the
+// (pixel, chunk) pairs with 16- or 32-byte loads, several in flight per thread.
+__global__ __launch_bounds__(256) void groupnorm_stats_vec_kernel(const void* x, int x_dt, float* mean, float* rstd,
+                                                                  int HW, int64_t C, int G, float eps) {
+  __shared__ float sm[4];
+  const int64_t b = blockIdx.x / G, g = blockIdx.x % G;
+  const int Cg = (int)(C / G), cpp = Cg / 8, nch = HW * cpp;
+  const int64_t base = b * HW * C + g * Cg;
+  float s = 0.f;
+#pragma unroll 4
+  for (int e = threadIdx.x; e < nch; e += 256) {
+    float v[8];
+    ld_vec<8>(x, base + (int64_t)(e / cpp) * C + (e % cpp) * 8, x_dt, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s += v[k];
+  }
+  const float n = (float)HW * (float)Cg;
+  const float mu = pf_block_sum<4>(s, sm) / n;
+  float q = 0.f;
+#pragma unroll 4
+  for (int e = threadIdx.x; e < nch; e += 256) {
+    float v[8];
+    ld_vec<8>(x, base + (int64_t)(e / cpp) * C + (e % cpp) * 8, x_dt, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const float t = v[k] - mu;
+      q += t * t;
+    }
+  }
+  const float var = pf_block_sum<4>(q, sm) / n;
+  if (threadIdx.x == 0) {
+    mean[blockIdx.x] = mu;
+    rstd[blockIdx.x] = 1.0f / sqrtf(var + eps);
+  }
+}
+
 // y = (x - mean[b,g]) * rstd[b,g] * gamma[c] + beta[c], 8 channels per thread (Cg % 8 == 0) or 1
 template <int W>
 __global__ __launch_bounds__(256) void groupnorm_apply_kernel(const void* x, int x_dt, const float* gamma,
@@ -419,6 +456,68 @@ __global__ __launch_bounds__(256) void groupnorm_bwd_stats_kernel(const void* dy
     const int64_t c = g * Cg + lane;
     ws[(b * 2) * C + c] = red[0][0][lane] + red[0][1][lane] + red[0][2][lane] + red[0][3][lane];
     ws[(b * 2 + 1) * C + c] = red[1][0][lane] + red[1][1][lane] + red[1][2][lane] + red[1][3][lane];
+  }
+}
+
+// Vectorised backward statistics (Cg % 8 == 0, Cg <= 64): thread t owns chunk t % cpp of the
+// pixels t / cpp, t / cpp + 256 / cpp, ... (the threads past cpp * (256 / cpp) idle), so its eight
+// channels are fixed and their partial sums stay in registers; the threads that share a chunk are
+// combined through LDS in a fixed order.
+__global__ __launch_bounds__(256) void groupnorm_bwd_stats_vec_kernel(const void* dy, int dy_dt, const void* x,
+                                                                      int x_dt, const float* gamma, const float* mean,
+                                                                      const float* rstd, float* c12, float* ws, int HW,
+                                                                      int64_t C, int G) {
+  __shared__ float sm[4];
+  __shared__ float red[256][17];
+  const int64_t b = blockIdx.x / G, g = blockIdx.x % G;
+  const int Cg = (int)(C / G), cpp = Cg / 8, ppt = 256 / cpp;   // pixels handled per sweep
+  const int t = threadIdx.x, j = t % cpp, p0 = t / cpp;
+  const float mu = mean[blockIdx.x], rs = rstd[blockIdx.x];
+  float s1 = 0.f, s2 = 0.f, pg[8], pb[8], gm[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) pg[k] = pb[k] = 0.f;
+  const int64_t c0 = g * Cg + j * 8;
+  ld_vec<8>(gamma, c0, PF_F32, gm);
+  if (p0 < ppt) {
+#pragma unroll 2
+    for (int p = p0; p < HW; p += ppt) {
+      const int64_t i = (b * HW + p) * C + c0;
+      float d[8], v[8];
+      ld_vec<8>(dy, i, dy_dt, d);
+      ld_vec<8>(x, i, x_dt, v);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float xh = (v[k] - mu) * rs;
+        const float dg = d[k] * gm[k];
+        s1 += dg;
+        s2 += dg * xh;
+        pg[k] += d[k] * xh;
+        pb[k] += d[k];
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    red[t][k] = pg[k];
+    red[t][8 + k] = pb[k];
+  }
+  const float n = (float)HW * (float)Cg;
+  s1 = pf_block_sum<4>(s1, sm);
+  s2 = pf_block_sum<4>(s2, sm);   // (the block sums synchronise, so `red` is complete below)
+  if (t == 0) {
+    c12[2 * blockIdx.x] = s1 / n;
+    c12[2 * blockIdx.x + 1] = s2 / n;
+  }
+  if (t < Cg) {   // thread t finishes channel t of the group: chunk t / 8, element t % 8
+    const int jj = t / 8, k = t % 8;
+    float a = 0.f, bsum = 0.f;
+    for (int q = 0; q < ppt; ++q) {
+      a += red[q * cpp + jj][k];
+      bsum += red[q * cpp + jj][8 + k];
+    }
+    const int64_t c = g * Cg + t;
+    ws[(b * 2) * C + c] = a;
+    ws[(b * 2 + 1) * C + c] = bsum;
   }
 }
 
@@ -638,11 +737,15 @@ extern "C" int pf_groupnorm_fwd(const void* x, int x_dtype, const float* gamma, 
   PF_REQUIRE(pf_is_float_dtype(x_dtype) && pf_is_float_dtype(y_dtype), "pf_groupnorm_fwd: bad dtype");
   PF_REQUIRE(B * groups < (1ll << 31), "pf_groupnorm_fwd: too many groups");
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(groupnorm_stats_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, x, x_dtype, mean, rstd, HW,
-                     C, groups, eps);
   const int64_t total = B * HW * C;
   const bool v = (C / groups) % 8 == 0 && vec_ok(x, x_dtype, C) && vec_ok(y, y_dtype, C) && vec_ok(gamma, PF_F32, C) &&
                  vec_ok(beta, PF_F32, C);
+  if ((C / groups) % 8 == 0 && vec_ok(x, x_dtype, C) && HW * (C / groups) < (1ll << 31))
+    hipLaunchKernelGGL(groupnorm_stats_vec_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, x, x_dtype, mean, rstd,
+                       (int)HW, C, groups, eps);
+  else
+    hipLaunchKernelGGL(groupnorm_stats_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, x, x_dtype, mean, rstd, HW,
+                       C, groups, eps);
   int64_t blocks = (total / (v ? 8 : 1) + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   if (blocks < 1) blocks = 1;
@@ -665,11 +768,16 @@ extern "C" int pf_groupnorm_bwd(const void* dy, int dy_dtype, const void* x, int
   hipStream_t st = (hipStream_t)stream;
   float* ws = workspace;                 // [B][2][C] channel partials
   float* c12 = workspace + B * 2 * C;    // [B*G][2]
-  hipLaunchKernelGGL(groupnorm_bwd_stats_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, dy, dy_dtype, x,
-                     x_dtype, gamma, mean, rstd, c12, ws, HW, C, groups);
   const int64_t total = B * HW * C;
   const bool v = (C / groups) % 8 == 0 && vec_ok(dy, dy_dtype, C) && vec_ok(x, x_dtype, C) && vec_ok(dx, dx_dtype, C) &&
                  vec_ok(gamma, PF_F32, C);
+  if ((C / groups) % 8 == 0 && vec_ok(dy, dy_dtype, C) && vec_ok(x, x_dtype, C) && vec_ok(gamma, PF_F32, C) &&
+      HW < (1ll << 31))
+    hipLaunchKernelGGL(groupnorm_bwd_stats_vec_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, dy, dy_dtype, x,
+                       x_dtype, gamma, mean, rstd, c12, ws, (int)HW, C, groups);
+  else
+    hipLaunchKernelGGL(groupnorm_bwd_stats_kernel, dim3((unsigned)(B * groups)), dim3(256), 0, st, dy, dy_dtype, x,
+                       x_dtype, gamma, mean, rstd, c12, ws, HW, C, groups);
   int64_t blocks = (total / (v ? 8 : 1) + 255) / 256;
   if (blocks > 4096) blocks = 4096;
   if (blocks < 1) blocks = 1;

@@ -540,7 +540,7 @@ def test_fused_attention(hip, oracle, dtype, case):
 
 @pytest.mark.parametrize("xdt,ydt", [(F32, F32), (F16, F16), (F32, BF16)])
 def test_groupnorm_and_channel_bias(hip, oracle, xdt, ydt):
-    for B, HW, C, G in [(4, 1024, 1280, 32), (2, 64, 64, 8), (3, 49, 96, 32)]:
+    for B, HW, C, G in [(4, 1024, 1280, 32), (2, 64, 64, 8), (3, 49, 96, 32), (2, 100, 128, 2), (1, 33, 64, 4)]:
         x = rnd((B, HW, C), xdt, 1) * 2 + 0.3
         gamma, beta = rnd((C,), F32, 2) + 1, rnd((C,), F32, 3)
         t = dict(x=x, gamma=gamma, beta=beta, y=torch.zeros(B, HW, C, dtype=ydt), mean=torch.zeros(B * G),
