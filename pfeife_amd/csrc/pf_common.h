@@ -212,6 +212,21 @@ __device__ __forceinline__ void st_vec(void* p, int64_t i, int dt, const float (
   }
 }
 
+// The same with the dtype known at compile time when DT >= 0 (W == 8): no branch around the
+// access, so several of them issue back to back and wait once.  (A runtime dtype switch puts
+// every access into a control-flow region of its own, and the compiler drains the memory
+// counter where regions join: one memory round trip per access.)
+template <int W, int DT>
+__device__ __forceinline__ void ld_vec_c(const void* p, int64_t i, int dt, float (&v)[W]) {
+  if constexpr (W == 8 && DT >= 0) Vec8<DT>::load(p, i, v);
+  else ld_vec<W>(p, i, dt, v);
+}
+template <int W, int DT>
+__device__ __forceinline__ void st_vec_c(void* p, int64_t i, int dt, const float (&v)[W]) {
+  if constexpr (W == 8 && DT >= 0) Vec8<DT>::store(p, i, v);
+  else st_vec<W>(p, i, dt, v);
+}
+
 // 64-lane wavefront reductions (butterfly; every lane ends with the result)
 __device__ __forceinline__ float pf_wave_sum(float v) {
 #pragma unroll

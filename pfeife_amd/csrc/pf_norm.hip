@@ -18,7 +18,8 @@ constexpr int COLRED_MAX_BLOCKS = 1024;
 // mean, then the sum of squared deviations, then the output come from the registers: one memory
 // round trip per row instead of three dependent ones (the kernel is latency-bound, a row is
 // 2-8 KB).  NV == 0: any d, three sweeps over the row (the second and third hit L2).
-template <int W, int NV>
+// XDT / YDT: dtypes of x and y when known at compile time (-1: read x_dt / y_dt at run time).
+template <int W, int NV, int XDT = -1, int YDT = -1>
 __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, const float* gamma, const float* beta,
                                                        void* y, int y_dt, float* mean, float* rstd, int64_t rows,
                                                        int64_t d, float eps, int rms) {
@@ -32,9 +33,9 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
     for (int i = 0; i < NV; ++i) {
       const int64_t c = ((int64_t)lane + i * 64) * W;
       if (c < d) {
-        ld_vec<W>(x, base + c, x_dt, v[i]);
-        ld_vec<W>(gamma, c, PF_F32, g[i]);
-        if (beta) ld_vec<W>(beta, c, PF_F32, b[i]);
+        ld_vec_c<W, XDT>(x, base + c, x_dt, v[i]);
+        ld_vec_c<W, PF_F32>(gamma, c, PF_F32, g[i]);
+        if (beta) ld_vec_c<W, PF_F32>(beta, c, PF_F32, b[i]);
       } else {
 #pragma unroll
         for (int k = 0; k < W; ++k) v[i][k] = 0.f;
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
 #pragma unroll
           for (int k = 0; k < W; ++k) o[k] = (v[i][k] - mu) * rs * g[i][k];
         }
-        st_vec<W>(y, base + c, y_dt, o);
+        st_vec_c<W, YDT>(y, base + c, y_dt, o);
       }
     }
     if (lane == 0) {
@@ -130,7 +131,9 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
 // ---- backward ----------------------------------------------------------------
 // NV = column groups a lane owns (d <= 64 * W * NV).  Column partials for
 // dgamma/dbeta stay in registers across the rows a wavefront processes.
-template <int W, int NV>
+// IODT: dtype of dy, x, dx_add and dx when they all share one known at compile time (-1: run time);
+// LPDT: dtype of dx_lp likewise.
+template <int W, int NV, int IODT = -1, int LPDT = -1>
 __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt, const void* x, int x_dt,
                                                        const float* gamma, const float* mean, const float* rstd,
                                                        const void* dx_add, int add_dt, void* dx, int dx_dt,
@@ -165,13 +168,13 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
       const int64_t c = ((int64_t)lane + i * 64) * W;
       if (c < d) {
         float vdy[W], vx[W], g[W];
-        ld_vec<W>(dy, base + c, dy_dt, vdy);
-        ld_vec<W>(x, base + c, x_dt, vx);
-        ld_vec<W>(gamma, c, PF_F32, g);
+        ld_vec_c<W, IODT>(dy, base + c, dy_dt, vdy);
+        ld_vec_c<W, IODT>(x, base + c, x_dt, vx);
+        ld_vec_c<W, PF_F32>(gamma, c, PF_F32, g);
         // the gradient already accumulated on x: requested with the other operands, so that the
         // row costs one memory round trip, not a second one after the reductions
         if constexpr (CACHE) {
-          if (dx_add) ld_vec<W>(dx_add, base + c, add_dt, cadd[i]);
+          if (dx_add) ld_vec_c<W, IODT>(dx_add, base + c, add_dt, cadd[i]);
         }
 #pragma unroll
         for (int k = 0; k < W; ++k) {
@@ -203,9 +206,9 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
           }
         } else {
           float vx[W], g[W];
-          ld_vec<W>(dy, base + c, dy_dt, vdy);
-          ld_vec<W>(x, base + c, x_dt, vx);
-          ld_vec<W>(gamma, c, PF_F32, g);
+          ld_vec_c<W, IODT>(dy, base + c, dy_dt, vdy);
+          ld_vec_c<W, IODT>(x, base + c, x_dt, vx);
+          ld_vec_c<W, PF_F32>(gamma, c, PF_F32, g);
 #pragma unroll
           for (int k = 0; k < W; ++k) {
             ggv[k] = vdy[k] * g[k];
@@ -224,18 +227,18 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
             for (int k = 0; k < W; ++k) o[k] += cadd[i][k];
           } else {
             float a[W];
-            ld_vec<W>(dx_add, base + c, add_dt, a);
+            ld_vec_c<W, IODT>(dx_add, base + c, add_dt, a);
 #pragma unroll
             for (int k = 0; k < W; ++k) o[k] += a[k];
           }
         }
-        st_vec<W>(dx, base + c, dx_dt, o);
+        st_vec_c<W, IODT>(dx, base + c, dx_dt, o);
         if (dx_lp) {
-          st_vec<W>(dx_lp, base + c, lp_dt, o);
+          st_vec_c<W, LPDT>(dx_lp, base + c, lp_dt, o);
           if constexpr (NS == NV) {
             if (want_colsum) {
 #pragma unroll
-              for (int k = 0; k < W; ++k) ps[i][k] += pf_round_to(lp_dt, o[k]);
+              for (int k = 0; k < W; ++k) ps[i][k] += pf_round_to(LPDT >= 0 ? LPDT : lp_dt, o[k]);
             }
           }
         }
@@ -579,11 +582,22 @@ int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, voi
   const bool v = vec_ok(x, x_dt, d) && vec_ok(y, y_dt, d) && vec_ok(gamma, PF_F32, d) && vec_ok(beta, PF_F32, d);
 #define PF_NF(W, NV) \
   hipLaunchKernelGGL((norm_fwd_kernel<W, NV>), grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms)
-  if (v && d <= 64 * 8 * 1) PF_NF(8, 1);
-  else if (v && d <= 64 * 8 * 2) PF_NF(8, 2);
-  else if (v && d <= 64 * 8 * 4) PF_NF(8, 4);
+#define PF_NFC(NV, XD, YD) \
+  hipLaunchKernelGGL((norm_fwd_kernel<8, NV, XD, YD>), grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms)
+  // the residual stream is fp32 and the consumers are matrix products (16-bit) or fp32: those
+  // pairs get straight-line code
+#define PF_NFD(NV)                                                     \
+  if (x_dt == PF_F32 && y_dt == PF_F16) PF_NFC(NV, PF_F32, PF_F16);     \
+  else if (x_dt == PF_F32 && y_dt == PF_BF16) PF_NFC(NV, PF_F32, PF_BF16); \
+  else if (x_dt == PF_F32 && y_dt == PF_F32) PF_NFC(NV, PF_F32, PF_F32); \
+  else PF_NF(8, NV)
+  if (v && d <= 64 * 8 * 1) { PF_NFD(1); }
+  else if (v && d <= 64 * 8 * 2) { PF_NFD(2); }
+  else if (v && d <= 64 * 8 * 4) { PF_NFD(4); }
   else if (v) PF_NF(8, 0);
   else PF_NF(1, 0);
+#undef PF_NFD
+#undef PF_NFC
 #undef PF_NF
   PF_CHECK_LAUNCH(name);
   return PF_OK;
@@ -610,9 +624,18 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
 #define PF_NB(W, NV)                                                                                          \
   hipLaunchKernelGGL((norm_bwd_kernel<W, NV>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, mean, \
                      rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want, dx_lp, lp_dt, want_colsum)
+  // the residual stream and its gradient are fp32, the side copy 16-bit: straight-line variants
+  const bool io32 = dy_dt == PF_F32 && x_dt == PF_F32 && dx_dt == PF_F32 && (!dx_add || add_dt == PF_F32);
+#define PF_NBC(NV, LP)                                                                                           \
+  hipLaunchKernelGGL((norm_bwd_kernel<8, NV, PF_F32, LP>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, \
+                     mean, rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want, dx_lp, lp_dt, want_colsum)
+#define PF_NBD(NV)                                                   \
+  if (io32 && (!dx_lp || lp_dt == PF_F16)) PF_NBC(NV, PF_F16);        \
+  else if (io32 && lp_dt == PF_BF16) PF_NBC(NV, PF_BF16);             \
+  else PF_NB(8, NV)
   if (v) {
-    if (d <= 64 * 8 * 2) PF_NB(8, 2);
-    else if (d <= 64 * 8 * 4) PF_NB(8, 4);
+    if (d <= 64 * 8 * 2) { PF_NBD(2); }
+    else if (d <= 64 * 8 * 4) { PF_NBD(4); }
     else if (d <= 64 * 8 * 8) PF_NB(8, 8);
     else if (d <= 64 * 8 * 16) PF_NB(8, 16);
     else { pf_set_error("%s: d=%lld exceeds 8192", name, (long long)d); return PF_ERR_UNSUPPORTED; }
@@ -621,6 +644,8 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
     else if (d <= 64 * 64) PF_NB(1, 64);
     else { pf_set_error("%s: unaligned d=%lld exceeds 4096", name, (long long)d); return PF_ERR_UNSUPPORTED; }
   }
+#undef PF_NBD
+#undef PF_NBC
 #undef PF_NB
   PF_CHECK_LAUNCH(name);
   if (want && !defer) {
