@@ -131,9 +131,9 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
 // ---- backward ----------------------------------------------------------------
 // NV = column groups a lane owns (d <= 64 * W * NV).  Column partials for
 // dgamma/dbeta stay in registers across the rows a wavefront processes.
-// IODT: dtype of dy, x, dx_add and dx when they all share one known at compile time (-1: run time);
-// LPDT: dtype of dx_lp likewise.
-template <int W, int NV, int IODT = -1, int LPDT = -1>
+// IODT: dtype of x, dx_add and dx when they all share one known at compile time (-1: run time);
+// LPDT: dtype of dx_lp likewise; DYDT: dtype of dy likewise.
+template <int W, int NV, int IODT = -1, int LPDT = -1, int DYDT = -1>
 __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt, const void* x, int x_dt,
                                                        const float* gamma, const float* mean, const float* rstd,
                                                        const void* dx_add, int add_dt, void* dx, int dx_dt,
@@ -157,6 +157,87 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
     for (int k = 0; k < W; ++k) ps[i][k] = 0.f;
 
   constexpr bool CACHE = (NV * W <= 32);   // keep the row's dy and x in registers between the two passes
+  // Straight-line variants with at most two column groups per lane: the operands of the wavefront's
+  // NEXT row are requested before the current row is reduced and stored, so a wavefront that
+  // owns two rows pays one memory round trip, not two.  Nothing around the loads branches (row and
+  // column indices are clamped, out-of-range lanes contribute zeros and store nothing).
+  constexpr bool PIPE = CACHE && NV <= 2 && IODT >= 0 && DYDT >= 0 && W == 8;
+  if constexpr (PIPE) {
+    const int64_t stride = (int64_t)gridDim.x * 4;
+    int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    const bool has_add = dx_add != nullptr;
+    bool ok[NV];
+    int64_t col[NV];
+    float g[NV][W];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int64_t c = ((int64_t)lane + i * 64) * W;
+      ok[i] = c < d;
+      col[i] = ok[i] ? c : 0;
+      ld_vec_c<W, PF_F32>(gamma, col[i], PF_F32, g[i]);
+    }
+    float ndy[NV][W], nx[NV][W], nadd[NV][W], nmu, nrs;
+    auto fetch = [&](int64_t r) {
+      const int64_t rr = r < rows ? r : rows - 1;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        ld_vec_c<W, DYDT>(dy, rr * d + col[i], dy_dt, ndy[i]);
+        ld_vec_c<W, IODT>(x, rr * d + col[i], x_dt, nx[i]);
+        if (has_add) ld_vec_c<W, IODT>(dx_add, rr * d + col[i], add_dt, nadd[i]);
+      }
+      nmu = rms ? 0.f : mean[rr];
+      nrs = rstd[rr];
+    };
+    if (row < rows) fetch(row);
+    while (row < rows) {
+      float cdy[NV][W], cx[NV][W], cadd[NV][W];
+      const float mu = nmu, rs = nrs;
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          cdy[i][k] = ok[i] ? ndy[i][k] : 0.f;
+          cx[i][k] = nx[i][k];
+          cadd[i][k] = has_add ? nadd[i][k] : 0.f;
+        }
+      fetch(row + stride);
+      float c1 = 0.f, c2 = 0.f;
+      float xh[NV][W], gg[NV][W];
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          gg[i][k] = cdy[i][k] * g[i][k];
+          xh[i][k] = ok[i] ? (cx[i][k] - mu) * rs : 0.f;
+          c1 += gg[i][k];
+          c2 += gg[i][k] * xh[i][k];
+        }
+      c1 = rms ? 0.f : pf_wave_sum(c1) / (float)d;
+      c2 = pf_wave_sum(c2) / (float)d;
+      const int64_t base = row * d;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        float o[W];
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+          o[k] = rs * (gg[i][k] - c1 - xh[i][k] * c2) + cadd[i][k];
+          pg[i][k] += cdy[i][k] * xh[i][k];
+          pb[i][k] += cdy[i][k];
+        }
+        if (ok[i]) {
+          st_vec_c<W, IODT>(dx, base + col[i], dx_dt, o);
+          if (dx_lp) {
+            st_vec_c<W, LPDT>(dx_lp, base + col[i], lp_dt, o);
+            if (want_colsum) {
+#pragma unroll
+              for (int k = 0; k < W; ++k) ps[i][k] += pf_round_to(LPDT >= 0 ? LPDT : lp_dt, o[k]);
+            }
+          }
+        }
+      }
+      row += stride;
+    }
+  } else
   for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < rows; row += (int64_t)gridDim.x * 4) {
     const int64_t base = row * d;
     const float mu = rms ? 0.f : mean[row];
@@ -168,7 +249,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
       const int64_t c = ((int64_t)lane + i * 64) * W;
       if (c < d) {
         float vdy[W], vx[W], g[W];
-        ld_vec_c<W, IODT>(dy, base + c, dy_dt, vdy);
+        ld_vec_c<W, DYDT>(dy, base + c, dy_dt, vdy);
         ld_vec_c<W, IODT>(x, base + c, x_dt, vx);
         ld_vec_c<W, PF_F32>(gamma, c, PF_F32, g);
         // the gradient already accumulated on x: requested with the other operands, so that the
@@ -206,7 +287,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
           }
         } else {
           float vx[W], g[W];
-          ld_vec_c<W, IODT>(dy, base + c, dy_dt, vdy);
+          ld_vec_c<W, DYDT>(dy, base + c, dy_dt, vdy);
           ld_vec_c<W, IODT>(x, base + c, x_dt, vx);
           ld_vec_c<W, PF_F32>(gamma, c, PF_F32, g);
 #pragma unroll
@@ -625,13 +706,16 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
   hipLaunchKernelGGL((norm_bwd_kernel<W, NV>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, mean, \
                      rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want, dx_lp, lp_dt, want_colsum)
   // the residual stream and its gradient are fp32, the side copy 16-bit: straight-line variants
-  const bool io32 = dy_dt == PF_F32 && x_dt == PF_F32 && dx_dt == PF_F32 && (!dx_add || add_dt == PF_F32);
-#define PF_NBC(NV, LP)                                                                                           \
-  hipLaunchKernelGGL((norm_bwd_kernel<8, NV, PF_F32, LP>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, \
+  // (the incoming gradient is the 16-bit result of a matrix product, or fp32)
+  const bool io32 = x_dt == PF_F32 && dx_dt == PF_F32 && (!dx_add || add_dt == PF_F32);
+#define PF_NBC(NV, LP, DY)                                                                                           \
+  hipLaunchKernelGGL((norm_bwd_kernel<8, NV, PF_F32, LP, DY>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, \
                      mean, rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want, dx_lp, lp_dt, want_colsum)
-#define PF_NBD(NV)                                                   \
-  if (io32 && (!dx_lp || lp_dt == PF_F16)) PF_NBC(NV, PF_F16);        \
-  else if (io32 && lp_dt == PF_BF16) PF_NBC(NV, PF_BF16);             \
+#define PF_NBD(NV)                                                                          \
+  if (io32 && dy_dt == PF_F16 && (!dx_lp || lp_dt == PF_F16)) PF_NBC(NV, PF_F16, PF_F16);    \
+  else if (io32 && dy_dt == PF_BF16 && (!dx_lp || lp_dt == PF_BF16)) PF_NBC(NV, PF_BF16, PF_BF16); \
+  else if (io32 && dy_dt == PF_F32 && (!dx_lp || lp_dt == PF_F16)) PF_NBC(NV, PF_F16, PF_F32);    \
+  else if (io32 && dy_dt == PF_F32 && lp_dt == PF_BF16) PF_NBC(NV, PF_BF16, PF_F32);         \
   else PF_NB(8, NV)
   if (v) {
     if (d <= 64 * 8 * 2) { PF_NBD(2); }
