@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
   // NEXT row are requested before the current row is reduced and stored, so a wavefront that
   // owns two rows pays one memory round trip, not two.  Nothing around the loads branches (row and
   // column indices are clamped, out-of-range lanes contribute zeros and store nothing).
-  constexpr bool PIPE = CACHE && NV <= 2 && IODT >= 0 && DYDT >= 0 && W == 8;
+  constexpr bool PIPE = CACHE && NV <= 4 && IODT >= 0 && DYDT >= 0 && W == 8;
   if constexpr (PIPE) {
     const int64_t stride = (int64_t)gridDim.x * 4;
     int64_t row = (int64_t)blockIdx.x * 4 + wave;
