@@ -122,34 +122,40 @@ struct BiasAdd {  // bias_len is a multiple of 8 on the vector path
 };
 
 // gated MLP: rows x cols with independent row strides; index space is rows*cols
+// DT: the operands' dtype when fixed at compile time (-1: read `dt` at run time).  With a fixed
+// dtype the two or three loads of an element group issue back to back and wait once.
+template <int DT = -1>
 struct GluFwd {
   const void* gate; const void* up; void* y; int64_t ldg, ldu, ldy, cols; int dt, act;
   template <int W> __device__ void run(int64_t i) const {
     const int64_t r = i / cols, c = i % cols;
+    const int edt = DT >= 0 ? DT : dt;
     float g[W], u[W];
-    ld_vec<W>(gate, r * ldg + c, dt, g);
-    ld_vec<W>(up, r * ldu + c, dt, u);
+    ld_vec_c<W, DT>(gate, r * ldg + c, dt, g);
+    ld_vec_c<W, DT>(up, r * ldu + c, dt, u);
 #pragma unroll
-    for (int k = 0; k < W; ++k) g[k] = pf_round_to(dt, pf_act(act, g[k])) * u[k];
-    st_vec<W>(y, r * ldy + c, dt, g);
+    for (int k = 0; k < W; ++k) g[k] = pf_round_to(edt, pf_act(act, g[k])) * u[k];
+    st_vec_c<W, DT>(y, r * ldy + c, dt, g);
   }
 };
+template <int DT = -1>
 struct GluBwd {
   const void* dy; const void* gate; const void* up; void* dgate; void* dup;
   int64_t lddy, ldg, ldu, lddg, lddu, cols; int dt, act;
   template <int W> __device__ void run(int64_t i) const {
     const int64_t r = i / cols, c = i % cols;
+    const int edt = DT >= 0 ? DT : dt;
     float d[W], g[W], u[W], dg[W], du[W];
-    ld_vec<W>(dy, r * lddy + c, dt, d);
-    ld_vec<W>(gate, r * ldg + c, dt, g);
-    ld_vec<W>(up, r * ldu + c, dt, u);
+    ld_vec_c<W, DT>(dy, r * lddy + c, dt, d);
+    ld_vec_c<W, DT>(gate, r * ldg + c, dt, g);
+    ld_vec_c<W, DT>(up, r * ldu + c, dt, u);
 #pragma unroll
     for (int k = 0; k < W; ++k) {
-      du[k] = d[k] * pf_round_to(dt, pf_act(act, g[k]));
+      du[k] = d[k] * pf_round_to(edt, pf_act(act, g[k]));
       dg[k] = d[k] * u[k] * pf_act_grad(act, g[k]);
     }
-    st_vec<W>(dgate, r * lddg + c, dt, dg);
-    st_vec<W>(dup, r * lddu + c, dt, du);
+    st_vec_c<W, DT>(dgate, r * lddg + c, dt, dg);
+    st_vec_c<W, DT>(dup, r * lddu + c, dt, du);
   }
 };
 
@@ -424,7 +430,13 @@ extern "C" int pf_glu_fwd(const void* gate, int64_t ld_gate, const void* up, int
   PF_REQUIRE(ld_gate >= cols && ld_up >= cols && ld_y >= cols, "pf_glu_fwd: leading dimension too small");
   const bool vec = al16(gate) && al16(up) && al16(y) && cols % 8 == 0 && ld_gate % 8 == 0 && ld_up % 8 == 0 &&
                    ld_y % 8 == 0;
-  GluFwd f{gate, up, y, ld_gate, ld_up, ld_y, cols, dtype, act};
+  if (vec && dtype == PF_BF16)
+    return ew_launch(GluFwd<PF_BF16>{gate, up, y, ld_gate, ld_up, ld_y, cols, dtype, act}, rows * cols, vec,
+                     (hipStream_t)stream, "pf_glu_fwd");
+  if (vec && dtype == PF_F16)
+    return ew_launch(GluFwd<PF_F16>{gate, up, y, ld_gate, ld_up, ld_y, cols, dtype, act}, rows * cols, vec,
+                     (hipStream_t)stream, "pf_glu_fwd");
+  GluFwd<> f{gate, up, y, ld_gate, ld_up, ld_y, cols, dtype, act};
   return ew_launch(f, rows * cols, vec, (hipStream_t)stream, "pf_glu_fwd");
 }
 
@@ -438,7 +450,13 @@ extern "C" int pf_glu_bwd(const void* dy, int64_t ld_dy, const void* gate, int64
              "pf_glu_bwd: leading dimension too small");
   const bool vec = al16(dy) && al16(gate) && al16(up) && al16(dgate) && al16(dup) && cols % 8 == 0 &&
                    ld_dy % 8 == 0 && ld_gate % 8 == 0 && ld_up % 8 == 0 && ld_dgate % 8 == 0 && ld_dup % 8 == 0;
-  GluBwd f{dy, gate, up, dgate, dup, ld_dy, ld_gate, ld_up, ld_dgate, ld_dup, cols, dtype, act};
+  if (vec && dtype == PF_BF16)
+    return ew_launch(GluBwd<PF_BF16>{dy, gate, up, dgate, dup, ld_dy, ld_gate, ld_up, ld_dgate, ld_dup, cols, dtype, act},
+                     rows * cols, vec, (hipStream_t)stream, "pf_glu_bwd");
+  if (vec && dtype == PF_F16)
+    return ew_launch(GluBwd<PF_F16>{dy, gate, up, dgate, dup, ld_dy, ld_gate, ld_up, ld_dgate, ld_dup, cols, dtype, act},
+                     rows * cols, vec, (hipStream_t)stream, "pf_glu_bwd");
+  GluBwd<> f{dy, gate, up, dgate, dup, ld_dy, ld_gate, ld_up, ld_dgate, ld_dup, cols, dtype, act};
   return ew_launch(f, rows * cols, vec, (hipStream_t)stream, "pf_glu_bwd");
 }
 

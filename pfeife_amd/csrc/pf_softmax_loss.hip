@@ -119,6 +119,72 @@ __global__ __launch_bounds__(256) void ce_bwd_kernel(const void* logits, int l_d
   }
 }
 
+// Vectorised variants (classes % 8 == 0, 16-byte aligned rows, dtype fixed at compile time):
+// eight classes per lane and access, several accesses in flight; same two passes over the row
+// (maximum, then sum of exponentials; the second pass is served by the caches).
+template <int DT>
+__global__ __launch_bounds__(256) void ce_fwd_vec_kernel(const void* logits, const int64_t* targets, float* row_loss,
+                                                         float* row_lse, int64_t classes, int64_t ignore_index) {
+  __shared__ float sm[4];
+  const int64_t row = blockIdx.x;
+  const int64_t base = row * classes;
+  float m = -INFINITY;
+#pragma unroll 4
+  for (int64_t c = (int64_t)threadIdx.x * 8; c < classes; c += 2048) {
+    float v[8];
+    Vec8<DT>::load(logits, base + c, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) m = fmaxf(m, v[k]);
+  }
+  m = pf_block_max<4>(m, sm);
+  float z = 0.f;
+#pragma unroll 4
+  for (int64_t c = (int64_t)threadIdx.x * 8; c < classes; c += 2048) {
+    float v[8];
+    Vec8<DT>::load(logits, base + c, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) z += expf(v[k] - m);
+  }
+  z = pf_block_sum<4>(z, sm);
+  if (threadIdx.x == 0) {
+    const float lse = m + logf(z);
+    const int64_t t = targets[row];
+    row_lse[row] = lse;
+    float l = 0.f;
+    if (t != ignore_index) l = (t >= 0 && t < classes) ? lse - pf_load_as_f32(logits, base + t, DT) : NAN;
+    row_loss[row] = l;
+  }
+}
+
+template <int DT, int ODT>
+__global__ __launch_bounds__(256) void ce_bwd_vec_kernel(const void* logits, const int64_t* targets,
+                                                         const float* row_lse, const float* dloss,
+                                                         const float* n_valid, void* dlogits, int64_t classes,
+                                                         int64_t ignore_index) {
+  const int64_t row = blockIdx.x;
+  const int64_t base = row * classes;
+  const int64_t t = targets[row];
+  const float g = (dloss ? dloss[0] : 1.f) / n_valid[0];
+  const float lse = row_lse[row];
+  const bool ignored = (t == ignore_index);
+#pragma unroll 4
+  for (int64_t c = (int64_t)threadIdx.x * 8; c < classes; c += 2048) {
+    float v[8];
+    Vec8<DT>::load(logits, base + c, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      float o = 0.f;
+      if (!ignored) {
+        o = expf(v[k] - lse);
+        if (c + k == t) o -= 1.f;
+        o *= g;
+      }
+      v[k] = o;
+    }
+    Vec8<ODT>::store(dlogits, base + c, v);
+  }
+}
+
 // ---- scalar reductions (MSE, sum) ---------------------------------------------
 constexpr int RED_MAX_BLOCKS = 1024;
 
@@ -200,8 +266,16 @@ extern "C" int pf_cross_entropy_fwd(const void* logits, int l_dtype, const int64
   hipStream_t st = (hipStream_t)stream;
   if (rows > 0) {
     PF_REQUIRE(logits && targets && row_loss && row_lse, "pf_cross_entropy_fwd: null pointer");
-    hipLaunchKernelGGL(ce_fwd_kernel, dim3((unsigned)rows), dim3(256), 0, st, logits, l_dtype, targets, row_loss,
-                       row_lse, classes, ignore_index);
+    const bool vec = classes % 8 == 0 && pf_aligned(logits, 16);
+#define PF_CEF(DT) \
+  hipLaunchKernelGGL(ce_fwd_vec_kernel<DT>, dim3((unsigned)rows), dim3(256), 0, st, logits, targets, row_loss, row_lse, classes, ignore_index)
+    if (vec && l_dtype == PF_F32) PF_CEF(PF_F32);
+    else if (vec && l_dtype == PF_F16) PF_CEF(PF_F16);
+    else if (vec && l_dtype == PF_BF16) PF_CEF(PF_BF16);
+    else
+      hipLaunchKernelGGL(ce_fwd_kernel, dim3((unsigned)rows), dim3(256), 0, st, logits, l_dtype, targets, row_loss,
+                         row_lse, classes, ignore_index);
+#undef PF_CEF
   }
   hipLaunchKernelGGL(ce_mean_kernel, dim3(1), dim3(256), 0, st, row_loss, targets, loss, rows, ignore_index);
   PF_CHECK_LAUNCH("pf_cross_entropy_fwd");
@@ -216,8 +290,19 @@ extern "C" int pf_cross_entropy_bwd(const void* logits, int l_dtype, const int64
   if (rows == 0) return PF_OK;
   PF_REQUIRE(logits && targets && row_lse && n_valid && dlogits, "pf_cross_entropy_bwd: null pointer");
   PF_REQUIRE(rows < (1ll << 31), "pf_cross_entropy_bwd: too many rows");
-  hipLaunchKernelGGL(ce_bwd_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, logits, l_dtype, targets,
-                     row_lse, dloss, n_valid, dlogits, dl_dtype, classes, ignore_index);
+  const bool vec = classes % 8 == 0 && pf_aligned(logits, 16) && pf_aligned(dlogits, 16);
+#define PF_CEB(DT, ODT)                                                                                         \
+  hipLaunchKernelGGL((ce_bwd_vec_kernel<DT, ODT>), dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, logits, \
+                     targets, row_lse, dloss, n_valid, dlogits, classes, ignore_index)
+  if (vec && l_dtype == PF_F32 && dl_dtype == PF_F32) PF_CEB(PF_F32, PF_F32);
+  else if (vec && l_dtype == PF_F16 && dl_dtype == PF_F16) PF_CEB(PF_F16, PF_F16);
+  else if (vec && l_dtype == PF_BF16 && dl_dtype == PF_BF16) PF_CEB(PF_BF16, PF_BF16);
+  else if (vec && l_dtype == PF_F32 && dl_dtype == PF_F16) PF_CEB(PF_F32, PF_F16);
+  else if (vec && l_dtype == PF_F32 && dl_dtype == PF_BF16) PF_CEB(PF_F32, PF_BF16);
+  else
+    hipLaunchKernelGGL(ce_bwd_kernel, dim3((unsigned)rows), dim3(256), 0, (hipStream_t)stream, logits, l_dtype, targets,
+                       row_lse, dloss, n_valid, dlogits, dl_dtype, classes, ignore_index);
+#undef PF_CEB
   PF_CHECK_LAUNCH("pf_cross_entropy_bwd");
   return PF_OK;
 }
