@@ -376,7 +376,8 @@ __global__ __launch_bounds__(256) void colreduce_finalize_kernel(const float* ws
 
 // column sums of x[rows, cols]: block = 4 wavefronts sharing one 64*W column
 // strip, wavefront w takes rows w, w+4, ... of its row chunk.
-template <int W>
+// XDT: dtype of x when fixed at compile time (-1: run time).
+template <int W, int XDT = -1>
 __global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, int64_t rows, int64_t cols, int64_t ld,
                                                      float* ws, int64_t rows_per_chunk) {
   __shared__ float red[4][64 * W];
@@ -388,21 +389,22 @@ __global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, in
 #pragma unroll
   for (int k = 0; k < W; ++k) s[k] = 0.f;
   if (c < cols) {
-    // 8 rows requested together (the loop is short and latency-bound), summed in row order
+    // 8 rows requested together (the loop is short and latency-bound), summed in row order; rows
+    // past the chunk are read from a valid row instead and not added, so that nothing around
+    // the loads branches
     for (int64_t r = r0 + wave; r < r1; r += 32) {
       float v[8][W];
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        if (r + 4 * u < r1) ld_vec<W>(x, (r + 4 * u) * ld + c, x_dt, v[u]);
-        else {
-#pragma unroll
-          for (int k = 0; k < W; ++k) v[u][k] = 0.f;
-        }
+        const int64_t rr = r + 4 * u < r1 ? r + 4 * u : r;
+        ld_vec_c<W, XDT>(x, rr * ld + c, x_dt, v[u]);
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < 8; ++u) {
+        const bool in = r + 4 * u < r1;
 #pragma unroll
-        for (int k = 0; k < W; ++k) s[k] += v[u][k];
+        for (int k = 0; k < W; ++k) s[k] += in ? v[u][k] : 0.f;
+      }
     }
   }
 #pragma unroll
@@ -917,7 +919,11 @@ extern "C" int pf_colsum_accumulate(const void* x, int x_dtype, int64_t rows, in
   const bool v = vec_ok(x, x_dtype, ld) && cols % 8 == 0;
   if (v) {
     const dim3 grid((unsigned)((cols + 511) / 512), (unsigned)chunks);
-    hipLaunchKernelGGL(colsum_kernel<8>, grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc);
+#define PF_CS(DT) hipLaunchKernelGGL((colsum_kernel<8, DT>), grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc)
+    if (x_dtype == PF_F16) PF_CS(PF_F16);
+    else if (x_dtype == PF_BF16) PF_CS(PF_BF16);
+    else PF_CS(PF_F32);
+#undef PF_CS
   } else {
     const dim3 grid((unsigned)((cols + 63) / 64), (unsigned)chunks);
     hipLaunchKernelGGL(colsum_kernel<1>, grid, dim3(256), 0, st, x, x_dtype, rows, cols, ld, workspace, rpc);
