@@ -28,18 +28,21 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
   if (row >= rows) return;
   const int64_t base = row * d;
   if constexpr (NV > 0) {
+    // nothing around the loads branches: out-of-range lanes read column 0 and are masked out of
+    // the sums and the stores; a missing beta reads gamma instead and is not added
     float v[NV][W], g[NV][W], b[NV][W];
+    bool ok[NV];
+    int64_t col[NV];
+    const bool has_beta = beta != nullptr;
+    const float* bsrc = has_beta ? beta : gamma;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int64_t c = ((int64_t)lane + i * 64) * W;
-      if (c < d) {
-        ld_vec_c<W, XDT>(x, base + c, x_dt, v[i]);
-        ld_vec_c<W, PF_F32>(gamma, c, PF_F32, g[i]);
-        if (beta) ld_vec_c<W, PF_F32>(beta, c, PF_F32, b[i]);
-      } else {
-#pragma unroll
-        for (int k = 0; k < W; ++k) v[i][k] = 0.f;
-      }
+      ok[i] = c < d;
+      col[i] = ok[i] ? c : 0;
+      ld_vec_c<W, XDT>(x, base + col[i], x_dt, v[i]);
+      ld_vec_c<W, PF_F32>(gamma, col[i], PF_F32, g[i]);
+      ld_vec_c<W, PF_F32>(bsrc, col[i], PF_F32, b[i]);
     }
     float mu = 0.f;
     if (!rms) {
@@ -47,36 +50,29 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const void* x, int x_dt, 
 #pragma unroll
       for (int i = 0; i < NV; ++i)
 #pragma unroll
-        for (int k = 0; k < W; ++k) s += v[i][k];
+        for (int k = 0; k < W; ++k) s += ok[i] ? v[i][k] : 0.f;
       mu = pf_wave_sum(s) / (float)d;
     }
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if (((int64_t)lane + i * 64) * W < d) {
 #pragma unroll
-        for (int k = 0; k < W; ++k) {
-          const float t = v[i][k] - mu;
-          q += t * t;
-        }
+      for (int k = 0; k < W; ++k) {
+        const float t = v[i][k] - mu;
+        q += ok[i] ? t * t : 0.f;
       }
     }
     const float var = pf_wave_sum(q) / (float)d;
     const float rs = 1.0f / sqrtf(var + eps);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int64_t c = ((int64_t)lane + i * 64) * W;
-      if (c < d) {
-        float o[W];
-        if (beta) {
+      float o[W];
 #pragma unroll
-          for (int k = 0; k < W; ++k) o[k] = (v[i][k] - mu) * rs * g[i][k] + b[i][k];
-        } else {
-#pragma unroll
-          for (int k = 0; k < W; ++k) o[k] = (v[i][k] - mu) * rs * g[i][k];
-        }
-        st_vec_c<W, YDT>(y, base + c, y_dt, o);
+      for (int k = 0; k < W; ++k) {
+        const float t = (v[i][k] - mu) * rs * g[i][k];
+        o[k] = has_beta ? t + b[i][k] : t;
       }
+      if (ok[i]) st_vec_c<W, YDT>(y, base + col[i], y_dt, o);
     }
     if (lane == 0) {
       if (mean) mean[row] = mu;
