@@ -306,6 +306,81 @@ def test_llama_style_four_stages_looped(mixed):
     _check_grads(model, ref, mixed)
 
 
+def test_lanes_give_bit_identical_steps(monkeypatch):
+    """Jobs of different pipeline ranks run on streams of their own (PFEIFE_LANES: per rank and
+    direction, per rank, or a single stream).  The lanes only change WHEN independent jobs run:
+    losses and every accumulated gradient must be bit-identical in the three modes, for a
+    two-stage ViT and for four looped decoder stages over two ranks, across several steps."""
+    from pfeife_amd.bench_models.llama import LlamaConfig, LlamaForCausalLM
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    def run_vit(mode):
+        monkeypatch.setenv("PFEIFE_LANES", mode)
+        cfg = ViTConfig(image_size=64, patch_size=16, dim=128, depth=4, heads=4, mlp_dim=256, num_classes=16)
+        torch.manual_seed(0)
+        model = VisionTransformer(cfg)
+        g = torch.Generator().manual_seed(42)
+        x = torch.randn(12, 3, 64, 64, generator=g).cuda()
+        y = torch.randint(0, 16, (12,), generator=g).cuda()
+        option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=3, split_points=["blocks.2"],
+                            mixed_precision="bf16", optimizer=dict(type="adam", lr=1e-3))
+        runner = _fresh_runner(option)
+        model.cuda()
+        cmodel = torch.compile(model, backend=partial_compiler)
+        crit = nn.CrossEntropyLoss()
+
+        def fn(px, labels):
+            loss = crit(cmodel(px).float(), labels)
+            loss.backward()
+            return loss.detach()
+
+        runner.set_exec_fn(fn)
+        out = []
+        for _ in range(3):
+            losses = runner.step(x, y)
+            torch.cuda.synchronize()
+            out.append(([float(l) for l in losses], [p.grad.clone() for p in model.parameters()]))
+        return out, runner
+
+    def run_llama(mode):
+        monkeypatch.setenv("PFEIFE_LANES", mode)
+        cfg = LlamaConfig(vocab=512, dim=256, layers=4, heads=4, ffn=688, max_seq=128)
+        torch.manual_seed(0)
+        model = LlamaForCausalLM(cfg)
+        ids = torch.randint(0, cfg.vocab, (16, 128), generator=torch.Generator().manual_seed(42)).cuda()
+        option = PipeOption(device_cnt=2, batch_cnt=8, batch_size=2, split_points=["layers.1", "layers.2", "layers.3"],
+                            mixed_precision="bf16", optimizer=dict(type="adam", lr=1e-3))
+        runner = _fresh_runner(option)
+        model.cuda()
+        cmodel = torch.compile(model, backend=partial_compiler)
+
+        def fn(tok):
+            loss = cmodel(tok, tok)
+            loss.backward()
+            return loss.detach()
+
+        runner.set_exec_fn(fn)
+        out = []
+        for _ in range(3):
+            losses = runner.step(ids)
+            torch.cuda.synchronize()
+            out.append(([float(l) for l in losses], [p.grad.clone() for p in model.parameters()]))
+        return out, runner
+
+    for run, streams in ((run_vit, {"0": 0, "rank": 2, "rankdir": 4}), (run_llama, {"0": 0, "rank": 2, "rankdir": 4})):
+        base, runner = run("0")
+        assert runner.worker.lanes is None
+        for mode in ("rank", "rankdir"):
+            got, runner = run(mode)
+            assert runner.worker.lanes is not None and len(runner.worker.lanes) == streams[mode]
+            for (l0, g0), (l1, g1) in zip(base, got):
+                assert l0 == l1, (mode, l0, l1)
+                for a, b in zip(g0, g1):
+                    assert torch.equal(a, b), mode
+
+
 @pytest.mark.parametrize("mixed", [None, "bf16"])
 def test_vit_g_block_share_head_dim_88(mixed):
     """The ViT-g/14 block-share configuration at reduced depth: blocks (dim 1408, 16 heads of 88,
