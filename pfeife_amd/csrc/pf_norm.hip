@@ -744,24 +744,68 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
 // fp32 elements needed by the two-stage column reductions over a [rows, cols]
 // matrix: the norm backward writes 2 partial rows per workgroup, the column sum
 // one partial row per row chunk.
-// One launch finishing many deferred column reductions: block (x, y) handles 32 columns
-// of item y.  Items live in device memory.
+// One launch finishing many deferred column reductions: block (x, y) handles 128 columns of
+// item y (four per lane, 16-byte loads, four partial rows in flight per lane) when the item's
+// rows are 16-byte aligned, else 32 columns.  Items live in device memory.  Per column the partial
+// rows are summed in a fixed order: rows part, part + 8, ... by group `part`, then the eight groups.
 __global__ __launch_bounds__(256) void colreduce_finalize_batch_kernel(const pf_reduce_item* items) {
-  __shared__ float red[8][32];
+  __shared__ float red[8][128];
   const pf_reduce_item it = items[blockIdx.y];
   const int cl = threadIdx.x & 31, part = threadIdx.x >> 5;
-  const int64_t c = (int64_t)blockIdx.x * 32 + cl;
-  if ((int64_t)blockIdx.x * 32 >= it.cols) return;  // uniform over the block
-  float s = 0.f;
-  if (c < it.cols)
-    for (int p = part; p < it.n_partials; p += 8) s += it.ws[(int64_t)p * it.stride + c];
-  red[part][cl] = s;
-  __syncthreads();
-  if (part == 0 && c < it.cols) {
-    float t = 0.f;
+  const bool vec = ((((uintptr_t)it.ws) | ((uintptr_t)it.acc)) & 15) == 0 && it.stride % 4 == 0 && it.cols % 4 == 0;
+  if (vec) {
+    if ((int64_t)blockIdx.x * 128 >= it.cols) return;  // uniform over the block
+    const int64_t c = (int64_t)blockIdx.x * 128 + cl * 4;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c < it.cols) {
+      int p = part;
+      for (; p + 24 < it.n_partials; p += 32) {
+        const float4 a0 = *(const float4*)(it.ws + (int64_t)p * it.stride + c);
+        const float4 a1 = *(const float4*)(it.ws + (int64_t)(p + 8) * it.stride + c);
+        const float4 a2 = *(const float4*)(it.ws + (int64_t)(p + 16) * it.stride + c);
+        const float4 a3 = *(const float4*)(it.ws + (int64_t)(p + 24) * it.stride + c);
+        s.x += a0.x; s.y += a0.y; s.z += a0.z; s.w += a0.w;
+        s.x += a1.x; s.y += a1.y; s.z += a1.z; s.w += a1.w;
+        s.x += a2.x; s.y += a2.y; s.z += a2.z; s.w += a2.w;
+        s.x += a3.x; s.y += a3.y; s.z += a3.z; s.w += a3.w;
+      }
+      for (; p < it.n_partials; p += 8) {
+        const float4 a = *(const float4*)(it.ws + (int64_t)p * it.stride + c);
+        s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+      }
+    }
+    *(float4*)&red[part][cl * 4] = s;
+    __syncthreads();
+    if (part == 0 && c < it.cols) {
+      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-    for (int q = 0; q < 8; ++q) t += red[q][cl];
-    it.acc[c] += t;
+      for (int q = 0; q < 8; ++q) {
+        const float4 r = *(const float4*)&red[q][cl * 4];
+        t.x += r.x; t.y += r.y; t.z += r.z; t.w += r.w;
+      }
+      float4 a = *(float4*)(it.acc + c);
+      a.x += t.x; a.y += t.y; a.z += t.z; a.w += t.w;
+      *(float4*)(it.acc + c) = a;
+    }
+    return;
+  }
+  // four 32-column strips per block, one after the other (same grid as the vector path)
+  for (int strip = 0; strip < 4; ++strip) {
+    const int64_t c0 = ((int64_t)blockIdx.x * 4 + strip) * 32;
+    if (c0 >= it.cols) return;  // uniform over the block
+    const int64_t c = c0 + cl;
+    float s = 0.f;
+    if (c < it.cols)
+      for (int p = part; p < it.n_partials; p += 8) s += it.ws[(int64_t)p * it.stride + c];
+    __syncthreads();
+    red[part][cl] = s;
+    __syncthreads();
+    if (part == 0 && c < it.cols) {
+      float t = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) t += red[q][cl];
+      it.acc[c] += t;
+    }
   }
 }
 
@@ -790,7 +834,7 @@ extern "C" int pf_colreduce_finalize_batch(const pf_reduce_item* items_dev, int 
   PF_REQUIRE(n_items >= 0 && max_cols >= 0, "pf_colreduce_finalize_batch: bad arguments");
   if (n_items == 0 || max_cols == 0) return PF_OK;
   PF_REQUIRE(items_dev != nullptr && n_items <= 65535, "pf_colreduce_finalize_batch: bad item list");
-  hipLaunchKernelGGL(colreduce_finalize_batch_kernel, dim3((unsigned)((max_cols + 31) / 32), (unsigned)n_items),
+  hipLaunchKernelGGL(colreduce_finalize_batch_kernel, dim3((unsigned)((max_cols + 127) / 128), (unsigned)n_items),
                      dim3(256), 0, (hipStream_t)stream, items_dev);
   PF_CHECK_LAUNCH("pf_colreduce_finalize_batch");
   return PF_OK;

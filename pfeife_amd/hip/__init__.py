@@ -426,7 +426,8 @@ class HipKernels:
         table = torch.tensor(rows, dtype=torch.int64).to(items[0][0].device)
         max_cols = max(r[4] for r in rows)
         keep = (table,) + tuple(i[0] for i in items) + tuple(i[5] for i in items)
-        return self._prep("pf_colreduce_finalize_batch", (table.data_ptr(), len(rows), max_cols), keep)
+        nbytes = sum(4 * (r[2] + 2) * r[4] for r in rows)   # partial rows read, accumulator read and written
+        return self._prep("pf_colreduce_finalize_batch", (table.data_ptr(), len(rows), max_cols), keep, nbytes)
 
     # -- softmax / losses ----------------------------------------------------------
     def softmax_fwd(self, s, ld_s, p, ld_p, rows, cols, q_len, causal):
