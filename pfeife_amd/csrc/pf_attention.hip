@@ -532,24 +532,24 @@ __device__ __forceinline__ void unpack8(const uint4& r, float (&v)[8]) {
 }
 
 // Two whole [T][hd] operands of one head -> LDS [rows][HD + 8] each (rows past T and hd
-// chunks past hd are zero); 256 threads, eight 16-byte loads in flight per thread
-template <int HD>
+// chunks past hd are zero); NT threads, eight 16-byte loads in flight per thread
+template <int HD, int NT>
 __device__ __forceinline__ void load_heads(const uint16_t* x, int64_t x_st, const uint16_t* y, int64_t y_st, int T,
                                            int hd, int rows, uint16_t* sx, uint16_t* sy, int tid) {
   constexpr int VPR = HD / 8, LD = HD + 8;
   const int n = rows * VPR;
-  for (int e0 = 0; e0 < n; e0 += 256 * 4) {
+  for (int e0 = 0; e0 < n; e0 += NT * 4) {
     uint4 vx[4], vy[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int e = e0 + i * 256 + tid;
+      const int e = e0 + i * NT + tid;
       const int t = e / VPR, c = (e % VPR) * 8;
       vx[i] = e < n ? load_row8(x, x_st, t, T, c, hd) : make_uint4(0, 0, 0, 0);
       vy[i] = e < n ? load_row8(y, y_st, t, T, c, hd) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int e = e0 + i * 256 + tid;
+      const int e = e0 + i * NT + tid;
       if (e < n) {
         *(uint4*)(sx + (e / VPR) * LD + (e % VPR) * 8) = vx[i];
         *(uint4*)(sy + (e / VPR) * LD + (e % VPR) * 8) = vy[i];
@@ -558,16 +558,18 @@ __device__ __forceinline__ void load_heads(const uint16_t* x, int64_t x_st, cons
   }
 }
 
-// forward: workgroup = 128 queries of one (batch, head), wavefront = 32 of them; keys in steps of 32
-template <int DT, int HD>
-__global__ __launch_bounds__(256) void attn_fwd_short_kernel(const AttnArgs a, int rows) {
+// forward: workgroup = NT / 2 queries of one (batch, head), wavefront = 32 of them; keys in steps of 32.
+// NT = 512 (eight wavefronts) lets ONE workgroup cover a head of up to 256 tokens, so that the head's
+// K and V are fetched once instead of once per 128 queries; NT = 256 otherwise.
+template <int DT, int HD, int NT>
+__global__ __launch_bounds__(NT) void attn_fwd_short_kernel(const AttnArgs a, int rows) {
   constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
   extern __shared__ __align__(16) uint16_t smem[];
   uint16_t* sK = smem;
   uint16_t* sV = smem + rows * LD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int q0 = blockIdx.x * 128 + wave * 32;
+  const int q0 = blockIdx.x * (NT / 2) + wave * 32;
   const int qi = q0 + (lane & 31);
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const float sc = a.scale * LOG2E;
@@ -576,7 +578,7 @@ __global__ __launch_bounds__(256) void attn_fwd_short_kernel(const AttnArgs a, i
   uint4 qf[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) qf[c] = load_row8(Q, a.q_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
-  load_heads<HD>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
+  load_heads<HD, NT>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
                  sV, tid);
   __syncthreads();
   if (q0 >= a.Tq) return;   // this wavefront has no query row (no barrier follows)
@@ -655,15 +657,15 @@ __global__ __launch_bounds__(256) void attn_fwd_short_kernel(const AttnArgs a, i
 }
 
 // dQ (and delta = rowsum(dO * O), which the dK/dV kernel launched after this one reads)
-template <int DT, int HD>
-__global__ __launch_bounds__(256) void attn_dq_short_kernel(const AttnArgs a, float* delta_out, int rows) {
+template <int DT, int HD, int NT>
+__global__ __launch_bounds__(NT) void attn_dq_short_kernel(const AttnArgs a, float* delta_out, int rows) {
   constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
   extern __shared__ __align__(16) uint16_t smem[];
   uint16_t* sK = smem;
   uint16_t* sV = smem + rows * LD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int q0 = blockIdx.x * 128 + wave * 32;
+  const int q0 = blockIdx.x * (NT / 2) + wave * 32;
   const int qi = q0 + (lane & 31);
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* DO = a.d_o + b * a.do_sb + h * a.do_sh;
@@ -689,7 +691,7 @@ __global__ __launch_bounds__(256) void attn_dq_short_kernel(const AttnArgs a, fl
   const bool qok = qi < a.Tq;
   if (qok && (lane >> 5) == 0) delta_out[(int64_t)bh * a.Tq + qi] = dlt;
   const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
-  load_heads<HD>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
+  load_heads<HD, NT>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
                  sV, tid);
   __syncthreads();
   if (q0 >= a.Tq) return;
@@ -744,9 +746,9 @@ __global__ __launch_bounds__(256) void attn_dq_short_kernel(const AttnArgs a, fl
   }
 }
 
-// dK/dV: workgroup = 128 keys, wavefront = 32 of them; queries in steps of 32
-template <int DT, int HD>
-__global__ __launch_bounds__(256) void attn_dkv_short_kernel(const AttnArgs a, int rows) {
+// dK/dV: workgroup = NT / 2 keys, wavefront = 32 of them; queries in steps of 32
+template <int DT, int HD, int NT>
+__global__ __launch_bounds__(NT) void attn_dkv_short_kernel(const AttnArgs a, int rows) {
   constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
   extern __shared__ __align__(16) uint16_t smem[];
   uint16_t* sQ = smem;
@@ -755,7 +757,7 @@ __global__ __launch_bounds__(256) void attn_dkv_short_kernel(const AttnArgs a, i
   float* sDelta = sLse + rows;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int kw0 = blockIdx.x * 128 + wave * 32;
+  const int kw0 = blockIdx.x * (NT / 2) + wave * 32;
   const int kj = kw0 + (lane & 31);
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
@@ -769,12 +771,12 @@ __global__ __launch_bounds__(256) void attn_dkv_short_kernel(const AttnArgs a, i
     kf[c] = load_row8(K, a.k_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
     vf[c] = load_row8(V, a.v_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
   }
-  for (int i = tid; i < rows; i += 256) {
+  for (int i = tid; i < rows; i += NT) {
     // rows past the end: Q and dO rows are zero, lse = +inf makes their P exactly zero
     sLse[i] = i < a.Tq ? a.lse[(int64_t)bh * a.Tq + i] * LOG2E : INFINITY;
     sDelta[i] = i < a.Tq ? a.delta[(int64_t)bh * a.Tq + i] : 0.f;
   }
-  load_heads<HD>(a.q + b * a.q_sb + h * a.q_sh, a.q_st, a.d_o + b * a.do_sb + h * a.do_sh, a.do_st, a.Tq, a.hd, rows,
+  load_heads<HD, NT>(a.q + b * a.q_sb + h * a.q_sh, a.q_st, a.d_o + b * a.do_sb + h * a.do_sh, a.do_st, a.Tq, a.hd, rows,
                  sQ, sDO, tid);
   __syncthreads();
   if (kw0 >= a.Tk) return;
@@ -876,7 +878,7 @@ AttnArgs make_args(const pf_attn_desc* d) {
 // Launch of a short-sequence kernel with `lds` bytes of dynamic LDS (above 64 KB the kernel is
 // opted in once per instantiation and device).
 template <typename K, typename... Args>
-int launch_short(K kern, dim3 grid, size_t lds, hipStream_t st, Args... args) {
+int launch_short(K kern, dim3 grid, int threads, size_t lds, hipStream_t st, Args... args) {
   if (lds > 64 * 1024) {
     static std::mutex mu;
     static bool raised[64] = {};
@@ -892,19 +894,26 @@ int launch_short(K kern, dim3 grid, size_t lds, hipStream_t st, Args... args) {
       raised[dev] = true;
     }
   }
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, st, args...);
+  hipLaunchKernelGGL(kern, grid, dim3((unsigned)threads), lds, st, args...);
   return PF_OK;
 }
 
-#define PF_ATTN_SHORT(KERNEL, rc, grid, lds, st, dt, hd, ...)                                            \
-  do {                                                                                                 \
-    if (dt == PF_F16) {                                                                                \
-      if (hd <= 64) rc = launch_short(KERNEL<PF_F16, 64>, grid, (lds)(64), st, __VA_ARGS__);            \
-      else rc = launch_short(KERNEL<PF_F16, 96>, grid, (lds)(96), st, __VA_ARGS__);                     \
-    } else {                                                                                           \
-      if (hd <= 64) rc = launch_short(KERNEL<PF_BF16, 64>, grid, (lds)(64), st, __VA_ARGS__);           \
-      else rc = launch_short(KERNEL<PF_BF16, 96>, grid, (lds)(96), st, __VA_ARGS__);                    \
-    }                                                                                                  \
+// T: tokens along the axis the workgroups divide (queries, or keys for dK/dV).  Heads of 129-256
+// tokens with head dim <= 64 take one 512-thread workgroup each (the wider head dims need more
+// registers per wavefront than two wavefronts per SIMD leave).
+#define PF_ATTN_SHORT(KERNEL, rc, T, BH, lds, st, dt, hd, ...)                                                   \
+  do {                                                                                                         \
+    const bool wide = (hd) <= 64 && (T) > 128 && (T) <= 256;                                                   \
+    const dim3 grid_((unsigned)(wide ? 1 : ((T) + 127) / 128), (unsigned)(BH));                                \
+    if (dt == PF_F16) {                                                                                        \
+      if (wide) rc = launch_short(KERNEL<PF_F16, 64, 512>, grid_, 512, (lds)(64), st, __VA_ARGS__);             \
+      else if (hd <= 64) rc = launch_short(KERNEL<PF_F16, 64, 256>, grid_, 256, (lds)(64), st, __VA_ARGS__);    \
+      else rc = launch_short(KERNEL<PF_F16, 96, 256>, grid_, 256, (lds)(96), st, __VA_ARGS__);                  \
+    } else {                                                                                                   \
+      if (wide) rc = launch_short(KERNEL<PF_BF16, 64, 512>, grid_, 512, (lds)(64), st, __VA_ARGS__);            \
+      else if (hd <= 64) rc = launch_short(KERNEL<PF_BF16, 64, 256>, grid_, 256, (lds)(64), st, __VA_ARGS__);   \
+      else rc = launch_short(KERNEL<PF_BF16, 96, 256>, grid_, 256, (lds)(96), st, __VA_ARGS__);                 \
+    }                                                                                                          \
   } while (0)
 
 #define PF_ATTN_DISPATCH(KERNEL, grid, st, a, dt, hd)                                          \
@@ -928,7 +937,7 @@ extern "C" int pf_attention_fwd(const pf_attn_desc* d, void* stream) {
   if (d->Tq <= SHORT_T && d->Tk <= SHORT_T) {
     const int rows = (d->Tk + 31) / 32 * 32;
     auto lds = [rows](int HD) { return (size_t)2 * rows * (HD + 8) * 2; };
-    PF_ATTN_SHORT(attn_fwd_short_kernel, rc, grid, lds, (hipStream_t)stream, d->dtype, d->hd, a, rows);
+    PF_ATTN_SHORT(attn_fwd_short_kernel, rc, d->Tq, d->B * d->H, lds, (hipStream_t)stream, d->dtype, d->hd, a, rows);
     if (rc != PF_OK) return rc;
   } else {
     PF_ATTN_DISPATCH(attn_fwd_kernel, grid, (hipStream_t)stream, a, d->dtype, d->hd);
@@ -958,9 +967,9 @@ extern "C" int pf_attention_bwd(const pf_attn_desc* d, void* stream) {
     const int rows_k = (d->Tk + 31) / 32 * 32, rows_q = (d->Tq + 31) / 32 * 32;
     auto lds_q = [rows_k](int HD) { return (size_t)2 * rows_k * (HD + 8) * 2; };
     auto lds_k = [rows_q](int HD) { return (size_t)2 * rows_q * (HD + 8) * 2 + (size_t)rows_q * 8; };
-    PF_ATTN_SHORT(attn_dq_short_kernel, rc, gq, lds_q, st, d->dtype, d->hd, a, d->delta, rows_k);
+    PF_ATTN_SHORT(attn_dq_short_kernel, rc, d->Tq, d->B * d->H, lds_q, st, d->dtype, d->hd, a, d->delta, rows_k);
     if (rc != PF_OK) return rc;
-    PF_ATTN_SHORT(attn_dkv_short_kernel, rc, gk, lds_k, st, d->dtype, d->hd, a, rows_q);
+    PF_ATTN_SHORT(attn_dkv_short_kernel, rc, d->Tk, d->B * d->H, lds_k, st, d->dtype, d->hd, a, rows_q);
     if (rc != PF_OK) return rc;
     PF_CHECK_LAUNCH("pf_attention_bwd");
     return PF_OK;
