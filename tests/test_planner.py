@@ -258,6 +258,50 @@ def test_split_points_none_profiles_and_partitions(capsys):
         assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
 
 
+def test_split_points_none_on_a_looped_decoder():
+    """Four stages on two ranks (loop_cnt=2) of a decoder whose rotary tables every block reads:
+    the planner has to find three cuts among the block boundaries and the step has to compute what
+    plain accumulation computes."""
+    from oracle.kernels_oracle import OracleKernels
+    from pfeife_amd.bench_models.llama import LlamaConfig, LlamaForCausalLM
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife, net_states, partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = LlamaConfig(vocab=256, dim=64, layers=4, heads=4, ffn=176, max_seq=32)
+    torch.manual_seed(0)
+    model = LlamaForCausalLM(cfg)
+    ref = copy.deepcopy(model)
+    torch._dynamo.reset()
+    net_states._reset_state_for_tests()
+    initialize_pfeife(device="cpu")
+    option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=2, split_points=None, loop_cnt=2,
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = PartialRunner(option, kernels=OracleKernels("cpu"))
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(tok):
+        loss = cmodel(tok, tok)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    ids = torch.randint(0, cfg.vocab, (8, 32), generator=torch.Generator().manual_seed(1))
+    losses = runner.step(ids)
+    worker = runner.worker
+    plan, prof = worker.plan, worker.profile
+    assert len(plan.split_points) == 3 and len(worker.part_graph.nodes) == 4
+    assert plan.split_points == sorted(set(plan.split_points))
+    cand = cut_candidates(prof)
+    assert all(p in cand and prof.cut_ok[p] for p in plan.split_points)
+    assert plan.sched_params.node_cnt == 4 and plan.sched_params.device_cnt == 2
+    for chunk, got in zip(ids.chunk(4), losses):
+        want = ref(chunk, chunk)
+        want.backward()
+        assert abs(float(got) - float(want.detach())) <= 1e-5 * abs(float(want.detach()))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+
+
 def test_manual_split_between_a_tuple_and_its_users_is_refused():
     from oracle.kernels_oracle import OracleKernels
     from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
