@@ -326,6 +326,71 @@ def cpu_baseline(name):
                            "" if family != "llama" else "; 512-token sequences, attention cost scaled linearly"))
 
 
+def torch_eager_gpu(name, device, steps=5, warmup=2):
+    """The same optimisation step in plain PyTorch on the same GPU: the un-partitioned model run
+    eagerly under torch.autocast, one forward + backward per micro-batch with gradient accumulation,
+    torch.amp.GradScaler for fp16 and torch.optim.Adam.  This is what the reference's stages execute
+    (eager ATen modules, pfeife/mp/worker.py:1457-1494 and 1585-1587, GradScaler :135-140) when all of
+    them sit on one device, without its queues and copies.  Reported beside `value`, never as it."""
+    import torch
+    import torch.nn.functional as F
+
+    from pfeife_amd.bench_models import llama, vit
+
+    family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
+    if family not in ("vit", "llama"):
+        return None
+    torch.manual_seed(42)
+    g = torch.Generator().manual_seed(42)
+    if family == "vit":
+        cfg = getattr(vit, cfg_name)
+        model = vit.VisionTransformer(cfg).to(device)
+        x = torch.randn(batch, cfg.channels, cfg.image_size, cfg.image_size, generator=g).to(device)
+        y = torch.randint(0, cfg.num_classes, (batch,), generator=g).to(device)
+
+        def loss_of(xb, yb):
+            return F.cross_entropy(model(xb).float(), yb)
+    else:
+        cfg = getattr(llama, cfg_name)
+        model = llama.LlamaForCausalLM(cfg).to(device)
+        x = torch.randint(0, cfg.vocab, (batch, cfg.max_seq), generator=g).to(device)
+        y = x
+
+        def loss_of(xb, yb):
+            return model(xb, yb)
+    dtype = {"fp16": torch.float16, "bf16": torch.bfloat16}.get(mixed)
+    opt = torch.optim.Adam(model.parameters(), lr=1e-5)
+    scaler = torch.amp.GradScaler("cuda", enabled=mixed == "fp16")
+    xs, ys = x.chunk(batch_cnt), y.chunk(batch_cnt)
+
+    def step():
+        opt.zero_grad(set_to_none=False)
+        for xb, yb in zip(xs, ys):
+            with torch.autocast("cuda", dtype=dtype, enabled=dtype is not None):
+                loss = loss_of(xb, yb)
+            scaler.scale(loss).backward()
+        scaler.step(opt)
+        scaler.update()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    last = float(loss)
+    del opt, model
+    torch.cuda.empty_cache()
+    return dict(value=round(batch * steps / dt, 2), unit="samples/s", ms_per_step=round(1e3 * dt / steps, 3), steps=steps,
+                sample="%s in PyTorch %s eager on this GPU: autocast %s, %d micro-batches x %d with gradient "
+                       "accumulation, GradScaler %s, torch.optim.Adam; last loss %.4f" % (
+                           cfg_name, torch.__version__, mixed, batch_cnt, batch // batch_cnt,
+                           "on" if mixed == "fp16" else "off", last))
+
+
 def model_flops_per_step(info):
     cfg, samples = info["cfg"], info["batch"]
     if info["family"] in ("vit", "vit_share"):
@@ -441,6 +506,8 @@ def main():
     ap.add_argument("--workload", default="vit_l16_fp16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-eager-baseline", action="store_true",
+                    help="skip timing the same step in plain PyTorch eager on this GPU")
     ap.add_argument("--no-others", action="store_true",
                     help="skip the bounded runs of the other GPU workloads that follow the headline measurement")
     ap.add_argument("--no-graph", action="store_true",
@@ -480,6 +547,14 @@ def main():
             launch(torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         del src, dst
+    eager = None
+    if not args.no_eager_baseline:
+        log("[bench] timing plain PyTorch eager on this GPU ...")
+        try:
+            eager = torch_eager_gpu(args.workload, device)
+        except Exception as e:   # report, do not lose the headline line
+            eager = dict(skipped="failed: %s" % (str(e)[:200],))
+        log("[bench] torch eager on this GPU", eager)
     cpu = None
     if not args.no_cpu_baseline:
         log("[bench] timing the CPU baseline ...")
@@ -527,6 +602,7 @@ def main():
         "roofline": head["roof"],
         "hbm_kernels": head["hbm"],
         "cpu_baseline": cpu,
+        "torch_eager_gpu": eager,
         "model_tflops": head["model_tflops"],
         "host_enqueue_ms_per_step": round(head["host_ms"], 3),
         "loss_scaling": head["loss_scaling"],
