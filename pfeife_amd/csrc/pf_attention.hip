@@ -19,6 +19,8 @@
 // strides (batch, head, token) and unit stride along hd, so heads can live inside a
 // packed qkv projection and the output can be token-major.
 #include <mutex>
+#include <set>
+#include <utility>
 
 #include "pf_common.h"
 
@@ -558,9 +560,10 @@ __device__ __forceinline__ void load_heads(const uint16_t* x, int64_t x_st, cons
   }
 }
 
-// forward: workgroup = NT / 2 queries of one (batch, head), wavefront = 32 of them; keys in steps of 32.
-// NT = 512 (eight wavefronts) lets ONE workgroup cover a head of up to 256 tokens, so that the head's
-// K and V are fetched once instead of once per 128 queries; NT = 256 otherwise.
+// forward: workgroup = NT / 2 queries of one (batch, head) at a time, wavefront = 32 of them; keys in
+// steps of 32.  A wavefront whose tile lies past what the grid covers at once (gridDim.x * NT / 2
+// queries) takes it in a second pass.  NT = 512 (eight wavefronts) lets ONE workgroup cover a whole head,
+// so that the head's K and V are fetched once instead of once per 128 queries; NT = 256 otherwise.
 template <int DT, int HD, int NT>
 __global__ __launch_bounds__(NT) void attn_fwd_short_kernel(const AttnArgs a, int rows) {
   constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8;
@@ -569,20 +572,22 @@ __global__ __launch_bounds__(NT) void attn_fwd_short_kernel(const AttnArgs a, in
   uint16_t* sV = smem + rows * LD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int q0 = blockIdx.x * (NT / 2) + wave * 32;
-  const int qi = q0 + (lane & 31);
+  const int q_step = (int)gridDim.x * (NT / 2);
+  int q0 = blockIdx.x * (NT / 2) + wave * 32;
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const float sc = a.scale * LOG2E;
   const int shift = a.Tk - a.Tq;
 
-  uint4 qf[NC];
+  uint4 qf[NC];   // the first tile's queries are requested before the head is loaded
 #pragma unroll
-  for (int c = 0; c < NC; ++c) qf[c] = load_row8(Q, a.q_st, qi, a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
+  for (int c = 0; c < NC; ++c) qf[c] = load_row8(Q, a.q_st, q0 + (lane & 31), a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
   load_heads<HD, NT>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
                  sV, tid);
   __syncthreads();
-  if (q0 >= a.Tq) return;   // this wavefront has no query row (no barrier follows)
-
+  // no barrier follows: a wavefront without a query tile leaves, one with several (the tiles past
+  // what the grid covers at once, e.g. the 257th token of a 256-token-wide grid) loops
+  for (; q0 < a.Tq; q0 += q_step) {
+  const int qi = q0 + (lane & 31);
   float16_t oacc[NO];
 #pragma unroll
   for (int o = 0; o < NO; ++o)
@@ -654,6 +659,12 @@ __global__ __launch_bounds__(NT) void attn_fwd_short_kernel(const AttnArgs a, in
       }
     if ((lane >> 5) == 0) a.lse[((int64_t)bh) * a.Tq + qi] = (l > 0.f) ? (m * sc + log2f(l)) / LOG2E : -INFINITY;
   }
+  if (q0 + q_step < a.Tq) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      qf[c] = load_row8(Q, a.q_st, q0 + q_step + (lane & 31), a.Tq, c * 16 + (lane >> 5) * 8, a.hd);
+  }
+  }
 }
 
 // dQ (and delta = rowsum(dO * O), which the dK/dV kernel launched after this one reads)
@@ -665,8 +676,8 @@ __global__ __launch_bounds__(NT) void attn_dq_short_kernel(const AttnArgs a, flo
   uint16_t* sV = smem + rows * LD;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int q0 = blockIdx.x * (NT / 2) + wave * 32;
-  const int qi = q0 + (lane & 31);
+  const int q_step = (int)gridDim.x * (NT / 2);
+  int q0 = blockIdx.x * (NT / 2) + wave * 32;
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* DO = a.d_o + b * a.do_sb + h * a.do_sh;
   const uint16_t* OO = a.o + b * a.o_sb + h * a.o_sh;
@@ -674,28 +685,35 @@ __global__ __launch_bounds__(NT) void attn_dq_short_kernel(const AttnArgs a, flo
   const int shift = a.Tk - a.Tq;
 
   uint4 qf[NC], dof[NC];
-  float dlt = 0.f;
+  float dlt, lse2;
+  // this lane's query row of the tile at `qs`: Q, dO, delta (also written out) and the row's lse
+  auto load_rows = [&](int qs) {
+    const int qr = qs + (lane & 31);
+    dlt = 0.f;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int h0 = c * 16 + (lane >> 5) * 8;
-    qf[c] = load_row8(Q, a.q_st, qi, a.Tq, h0, a.hd);
-    dof[c] = load_row8(DO, a.do_st, qi, a.Tq, h0, a.hd);
-    const uint4 of = load_row8(OO, a.o_st, qi, a.Tq, h0, a.hd);
-    float x[8], y[8];
-    unpack8<DT>(dof[c], x);
-    unpack8<DT>(of, y);
+    for (int c = 0; c < NC; ++c) {
+      const int h0 = c * 16 + (lane >> 5) * 8;
+      qf[c] = load_row8(Q, a.q_st, qr, a.Tq, h0, a.hd);
+      dof[c] = load_row8(DO, a.do_st, qr, a.Tq, h0, a.hd);
+      const uint4 of = load_row8(OO, a.o_st, qr, a.Tq, h0, a.hd);
+      float x[8], y[8];
+      unpack8<DT>(dof[c], x);
+      unpack8<DT>(of, y);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) dlt += x[k] * y[k];
-  }
-  dlt += __shfl_xor(dlt, 32, 64);
-  const bool qok = qi < a.Tq;
-  if (qok && (lane >> 5) == 0) delta_out[(int64_t)bh * a.Tq + qi] = dlt;
-  const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
+      for (int k = 0; k < 8; ++k) dlt += x[k] * y[k];
+    }
+    dlt += __shfl_xor(dlt, 32, 64);
+    if (qr < a.Tq && (lane >> 5) == 0) delta_out[(int64_t)bh * a.Tq + qr] = dlt;
+    lse2 = qr < a.Tq ? a.lse[(int64_t)bh * a.Tq + qr] * LOG2E : INFINITY;
+  };
+  load_rows(q0);   // the first tile's rows are requested before the head is loaded
   load_heads<HD, NT>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows, sK,
                  sV, tid);
   __syncthreads();
-  if (q0 >= a.Tq) return;
-
+  // no barrier follows: a wavefront without a query tile leaves, one with several loops
+  for (; q0 < a.Tq; q0 += q_step) {
+  const int qi = q0 + (lane & 31);
+  const bool qok = qi < a.Tq;
   float16_t acc[NO];
 #pragma unroll
   for (int o = 0; o < NO; ++o)
@@ -744,6 +762,8 @@ __global__ __launch_bounds__(NT) void attn_dq_short_kernel(const AttnArgs a, flo
                                           M32<DT>::pack(acc[o][4 * g + 2] * a.scale, acc[o][4 * g + 3] * a.scale));
       }
   }
+  if (q0 + q_step < a.Tq) load_rows(q0 + q_step);
+  }
 }
 
 // dK/dV: workgroup = NT / 2 keys, wavefront = 32 of them; queries in steps of 32
@@ -757,20 +777,22 @@ __global__ __launch_bounds__(NT) void attn_dkv_short_kernel(const AttnArgs a, in
   float* sDelta = sLse + rows;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-  const int kw0 = blockIdx.x * (NT / 2) + wave * 32;
-  const int kj = kw0 + (lane & 31);
+  const int k_step = (int)gridDim.x * (NT / 2);
+  int kw0 = blockIdx.x * (NT / 2) + wave * 32;
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t* V = a.v + b * a.v_sb + h * a.v_sh;
   const float sc = a.scale * LOG2E;
   const int shift = a.Tk - a.Tq;
-  const bool kok = kj < a.Tk;
 
   uint4 kf[NC], vf[NC];
+  auto load_rows = [&](int ks) {   // this lane's key row of the tile at `ks`
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    kf[c] = load_row8(K, a.k_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
-    vf[c] = load_row8(V, a.v_st, kj, a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
-  }
+    for (int c = 0; c < NC; ++c) {
+      kf[c] = load_row8(K, a.k_st, ks + (lane & 31), a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
+      vf[c] = load_row8(V, a.v_st, ks + (lane & 31), a.Tk, c * 16 + (lane >> 5) * 8, a.hd);
+    }
+  };
+  load_rows(kw0);   // the first tile's rows are requested before the head is loaded
   for (int i = tid; i < rows; i += NT) {
     // rows past the end: Q and dO rows are zero, lse = +inf makes their P exactly zero
     sLse[i] = i < a.Tq ? a.lse[(int64_t)bh * a.Tq + i] * LOG2E : INFINITY;
@@ -779,8 +801,10 @@ __global__ __launch_bounds__(NT) void attn_dkv_short_kernel(const AttnArgs a, in
   load_heads<HD, NT>(a.q + b * a.q_sb + h * a.q_sh, a.q_st, a.d_o + b * a.do_sb + h * a.do_sh, a.do_st, a.Tq, a.hd, rows,
                  sQ, sDO, tid);
   __syncthreads();
-  if (kw0 >= a.Tk) return;
-
+  // no barrier follows: a wavefront without a key tile leaves, one with several loops
+  for (; kw0 < a.Tk; kw0 += k_step) {
+  const int kj = kw0 + (lane & 31);
+  const bool kok = kj < a.Tk;
   float16_t dk[NO], dv[NO];
 #pragma unroll
   for (int o = 0; o < NO; ++o)
@@ -834,6 +858,8 @@ __global__ __launch_bounds__(NT) void attn_dkv_short_kernel(const AttnArgs a, in
         }
       }
   }
+  if (kw0 + k_step < a.Tk) load_rows(kw0 + k_step);
+  }
 }
 
 bool strides_ok(const void* p, int64_t sb, int64_t sh, int64_t st) {
@@ -876,42 +902,50 @@ AttnArgs make_args(const pf_attn_desc* d) {
 }  // namespace
 
 // Launch of a short-sequence kernel with `lds` bytes of dynamic LDS (above 64 KB the kernel is
-// opted in once per instantiation and device).
+// opted in once per kernel and device).
 template <typename K, typename... Args>
 int launch_short(K kern, dim3 grid, int threads, size_t lds, hipStream_t st, Args... args) {
   if (lds > 64 * 1024) {
     static std::mutex mu;
-    static bool raised[64] = {};
+    static std::set<std::pair<const void*, int>> raised;   // instantiations share this function's type
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
     std::lock_guard<std::mutex> lock(mu);
-    if (!raised[dev]) {
+    if (!raised.count({(const void*)kern, dev})) {
       const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) {
         pf_set_error("pf_attention: cannot raise dynamic LDS: %s", hipGetErrorString(e));
         return PF_ERR_HIP;
       }
-      raised[dev] = true;
+      raised.insert({(const void*)kern, dev});
     }
   }
   hipLaunchKernelGGL(kern, grid, dim3((unsigned)threads), lds, st, args...);
   return PF_OK;
 }
 
-// T: tokens along the axis the workgroups divide (queries, or keys for dK/dV).  Heads of 129-256
-// tokens with head dim <= 64 take one 512-thread workgroup each (the wider head dims need more
-// registers per wavefront than two wavefronts per SIMD leave).
-#define PF_ATTN_SHORT(KERNEL, rc, T, BH, lds, st, dt, hd, ...)                                                   \
+// T: tokens along the axis the workgroups divide (queries, or keys for dK/dV), in tiles of 32 per
+// wavefront.  A head of more than 128 tokens takes ONE workgroup of eight wavefronts (its two LDS
+// operands are fetched once; the tiles past the eighth, e.g. the 257th token's, are a second pass of
+// the first wavefronts).  NT96: workgroup size for head dims above 64, 512 where the kernel's
+// registers allow two wavefronts per SIMD (forward, dQ), else 256: then every workgroup takes four
+// tiles and a remainder of one or two tiles becomes a second pass instead of a workgroup (and a
+// load of the whole head) of its own.
+#define PF_ATTN_SHORT(KERNEL, NT96, rc, T, BH, lds, st, dt, hd, ...)                                            \
   do {                                                                                                         \
-    const bool wide = (hd) <= 64 && (T) > 128 && (T) <= 256;                                                   \
-    const dim3 grid_((unsigned)(wide ? 1 : ((T) + 127) / 128), (unsigned)(BH));                                \
+    const int tiles_ = ((T) + 31) / 32;                                                                        \
+    const bool w64_ = (hd) <= 64 && (T) > 128, w96_ = (hd) > 64 && (NT96) == 512 && (T) > 128;                  \
+    const int gx_ = (w64_ || w96_) ? 1 : ((tiles_ + 1) / 4 > 1 ? (tiles_ + 1) / 4 : 1);                         \
+    const dim3 grid_((unsigned)gx_, (unsigned)(BH));                                                           \
     if (dt == PF_F16) {                                                                                        \
-      if (wide) rc = launch_short(KERNEL<PF_F16, 64, 512>, grid_, 512, (lds)(64), st, __VA_ARGS__);             \
+      if (w64_) rc = launch_short(KERNEL<PF_F16, 64, 512>, grid_, 512, (lds)(64), st, __VA_ARGS__);             \
       else if (hd <= 64) rc = launch_short(KERNEL<PF_F16, 64, 256>, grid_, 256, (lds)(64), st, __VA_ARGS__);    \
+      else if (w96_) rc = launch_short(KERNEL<PF_F16, 96, NT96>, grid_, NT96, (lds)(96), st, __VA_ARGS__);      \
       else rc = launch_short(KERNEL<PF_F16, 96, 256>, grid_, 256, (lds)(96), st, __VA_ARGS__);                  \
     } else {                                                                                                   \
-      if (wide) rc = launch_short(KERNEL<PF_BF16, 64, 512>, grid_, 512, (lds)(64), st, __VA_ARGS__);            \
+      if (w64_) rc = launch_short(KERNEL<PF_BF16, 64, 512>, grid_, 512, (lds)(64), st, __VA_ARGS__);            \
       else if (hd <= 64) rc = launch_short(KERNEL<PF_BF16, 64, 256>, grid_, 256, (lds)(64), st, __VA_ARGS__);   \
+      else if (w96_) rc = launch_short(KERNEL<PF_BF16, 96, NT96>, grid_, NT96, (lds)(96), st, __VA_ARGS__);     \
       else rc = launch_short(KERNEL<PF_BF16, 96, 256>, grid_, 256, (lds)(96), st, __VA_ARGS__);                 \
     }                                                                                                          \
   } while (0)
@@ -937,7 +971,7 @@ extern "C" int pf_attention_fwd(const pf_attn_desc* d, void* stream) {
   if (d->Tq <= SHORT_T && d->Tk <= SHORT_T) {
     const int rows = (d->Tk + 31) / 32 * 32;
     auto lds = [rows](int HD) { return (size_t)2 * rows * (HD + 8) * 2; };
-    PF_ATTN_SHORT(attn_fwd_short_kernel, rc, d->Tq, d->B * d->H, lds, (hipStream_t)stream, d->dtype, d->hd, a, rows);
+    PF_ATTN_SHORT(attn_fwd_short_kernel, 512, rc, d->Tq, d->B * d->H, lds, (hipStream_t)stream, d->dtype, d->hd, a, rows);
     if (rc != PF_OK) return rc;
   } else {
     PF_ATTN_DISPATCH(attn_fwd_kernel, grid, (hipStream_t)stream, a, d->dtype, d->hd);
@@ -967,9 +1001,9 @@ extern "C" int pf_attention_bwd(const pf_attn_desc* d, void* stream) {
     const int rows_k = (d->Tk + 31) / 32 * 32, rows_q = (d->Tq + 31) / 32 * 32;
     auto lds_q = [rows_k](int HD) { return (size_t)2 * rows_k * (HD + 8) * 2; };
     auto lds_k = [rows_q](int HD) { return (size_t)2 * rows_q * (HD + 8) * 2 + (size_t)rows_q * 8; };
-    PF_ATTN_SHORT(attn_dq_short_kernel, rc, d->Tq, d->B * d->H, lds_q, st, d->dtype, d->hd, a, d->delta, rows_k);
+    PF_ATTN_SHORT(attn_dq_short_kernel, 512, rc, d->Tq, d->B * d->H, lds_q, st, d->dtype, d->hd, a, d->delta, rows_k);
     if (rc != PF_OK) return rc;
-    PF_ATTN_SHORT(attn_dkv_short_kernel, rc, d->Tk, d->B * d->H, lds_k, st, d->dtype, d->hd, a, rows_q);
+    PF_ATTN_SHORT(attn_dkv_short_kernel, 256, rc, d->Tk, d->B * d->H, lds_k, st, d->dtype, d->hd, a, rows_q);
     if (rc != PF_OK) return rc;
     PF_CHECK_LAUNCH("pf_attention_bwd");
     return PF_OK;

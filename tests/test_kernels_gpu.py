@@ -490,6 +490,8 @@ def test_deferred_reductions_match_immediate(hip):
     dict(B=2, H=2, Tq=100, Tk=130, hd=64, causal=1, packed=False),   # short causal, more keys than queries
     dict(B=1, H=3, Tq=200, Tk=40, hd=88, causal=0, packed=False),    # short, several query blocks, few keys
     dict(B=1, H=2, Tq=320, Tk=290, hd=64, causal=0, packed=False),   # beyond the whole-head-in-LDS kernels
+    dict(B=2, H=2, Tq=280, Tk=280, hd=64, causal=1, packed=False),   # ninth tile: second pass of the first wavefront
+    dict(B=1, H=2, Tq=160, Tk=170, hd=96, causal=0, packed=False),   # head dim 96: six key tiles in one 4-wavefront workgroup
 ])
 def test_fused_attention(hip, oracle, dtype, case):
     B, H, Tq, Tk, hd = case["B"], case["H"], case["Tq"], case["Tk"], case["hd"]
