@@ -364,7 +364,9 @@ int pf_transpose_cast(const void* src, int src_dtype, int64_t ld_src, void* dst,
 int pf_fill(void* dst, int dtype, float value, int64_t n, void* stream);
 /* Generic strided copy with dtype conversion of a tensor of up to 6 dims:
  * dst[idx . dst_strides] = src[idx . src_strides]  (strides in elements). Used
- * for layout changes that are not views: patch extraction, head merges, cat.
+ * for layout changes that are not views: patch extraction, head merges, cat,
+ * NCHW <-> NHWC and convolution-weight re-layouts (a copy whose source and destination are
+ * contiguous along different dimensions is tiled through LDS as a batched transpose).
  * Integer dtypes (token ids) are copied raw: same dtype on both sides, no accumulate. */
 int pf_copy_strided(const void* src, int src_dtype, const int64_t* src_strides, void* dst, int dst_dtype,
                     const int64_t* dst_strides, const int64_t* sizes, int ndim, int accumulate, void* stream);

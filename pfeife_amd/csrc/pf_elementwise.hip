@@ -211,6 +211,50 @@ __global__ __launch_bounds__(EW_BLOCK) void copy_strided_raw_kernel(const U* src
   }
 }
 
+// Strided copy in which the source is contiguous along one dimension (`j`) and the destination
+// along another (`l`): a batched transpose (NCHW <-> NHWC, [B, C, T] <-> [B, T, C], a convolution
+// weight [out, in, 9] <-> [out, 9, in]).  64x64 tiles over (j, l) go through LDS so that reads run
+// along j and writes along l, both in runs of up to 64 elements; the remaining dimensions are the
+// batch (blockIdx.z).
+struct TransposeDesc {
+  int64_t nj, nl;            // extents of dimensions j and l
+  int64_t s_l, d_j;          // source stride along l, destination stride along j
+  int64_t bsize[4], bss[4], bds[4];
+  int nb;
+};
+__global__ __launch_bounds__(256) void copy_transpose_kernel(const void* src, int sdt, void* dst, int ddt,
+                                                             TransposeDesc td, int accumulate) {
+  __shared__ float tile[64][65];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  int64_t rem = blockIdx.z, so = 0, dof = 0;
+#pragma unroll
+  for (int k = 3; k >= 0; --k) {
+    if (k < td.nb) {
+      const int64_t idx = rem % td.bsize[k];
+      rem /= td.bsize[k];
+      so += idx * td.bss[k];
+      dof += idx * td.bds[k];
+    }
+  }
+  const int64_t j0 = (int64_t)blockIdx.x * 64, l0 = (int64_t)blockIdx.y * 64;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t l = l0 + ty + i * 4, j = j0 + tx;
+    tile[ty + i * 4][tx] = (l < td.nl && j < td.nj) ? pf_load_as_f32(src, so + l * td.s_l + j, sdt) : 0.f;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int64_t j = j0 + ty + i * 4, l = l0 + tx;
+    if (j < td.nj && l < td.nl) {
+      const int64_t o = dof + j * td.d_j + l;
+      float v = tile[tx][ty + i * 4];
+      if (accumulate) v += pf_load_as_f32(dst, o, ddt);
+      pf_store_from_f32(dst, o, ddt, v);
+    }
+  }
+}
+
 // dst[c, r] = src[r, c] with dtype conversion, 64x64 tiles through LDS so that both
 // the reads and the writes are contiguous runs of 64 elements
 __global__ __launch_bounds__(256) void transpose_cast_kernel(const void* src, int sdt, int64_t ld_src, void* dst,
@@ -576,6 +620,35 @@ extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* sr
     hipLaunchKernelGGL(copy_strided_kernel<8>, ew_grid(total), dim3(EW_BLOCK), 0, st, src, src_dtype, dst, dst_dtype,
                        cd, total, accumulate);
   } else {
+    // batched transpose: the source is contiguous along one dimension (p), the destination along another (q)
+    int pdim = -1, qdim = -1;
+    if (ndim >= 2 && ndim <= 6) {
+      for (int k = ndim - 1; k >= 0; --k) {
+        if (pdim < 0 && src_strides[k] == 1 && sizes[k] >= 2) pdim = k;
+        if (qdim < 0 && dst_strides[k] == 1 && sizes[k] >= 2) qdim = k;
+      }
+    }
+    if (pdim >= 0 && qdim >= 0 && pdim != qdim && ndim - 2 <= 4) {
+      TransposeDesc td;
+      td.nj = sizes[pdim]; td.nl = sizes[qdim];
+      td.s_l = src_strides[qdim]; td.d_j = dst_strides[pdim];
+      td.nb = 0;
+      int64_t batch = 1;
+      for (int k = 0; k < ndim; ++k) {
+        if (k == pdim || k == qdim) continue;
+        td.bsize[td.nb] = sizes[k]; td.bss[td.nb] = src_strides[k]; td.bds[td.nb] = dst_strides[k];
+        ++td.nb;
+        batch *= sizes[k];
+      }
+      for (int k = td.nb; k < 4; ++k) { td.bsize[k] = 1; td.bss[k] = 0; td.bds[k] = 0; }
+      const int64_t gx = (td.nj + 63) / 64, gy = (td.nl + 63) / 64;
+      if (batch <= 65535 && gy <= 65535) {
+        hipLaunchKernelGGL(copy_transpose_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)batch), dim3(256), 0, st, src,
+                           src_dtype, dst, dst_dtype, td, accumulate);
+        PF_CHECK_LAUNCH("pf_copy_strided");
+        return PF_OK;
+      }
+    }
     hipLaunchKernelGGL(copy_strided_kernel<1>, ew_grid(total), dim3(EW_BLOCK), 0, st, src, src_dtype, dst, dst_dtype,
                        cd, total, accumulate);
   }

@@ -186,6 +186,7 @@ enum {
   EC_ACC32 = 4,    // C fp32 accumulated in place (beta = 1)
   EC_DACT16 = 5,   // C 16-bit, multiplied by GELU'(aux_in)
   EC_ACC16 = 6,    // C 16-bit accumulated in place (beta = 1)
+  EC_RES16 = 7,    // C 16-bit, residual of the same 16-bit dtype added (a 16-bit residual stream)
 };
 // Epilogue class of a problem (see the EC_* list): the straight-line classes need 16-byte
 // vector access to every epilogue operand, whole 8-column groups, and 32-bit byte offsets.
@@ -195,7 +196,7 @@ inline int epi_class(const pf_gemm_desc& d, int vec_ok) {
   if (d.M * d.ldc * 4 >= lim) return EC_GENERIC;
   if (d.aux_out && d.M * d.ld_aux_out * 2 >= lim) return EC_GENERIC;
   if (d.aux_in && d.M * d.ld_aux_in * 2 >= lim) return EC_GENERIC;
-  if (d.residual && d.M * d.ld_res * 4 >= lim) return EC_GENERIC;
+  if (d.residual && d.M * d.ld_res * 4 >= lim) return EC_GENERIC;   // (bounds the 16-bit case too)
   const bool c16 = d.c_dtype == d.in_dtype, c32 = d.c_dtype == PF_F32;
   if (!c16 && !c32) return EC_GENERIC;
   const bool act = d.act != PF_ACT_NONE, dact = d.dact != PF_ACT_NONE, res = d.residual != nullptr, beta = d.beta != 0;
@@ -205,7 +206,7 @@ inline int epi_class(const pf_gemm_desc& d, int vec_ok) {
   if (n > 1) return EC_GENERIC;
   if (act) return (c16 && d.act == PF_ACT_GELU) ? EC_ACT16 : EC_GENERIC;
   if (dact) return (c16 && d.dact == PF_ACT_GELU) ? EC_DACT16 : EC_GENERIC;
-  if (res) return (c32 && d.res_dtype == PF_F32) ? EC_RES32 : EC_GENERIC;
+  if (res) return (c32 && d.res_dtype == PF_F32) ? EC_RES32 : ((c16 && d.res_dtype == d.in_dtype) ? EC_RES16 : EC_GENERIC);
   return c32 ? EC_ACC32 : EC_ACC16;
 }
 

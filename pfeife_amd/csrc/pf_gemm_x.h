@@ -367,7 +367,7 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
     // order, "those loads have landed" is "at most <the operations issued after them>
     // outstanding", a compile-time number because nothing here is predicated.
     constexpr bool C32 = EC == EC_STORE32 || EC == EC_RES32 || EC == EC_ACC32;
-    constexpr bool LOADS = EC == EC_RES32 || EC == EC_ACC32 || EC == EC_DACT16 || EC == EC_ACC16;
+    constexpr bool LOADS = EC == EC_RES32 || EC == EC_ACC32 || EC == EC_DACT16 || EC == EC_ACC16 || EC == EC_RES16;
     constexpr bool LOAD32 = EC == EC_RES32 || EC == EC_ACC32;
     constexpr int HB = 16;                 // rows per step
     constexpr int NHB = TM * 2;            // steps
@@ -386,8 +386,9 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
     const __amdgpu_buffer_rsrc_t rs_c = make_rsrc((const char*)epi.C + c_base * ESC, (uint32_t)(((M - 1) * epi.ldc + N) * ESC));
     const uint32_t off_c = col_ok ? (uint32_t)((row0 * epi.ldc + c8) * ESC) : OOB;
     const uint32_t step_c = (uint32_t)(epi.ldc * ESC);
-    const void* lp = EC == EC_RES32 ? epi.residual : (EC == EC_DACT16 ? epi.aux_in : (const void*)((const char*)epi.C + c_base * ESC));
-    const int64_t ld_l = EC == EC_RES32 ? epi.ld_res : (EC == EC_DACT16 ? epi.ld_aux_in : epi.ldc);
+    const void* lp = (EC == EC_RES32 || EC == EC_RES16) ? epi.residual
+                                                            : (EC == EC_DACT16 ? epi.aux_in : (const void*)((const char*)epi.C + c_base * ESC));
+    const int64_t ld_l = (EC == EC_RES32 || EC == EC_RES16) ? epi.ld_res : (EC == EC_DACT16 ? epi.ld_aux_in : epi.ldc);
     constexpr int ESL = LOAD32 ? 4 : 2;
     const __amdgpu_buffer_rsrc_t rs_l = make_rsrc(LOADS ? lp : epi.C, LOADS ? (uint32_t)(((M - 1) * ld_l + N) * ESL) : 0u);
     const uint32_t off_l = col_ok ? (uint32_t)((row0 * ld_l + c8) * ESL) : OOB;
@@ -464,7 +465,7 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
 #pragma unroll
           for (int k = 0; k < 8; ++k) v[k] = pf_gelu_erf(v[k]);
         }
-        if constexpr (EC == EC_DACT16 || EC == EC_ACC16) {
+        if constexpr (EC == EC_DACT16 || EC == EC_ACC16 || EC == EC_RES16) {
           const float8_t t = unpack16<DT>(ra);
           if constexpr (EC == EC_DACT16) {
 #pragma unroll
@@ -617,6 +618,7 @@ int launch16x(const pf_gemm_desc& d, hipStream_t st) {
       case EC_ACC32: return PF_X(false, false, EC_ACC32);
       case EC_DACT16: return PF_X(false, false, EC_DACT16);
       case EC_ACC16: return PF_X(false, false, EC_ACC16);
+      case EC_RES16: return PF_X(false, false, EC_RES16);
       default: return PF_X(false, false, EC_GENERIC);
     }
   }

@@ -122,6 +122,53 @@ def test_gemm_epilogues(hip, oracle, dtype):
     close(r["c"], rtol=1e-4, atol=2e-3)
 
 
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32"), (2, "256, 128, 64"), (3, "128, 128, 64"), (4, "192, 256, 32")])
+def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
+    """Every straight-line epilogue class of the direct-to-LDS kernel on every tile shape, ragged in M
+    (and in N against the 256- and 192-wide tiles), against the oracle; the launch names the class."""
+    M, N, K = 1000, 1160, 320
+    dt = {F16: 1, BF16: 2}[dtype]
+    x, w = rnd((M, K), dtype, 1), rnd((N, K), dtype, 2, 0.1)
+    bias = rnd((N,), dtype, 3)
+    rt, at = TOL[dtype]
+
+    def run(ec, tensors, outs, **kw):
+        print("gemm variant", variant, "class", ec, flush=True)
+        dev = {k: (None if v is None else v.cuda()) for k, v in tensors.items()}
+        cpu = {k: (None if v is None else v.clone()) for k, v in tensors.items()}
+        launch = hip.gemm(**dev, variant=variant, **kw)
+        assert launch.variant == "gemm16x_kernel<%d, %s, 2, 2, %d, false, false, %d>" % (
+            dt, tile, 3 if tile.endswith("64") else 5, ec), launch.variant
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        oracle.gemm(**cpu, **kw)()
+        return {o: (dev[o].cpu(), cpu[o]) for o in outs}
+
+    base = dict(M=M, N=N, K=K, lda=K, ldb=K, ldc=N)
+    z16 = lambda: torch.zeros(M, N, dtype=dtype)
+    r = run(0, dict(a=x, b=w, c=z16(), bias=bias), ["c"], round_mid=1, **base)
+    close(r["c"], rt, at)
+    r = run(1, dict(a=x, b=w, c=torch.zeros(M, N, dtype=F32), bias=bias), ["c"], **base)
+    close(r["c"], 1e-3, 1e-2)
+    r = run(2, dict(a=x, b=w, c=z16(), bias=bias, aux_out=z16()), ["c", "aux_out"], round_mid=1, act=1, ld_aux_out=N, **base)
+    close(r["c"], rt, at)
+    close(r["aux_out"], rt, at)
+    r = run(3, dict(a=x, b=w, c=torch.zeros(M, N, dtype=F32), bias=bias, residual=rnd((M, N), F32, 4)), ["c"],
+            round_mid=1, ld_res=N, **base)
+    close(r["c"], rt, at)
+    r = run(4, dict(a=x, b=w, c=rnd((M, N), F32, 5)), ["c"], beta=1, **base)
+    close(r["c"], 1e-3, 1e-2)
+    r = run(5, dict(a=x, b=w, c=z16(), aux_in=rnd((M, N), dtype, 6)), ["c"], dact=1, ld_aux_in=N, **base)
+    close(r["c"], rt, at * 4)
+    r = run(6, dict(a=x, b=w, c=rnd((M, N), dtype, 7)), ["c"], beta=1, **base)
+    close(r["c"], rt, at * 2)
+    # 16-bit residual stream (UNet transformer blocks under autocast): residual row stride wider than N
+    res16 = rnd((M, N + 8), dtype, 8)
+    r = run(7, dict(a=x, b=w, c=z16(), bias=bias, residual=res16), ["c"], round_mid=1, ld_res=N + 8, **base)
+    close(r["c"], rt, at * 2)
+
+
 def test_gemm_full_size_vit_l(hip, oracle):
     # qkv projection of ViT-L/16 at micro-batch 16: [3152 x 1024] . [1024 x 3072]
     M, N, K = 3152, 3072, 1024
@@ -355,6 +402,35 @@ def test_copy_strided_and_rope(hip, oracle, dtype):
     r = both(hip, oracle, "copy_strided", dict(src=src, dst=dst), ["dst"], src_strides=(21, 3, 1),
              dst_strides=(7, 1, 35), sizes=(5, 7, 3), accumulate=1)
     close(r["dst"], *TOL[dtype])
+    # batched transposes (tiled through LDS): NCHW -> NHWC and back, ragged extents, plain and accumulating
+    for (Bt, Ct, HW) in ((2, 70, 100), (3, 16, 33), (1, 128, 64)):
+        nchw = rnd((Bt, Ct, HW), dtype, 6)
+        nhwc = torch.zeros(Bt, HW, Ct, dtype=dtype)
+        r = both(hip, oracle, "copy_strided", dict(src=nchw, dst=nhwc), ["dst"], src_strides=(Ct * HW, 1, HW),
+                 dst_strides=(HW * Ct, Ct, 1), sizes=(Bt, HW, Ct))
+        assert torch.equal(r["dst"][0], r["dst"][1]) and torch.equal(r["dst"][0], nchw.permute(0, 2, 1).contiguous())
+        acc0 = rnd((Bt, Ct, HW), dtype, 7)
+        r = both(hip, oracle, "copy_strided", dict(src=r["dst"][0], dst=acc0), ["dst"], src_strides=(HW * Ct, 1, Ct),
+                 dst_strides=(Ct * HW, HW, 1), sizes=(Bt, Ct, HW), accumulate=1)
+        close(r["dst"], *TOL[dtype])
+        close((r["dst"][0], (acc0.float() + nchw.float()).to(dtype)), *TOL[dtype])
+    # four dimensions with the source-contiguous one in the middle: [B, H, T, D] -> [B, D, H, T]
+    x4 = rnd((2, 3, 40, 24), dtype, 8)
+    y4 = torch.zeros(2, 24, 3, 40, dtype=dtype)
+    r = both(hip, oracle, "copy_strided", dict(src=x4, dst=y4), ["dst"], src_strides=(3 * 40 * 24, 1, 40 * 24, 24),
+             dst_strides=(24 * 3 * 40, 3 * 40, 40, 1), sizes=(2, 24, 3, 40))
+    assert torch.equal(r["dst"][0], x4.permute(0, 3, 1, 2).contiguous())
+    # convolution weight [out, in, 9] -> [out, 9, in] (a short source-contiguous dimension) and its gradient back
+    wt = rnd((20, 70, 9), F32, 9)
+    w9 = torch.zeros(20, 9, 70, dtype=dtype)
+    r = both(hip, oracle, "copy_strided", dict(src=wt, dst=w9), ["dst"], src_strides=(630, 1, 9), dst_strides=(630, 70, 1),
+             sizes=(20, 9, 70))
+    assert torch.equal(r["dst"][0], r["dst"][1]) and torch.equal(r["dst"][0], wt.permute(0, 2, 1).to(dtype))
+    g9, gacc = rnd((20, 9, 70), F32, 10), rnd((20, 70, 9), F32, 11)
+    r = both(hip, oracle, "copy_strided", dict(src=g9, dst=gacc), ["dst"], src_strides=(630, 70, 1), dst_strides=(630, 1, 9),
+             sizes=(20, 9, 70), accumulate=1)
+    close(r["dst"], 1e-6, 1e-6)
+    close((r["dst"][0], gacc + g9.permute(0, 2, 1)), 1e-6, 1e-6)
     # rotary embedding on q inside a packed [B, T, 3, H, D] tensor, forward then inverse = identity
     Bq, T, H, D = 2, 33, 4, 64
     qkv = rnd((Bq, T, 3 * H * D), dtype, 4)
