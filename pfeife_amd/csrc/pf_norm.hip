@@ -663,12 +663,15 @@ int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, voi
   hipLaunchKernelGGL((norm_fwd_kernel<W, NV>), grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms)
 #define PF_NFC(NV, XD, YD) \
   hipLaunchKernelGGL((norm_fwd_kernel<8, NV, XD, YD>), grid, dim3(256), 0, st, x, x_dt, gamma, beta, y, y_dt, mean, rstd, rows, d, eps, rms)
-  // the residual stream is fp32 and the consumers are matrix products (16-bit) or fp32: those
-  // pairs get straight-line code
+  // the residual stream is fp32 and the consumers are matrix products (16-bit) or fp32, or the
+  // whole stream is 16-bit (a UNet's transformer blocks under autocast): those pairs get
+  // straight-line code
 #define PF_NFD(NV)                                                     \
   if (x_dt == PF_F32 && y_dt == PF_F16) PF_NFC(NV, PF_F32, PF_F16);     \
   else if (x_dt == PF_F32 && y_dt == PF_BF16) PF_NFC(NV, PF_F32, PF_BF16); \
   else if (x_dt == PF_F32 && y_dt == PF_F32) PF_NFC(NV, PF_F32, PF_F32); \
+  else if (x_dt == PF_F16 && y_dt == PF_F16) PF_NFC(NV, PF_F16, PF_F16); \
+  else if (x_dt == PF_BF16 && y_dt == PF_BF16) PF_NFC(NV, PF_BF16, PF_BF16); \
   else PF_NF(8, NV)
   if (v && d <= 64 * 8 * 1) { PF_NFD(1); }
   else if (v && d <= 64 * 8 * 2) { PF_NFD(2); }
@@ -706,14 +709,20 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
   // the residual stream and its gradient are fp32, the side copy 16-bit: straight-line variants
   // (the incoming gradient is the 16-bit result of a matrix product, or fp32)
   const bool io32 = x_dt == PF_F32 && dx_dt == PF_F32 && (!dx_add || add_dt == PF_F32);
-#define PF_NBC(NV, LP, DY)                                                                                           \
-  hipLaunchKernelGGL((norm_bwd_kernel<8, NV, PF_F32, LP, DY>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, \
+  // ... or everything is one 16-bit dtype and there is no side copy
+  const bool io16 = (x_dt == PF_F16 || x_dt == PF_BF16) && dx_dt == x_dt && dy_dt == x_dt && (!dx_add || add_dt == x_dt) &&
+                    !dx_lp;
+#define PF_NBC(NV, LP, DY) PF_NBI(NV, PF_F32, LP, DY)
+#define PF_NBI(NV, IO, LP, DY)                                                                                       \
+  hipLaunchKernelGGL((norm_bwd_kernel<8, NV, IO, LP, DY>), dim3(blocks), dim3(256), 0, st, dy, dy_dt, x, x_dt, gamma, \
                      mean, rstd, dx_add, add_dt, dx, dx_dt, ws, rows, d, rms, want, dx_lp, lp_dt, want_colsum)
 #define PF_NBD(NV)                                                                          \
   if (io32 && dy_dt == PF_F16 && (!dx_lp || lp_dt == PF_F16)) PF_NBC(NV, PF_F16, PF_F16);    \
   else if (io32 && dy_dt == PF_BF16 && (!dx_lp || lp_dt == PF_BF16)) PF_NBC(NV, PF_BF16, PF_BF16); \
   else if (io32 && dy_dt == PF_F32 && (!dx_lp || lp_dt == PF_F16)) PF_NBC(NV, PF_F16, PF_F32);    \
   else if (io32 && dy_dt == PF_F32 && lp_dt == PF_BF16) PF_NBC(NV, PF_BF16, PF_F32);         \
+  else if (io16 && x_dt == PF_F16) PF_NBI(NV, PF_F16, PF_F16, PF_F16);                       \
+  else if (io16 && x_dt == PF_BF16) PF_NBI(NV, PF_BF16, PF_BF16, PF_BF16);                   \
   else PF_NB(8, NV)
   if (v) {
     if (d <= 64 * 8 * 2) { PF_NBD(2); }
@@ -728,6 +737,7 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
   }
 #undef PF_NBD
 #undef PF_NBC
+#undef PF_NBI
 #undef PF_NB
   PF_CHECK_LAUNCH(name);
   if (want && !defer) {
