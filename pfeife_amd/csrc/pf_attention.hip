@@ -72,23 +72,23 @@ __device__ __forceinline__ uint4 load_row8(const uint16_t* base, int64_t st, int
   return make_uint4(0, 0, 0, 0);
 }
 
-// One [KT tokens][HD] tile in flight: NV 16-byte vectors per thread, loaded from global into
+// One [ROWS tokens][HD] tile in flight: NV 16-byte vectors per thread, loaded from global into
 // registers while the previous tile is being multiplied, stored to LDS ([KT][HD + 8]) afterwards.
-template <int HD> struct Tile {
-  static constexpr int LD = HD + 8, VPR = HD / 8, NV = (KT * VPR + 255) / 256;
+template <int HD, int ROWS = KT> struct Tile {
+  static constexpr int LD = HD + 8, VPR = HD / 8, NV = (ROWS * VPR + 255) / 256;
   uint4 v[NV];
   __device__ __forceinline__ void load(const uint16_t* base, int64_t st, int t0, int T, int hd, int tid) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int e = tid + i * 256;
-      v[i] = (e < KT * VPR) ? load_row8(base, st, t0 + e / VPR, T, (e % VPR) * 8, hd) : make_uint4(0, 0, 0, 0);
+      v[i] = (e < ROWS * VPR) ? load_row8(base, st, t0 + e / VPR, T, (e % VPR) * 8, hd) : make_uint4(0, 0, 0, 0);
     }
   }
   __device__ __forceinline__ void store(uint16_t* s, int tid) const {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int e = tid + i * 256;
-      if (e < KT * VPR) *(uint4*)(s + (e / VPR) * LD + (e % VPR) * 8) = v[i];
+      if (e < ROWS * VPR) *(uint4*)(s + (e / VPR) * LD + (e % VPR) * 8) = v[i];
     }
   }
 };
@@ -397,17 +397,25 @@ __global__ __launch_bounds__(256, HD <= 64 ? 2 : 1) void attn_dq_kernel(const At
 // dK/dV: column = key row; S[q][kv] = Q K^T, dV^T[hd][kv] += dO^T[hd][q] P[q][kv],
 //        dK^T[hd][kv] += Q^T[hd][q] dS[q][kv]
 // ---------------------------------------------------------------------------------
-template <int DT, int HD>
-__global__ __launch_bounds__(256, 2) void attn_dkv_kernel(const AttnArgs a) {
+// SPLITQ (few keys, many queries: cross attention to a short context): a workgroup owns ONE 32-key
+// tile, its four wavefronts each take a quarter of every staged block of 128 queries, and their
+// accumulators are added at the end through LDS in wavefront order, so that a head's dK/dV come
+// from 4 x ceil(Tk / 32) wavefronts instead of ceil(Tk / 32).
+template <int DT, int HD, bool SPLITQ = false>
+__global__ __launch_bounds__(256, SPLITQ ? 1 : 2) void attn_dkv_kernel(const AttnArgs a) {
   constexpr int NC = HD / 16, NO = HD / 32, QLD = HD + 8;
-  __shared__ __align__(16) uint16_t sQ[KT * QLD];
-  __shared__ __align__(16) uint16_t sDO[KT * QLD];
-  __shared__ float sLse[KT], sDelta[KT];
+  constexpr int QT = SPLITQ ? 128 : KT;        // queries staged per iteration
+  constexpr int NH = SPLITQ ? 1 : 2;           // 32-query halves per wavefront and iteration
+  __shared__ __align__(16) uint16_t sQD[2 * QT * QLD];
+  uint16_t* sQ = sQD;
+  uint16_t* sDO = sQD + QT * QLD;
+  __shared__ float sLse[QT], sDelta[QT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int kb, bh;
   attn_block(a, false, kb, bh);
   const int b = bh / a.H, h = bh % a.H;
-  const int kw0 = kb * 128 + wave * 32;                        // this wavefront's first key row
+  const int kw0 = SPLITQ ? kb * 32 : kb * 128 + wave * 32;     // this wavefront's first key row
+  const int qoff = SPLITQ ? wave * 32 : 0;                     // its first query row inside a staged block
   const int kj = kw0 + (lane & 31);                            // this lane's key row
   const uint16_t* Q = a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t* K = a.k + b * a.k_sb + h * a.k_sh;
@@ -431,15 +439,15 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(const AttnArgs a) {
 
   int q_begin = 0;
   if (a.causal) {  // queries i with i + shift >= first key of the block see it
-    q_begin = max(0, kb * 128 - shift);
-    q_begin = q_begin / KT * KT;
+    q_begin = max(0, (SPLITQ ? kb * 32 : kb * 128) - shift);
+    q_begin = q_begin / QT * QT;
   }
-  Tile<HD> tq, tdo;
+  Tile<HD, QT> tq, tdo;
   float r_lse = 0.f, r_dlt = 0.f;
   auto prefetch = [&](int q0) {
     tq.load(Q, a.q_st, q0, a.Tq, a.hd, tid);
     tdo.load(DO, a.do_st, q0, a.Tq, a.hd, tid);
-    if (tid < KT) {
+    if (tid < QT) {
       const int qi = q0 + tid;
       // rows past the end: Q and dO rows are zero, lse = +inf makes their P exactly zero
       r_lse = qi < a.Tq ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
@@ -447,32 +455,32 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(const AttnArgs a) {
     }
   };
   if (q_begin < a.Tq) prefetch(q_begin);
-  for (int q0 = q_begin; q0 < a.Tq; q0 += KT) {
+  for (int q0 = q_begin; q0 < a.Tq; q0 += QT) {
     __syncthreads();
     tq.store(sQ, tid);
     tdo.store(sDO, tid);
-    if (tid < KT) {
+    if (tid < QT) {
       sLse[tid] = r_lse;
       sDelta[tid] = r_dlt;
     }
-    if (q0 + KT < a.Tq) prefetch(q0 + KT);
+    if (q0 + QT < a.Tq) prefetch(q0 + QT);
     __syncthreads();
     // causal: the tile needs element masks only where it crosses the diagonal
-    const bool masked = a.causal && (kw0 + 31 > q0 + shift);
-    float16_t s[2], dp[2];
+    const bool masked = a.causal && (kw0 + 31 > q0 + qoff + shift);
+    float16_t s[NH], dp[NH];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int t = 0; t < NH; ++t) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[t][r] = dp[t][r] = 0.f;
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
-        const int off = (t * 32 + (lane & 31)) * QLD + c * 16 + (lane >> 5) * 8;
+        const int off = (qoff + t * 32 + (lane & 31)) * QLD + c * 16 + (lane >> 5) * 8;
         s[t] = M32<DT>::run(*(const uint4*)(sQ + off), kf[c], s[t]);
         dp[t] = M32<DT>::run(*(const uint4*)(sDO + off), vf[c], dp[t]);
       }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int ql = t * 32 + acc_row(r, lane);
+        const int ql = qoff + t * 32 + acc_row(r, lane);
         float p = __builtin_amdgcn_exp2f(s[t][r] * sc - sLse[ql]);
         if (masked && kj > q0 + ql + shift) p = 0.f;
         s[t][r] = p;                                         // P
@@ -480,15 +488,44 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(const AttnArgs a) {
       }
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 2 * NH; ++j) {
       const uint4 pf = pack8<DT>(s[j >> 1], 8 * (j & 1));
       const uint4 dsf = pack8<DT>(dp[j >> 1], 8 * (j & 1));
 #pragma unroll
       for (int o = 0; o < NO; ++o) {
-        dv[o] = M32<DT>::run(frag_tr<QLD>(sDO, 16 * j, o * 32, lane), pf, dv[o]);
-        dk[o] = M32<DT>::run(frag_tr<QLD>(sQ, 16 * j, o * 32, lane), dsf, dk[o]);
+        dv[o] = M32<DT>::run(frag_tr<QLD>(sDO, qoff + 16 * j, o * 32, lane), pf, dv[o]);
+        dk[o] = M32<DT>::run(frag_tr<QLD>(sQ, qoff + 16 * j, o * 32, lane), dsf, dk[o]);
       }
     }
+  }
+  if constexpr (SPLITQ) {
+    // wavefront 0 adds the other three's accumulators in wavefront order: dV, then dK
+    float* red = (float*)sQD;
+    static_assert(3 * NO * 16 * 64 * 4 <= 2 * QT * QLD * 2, "reduction patch exceeds the operand tiles");
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      __syncthreads();   // the tiles (or the previous pass's patch) are no longer read
+      if (wave > 0) {
+#pragma unroll
+        for (int o = 0; o < NO; ++o)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            red[(((wave - 1) * NO + o) * 16 + r) * 64 + lane] = pass == 0 ? dv[o][r] : dk[o][r];
+      }
+      __syncthreads();
+      if (wave == 0) {
+#pragma unroll
+        for (int w = 0; w < 3; ++w)
+#pragma unroll
+          for (int o = 0; o < NO; ++o)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const float x = red[((w * NO + o) * 16 + r) * 64 + lane];
+              if (pass == 0) dv[o][r] += x; else dk[o][r] += x;
+            }
+      }
+    }
+    if (wave != 0) return;
   }
   if (kok) {
     uint16_t* DK = a.dk + b * a.dk_sb + h * a.dk_sh + (int64_t)kj * a.dk_st;
@@ -1010,7 +1047,20 @@ extern "C" int pf_attention_bwd(const pf_attn_desc* d, void* stream) {
   }
   const int64_t rows = (int64_t)d->B * d->H * d->Tq;
   hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, ad, d->delta);
-  PF_ATTN_DISPATCH(attn_dkv_kernel, gk, st, a, d->dtype, d->hd);
+  // few keys, many queries (cross attention to a short context): split each key tile's query sweep
+  // over the four wavefronts of a workgroup
+  if ((int64_t)gk.x * gk.y < 200 && d->Tq >= 256) {
+    const dim3 gs((unsigned)((d->Tk + 31) / 32), (unsigned)(d->B * d->H));
+    if (d->dtype == PF_F16) {
+      if (d->hd <= 64) hipLaunchKernelGGL((attn_dkv_kernel<PF_F16, 64, true>), gs, dim3(256), 0, st, a);
+      else hipLaunchKernelGGL((attn_dkv_kernel<PF_F16, 96, true>), gs, dim3(256), 0, st, a);
+    } else {
+      if (d->hd <= 64) hipLaunchKernelGGL((attn_dkv_kernel<PF_BF16, 64, true>), gs, dim3(256), 0, st, a);
+      else hipLaunchKernelGGL((attn_dkv_kernel<PF_BF16, 96, true>), gs, dim3(256), 0, st, a);
+    }
+  } else {
+    PF_ATTN_DISPATCH(attn_dkv_kernel, gk, st, a, d->dtype, d->hd);
+  }
   PF_ATTN_DISPATCH(attn_dq_kernel, gq, st, a, d->dtype, d->hd);
   PF_CHECK_LAUNCH("pf_attention_bwd");
   return PF_OK;

@@ -567,6 +567,8 @@ def test_deferred_reductions_match_immediate(hip):
     dict(B=1, H=3, Tq=200, Tk=40, hd=88, causal=0, packed=False),    # short, several query blocks, few keys
     dict(B=1, H=2, Tq=320, Tk=290, hd=64, causal=0, packed=False),   # beyond the whole-head-in-LDS kernels
     dict(B=2, H=2, Tq=280, Tk=280, hd=64, causal=1, packed=False),   # ninth tile: second pass of the first wavefront
+    dict(B=2, H=2, Tq=600, Tk=77, hd=64, causal=0, packed=False),    # cross attention from many queries: split-query dK/dV
+    dict(B=1, H=2, Tq=330, Tk=40, hd=88, causal=0, packed=False),    # the same at head dim 88, ragged query blocks
     dict(B=1, H=2, Tq=160, Tk=170, hd=96, causal=0, packed=False),   # head dim 96: six key tiles in one 4-wavefront workgroup
 ])
 def test_fused_attention(hip, oracle, dtype, case):
