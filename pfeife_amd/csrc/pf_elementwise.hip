@@ -255,6 +255,56 @@ __global__ __launch_bounds__(256) void copy_transpose_kernel(const void* src, in
   }
 }
 
+// The same when one of the two dimensions is short (a 3x3 convolution's 9 taps) and the block of
+// (long, short) elements is contiguous on the side where the short dimension is the contiguous one:
+// that side is streamed linearly, 256 x n elements per workgroup, the other side in runs of 256.
+//   SRC_NARROW: source element (l, j) at l * nj + j (nj <= 32), destination at j * d_j + l
+//   else:       source at l * s_l + j, destination element (j, l) at j * nl + l (nl <= 32)
+template <bool SRC_NARROW>
+__global__ __launch_bounds__(256) void copy_transpose_narrow_kernel(const void* src, int sdt, void* dst, int ddt,
+                                                                    TransposeDesc td, int accumulate) {
+  __shared__ float buf[256 * 33];
+  const int t = threadIdx.x;
+  int64_t rem = blockIdx.z, so = 0, dof = 0;
+#pragma unroll
+  for (int k = 3; k >= 0; --k) {
+    if (k < td.nb) {
+      const int64_t idx = rem % td.bsize[k];
+      rem /= td.bsize[k];
+      so += idx * td.bss[k];
+      dof += idx * td.bds[k];
+    }
+  }
+  if (SRC_NARROW) {
+    const int n = (int)td.nj, np = n | 1;
+    const int64_t l0 = (int64_t)blockIdx.x * 256;
+    const int cnt = (int)((td.nl - l0 < 256 ? td.nl - l0 : 256) * n);
+    for (int i = t; i < cnt; i += 256) buf[(i / n) * np + (i % n)] = pf_load_as_f32(src, so + l0 * n + i, sdt);
+    __syncthreads();
+    if (l0 + t < td.nl) {
+      for (int j = 0; j < n; ++j) {
+        const int64_t o = dof + j * td.d_j + l0 + t;
+        float v = buf[t * np + j];
+        if (accumulate) v += pf_load_as_f32(dst, o, ddt);
+        pf_store_from_f32(dst, o, ddt, v);
+      }
+    }
+  } else {
+    const int n = (int)td.nl, np = n | 1;
+    const int64_t j0 = (int64_t)blockIdx.x * 256;
+    if (j0 + t < td.nj)
+      for (int l = 0; l < n; ++l) buf[t * np + l] = pf_load_as_f32(src, so + l * td.s_l + j0 + t, sdt);
+    __syncthreads();
+    const int cnt = (int)((td.nj - j0 < 256 ? td.nj - j0 : 256) * n);
+    for (int i = t; i < cnt; i += 256) {
+      const int64_t o = dof + j0 * n + i;
+      float v = buf[(i / n) * np + (i % n)];
+      if (accumulate) v += pf_load_as_f32(dst, o, ddt);
+      pf_store_from_f32(dst, o, ddt, v);
+    }
+  }
+}
+
 // dst[c, r] = src[r, c] with dtype conversion, 64x64 tiles through LDS so that both
 // the reads and the writes are contiguous runs of 64 elements
 __global__ __launch_bounds__(256) void transpose_cast_kernel(const void* src, int sdt, int64_t ld_src, void* dst,
@@ -642,6 +692,18 @@ extern "C" int pf_copy_strided(const void* src, int src_dtype, const int64_t* sr
       }
       for (int k = td.nb; k < 4; ++k) { td.bsize[k] = 1; td.bss[k] = 0; td.bds[k] = 0; }
       const int64_t gx = (td.nj + 63) / 64, gy = (td.nl + 63) / 64;
+      if (batch <= 65535 && td.nj <= 32 && td.s_l == td.nj) {
+        hipLaunchKernelGGL(copy_transpose_narrow_kernel<true>, dim3((unsigned)((td.nl + 255) / 256), 1, (unsigned)batch),
+                           dim3(256), 0, st, src, src_dtype, dst, dst_dtype, td, accumulate);
+        PF_CHECK_LAUNCH("pf_copy_strided");
+        return PF_OK;
+      }
+      if (batch <= 65535 && td.nl <= 32 && td.d_j == td.nl) {
+        hipLaunchKernelGGL(copy_transpose_narrow_kernel<false>, dim3((unsigned)((td.nj + 255) / 256), 1, (unsigned)batch),
+                           dim3(256), 0, st, src, src_dtype, dst, dst_dtype, td, accumulate);
+        PF_CHECK_LAUNCH("pf_copy_strided");
+        return PF_OK;
+      }
       if (batch <= 65535 && gy <= 65535) {
         hipLaunchKernelGGL(copy_transpose_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)batch), dim3(256), 0, st, src,
                            src_dtype, dst, dst_dtype, td, accumulate);
