@@ -755,7 +755,7 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
 // matrix: the norm backward writes 2 partial rows per workgroup, the column sum
 // one partial row per row chunk.
 // One launch finishing many deferred column reductions: block (x, y) handles 128 columns of
-// item y (four per lane, 16-byte loads, four partial rows in flight per lane) when the item's
+// item y (four per lane, 16-byte loads, up to eight partial rows in flight per lane) when the item's
 // rows are 16-byte aligned, else 32 columns.  Items live in device memory.  Per column the partial
 // rows are summed in a fixed order: rows part, part + 8, ... by group `part`, then the eight groups.
 __global__ __launch_bounds__(256) void colreduce_finalize_batch_kernel(const pf_reduce_item* items) {
@@ -769,6 +769,13 @@ __global__ __launch_bounds__(256) void colreduce_finalize_batch_kernel(const pf_
     float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     if (c < it.cols) {
       int p = part;
+      for (; p + 56 < it.n_partials; p += 64) {   // eight partial rows in flight, added in row order
+        float4 a[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a[u] = *(const float4*)(it.ws + (int64_t)(p + 8 * u) * it.stride + c);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) { s.x += a[u].x; s.y += a[u].y; s.z += a[u].z; s.w += a[u].w; }
+      }
       for (; p + 24 < it.n_partials; p += 32) {
         const float4 a0 = *(const float4*)(it.ws + (int64_t)p * it.stride + c);
         const float4 a1 = *(const float4*)(it.ws + (int64_t)(p + 8) * it.stride + c);
