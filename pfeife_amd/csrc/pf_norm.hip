@@ -675,6 +675,7 @@ int norm_fwd(const void* x, int x_dt, const float* gamma, const float* beta, voi
   else PF_NF(8, NV)
   if (v && d <= 64 * 8 * 1) { PF_NFD(1); }
   else if (v && d <= 64 * 8 * 2) { PF_NFD(2); }
+  else if (v && d <= 64 * 8 * 3) { PF_NFD(3); }
   else if (v && d <= 64 * 8 * 4) { PF_NFD(4); }
   else if (v) PF_NF(8, 0);
   else PF_NF(1, 0);
@@ -726,6 +727,7 @@ int norm_bwd(const void* dy, int dy_dt, const void* x, int x_dt, const float* ga
   else PF_NB(8, NV)
   if (v) {
     if (d <= 64 * 8 * 2) { PF_NBD(2); }
+    else if (d <= 64 * 8 * 3) { PF_NBD(3); }
     else if (d <= 64 * 8 * 4) { PF_NBD(4); }
     else if (d <= 64 * 8 * 8) PF_NB(8, 8);
     else if (d <= 64 * 8 * 16) PF_NB(8, 16);

@@ -187,7 +187,7 @@ def test_gemm_rejects_bad_arguments(hip):
 
 
 @pytest.mark.parametrize("xdt,ydt", [(F32, F16), (F32, BF16), (F32, F32), (F16, F16), (BF16, BF16)])
-@pytest.mark.parametrize("rows,d", [(37, 1024), (5, 1408), (9, 100), (3, 2048)])
+@pytest.mark.parametrize("rows,d", [(37, 1024), (5, 1408), (21, 1280), (9, 100), (3, 2048)])
 def test_layernorm_rmsnorm(hip, oracle, xdt, ydt, rows, d):
     x = rnd((rows, d), xdt, 1) + 0.5
     gamma, beta = rnd((d,), F32, 2) + 1, rnd((d,), F32, 3)
