@@ -337,12 +337,29 @@ def torch_eager_gpu(name, device, steps=5, warmup=2):
 
     from pfeife_amd.bench_models import llama, vit
 
+    from pfeife_amd.bench_models import unet_stage
+
     family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
-    if family not in ("vit", "llama"):
+    if family not in ("vit", "llama", "unet"):
         return None
     torch.manual_seed(42)
     g = torch.Generator().manual_seed(42)
-    if family == "vit":
+    if family == "unet":
+        cfg = getattr(unet_stage, cfg_name)
+        model = unet_stage.UNetStage(cfg).to(device)
+        x = torch.randn(batch, cfg.in_channels, 32, 32, generator=g).to(device)
+        temb = torch.randn(batch, cfg.temb_dim, generator=g).to(device)
+        ctx = torch.randn(batch, 77, cfg.context_dim, generator=g).to(device)
+        y = torch.randn(batch, cfg.channels, 32, 32, generator=g).to(device)
+        per = batch // batch_cnt
+        state = {"i": 0}
+
+        def loss_of(xb, yb):
+            i = state["i"] % batch_cnt
+            state["i"] += 1
+            sl = slice(i * per, (i + 1) * per)
+            return F.mse_loss(model(xb, temb[sl], ctx[sl]).float(), yb.float())
+    elif family == "vit":
         cfg = getattr(vit, cfg_name)
         model = vit.VisionTransformer(cfg).to(device)
         x = torch.randn(batch, cfg.channels, cfg.image_size, cfg.image_size, generator=g).to(device)
@@ -373,15 +390,18 @@ def torch_eager_gpu(name, device, steps=5, warmup=2):
         scaler.update()
         return loss
 
+    trace = []
     for _ in range(warmup):
-        step()
+        trace.append(step())
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         loss = step()
+        trace.append(loss)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     last = float(loss)
+    log("[bench] torch eager: last micro-batch loss per step", [round(float(l), 4) for l in trace])
     del opt, model
     torch.cuda.empty_cache()
     return dict(value=round(batch * steps / dt, 2), unit="samples/s", ms_per_step=round(1e3 * dt / steps, 3), steps=steps,

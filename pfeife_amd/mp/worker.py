@@ -416,9 +416,14 @@ class StageWorker:
             raise RuntimeError("loss gradient of output %d has shape %s, expected %s"
                                % (out_idx, tuple(g.shape), tuple(buf.shape)))
         if self.dyn_scale:
-            if not (g.device == buf.device and g.dtype.is_floating_point):
-                g = g.to(device=buf.device, dtype=buf.dtype)
-            self.kernels.scale_by_state(g.contiguous(), self.scaler_state, buf, g.numel())(self.stream())
+            if g.device == buf.device and g.dtype.is_floating_point and g.is_contiguous() and buf.is_contiguous():
+                self.kernels.scale_by_state(g, self.scaler_state, buf, g.numel())(self.stream())
+            else:
+                # the kernel walks both operands as flat arrays: anything with strides of its own (an output
+                # kept channels-last in memory, a permuted gradient) goes through a stride-aware copy first;
+                # the scale stays on the device (a 0-dim view of the scaler state, no host read)
+                buf.copy_(g)
+                buf.mul_(self.scaler_state[0])
             return
         scale = self.option.loss_scale
         if g.device == buf.device and g.is_contiguous() and buf.is_contiguous() and g.dtype.is_floating_point:

@@ -483,6 +483,69 @@ def test_unet_stage_sdxl_style(mixed):
     _check_grads(model, ref, mixed)
 
 
+def test_unet_stage_dynamic_loss_scale_with_a_tensor_valued_loss_gradient():
+    """Dynamic loss scaling when user code computes the loss with ATen and the stage output it
+    differentiates is a tensor kept channels-last in memory: the incoming gradient has to be scaled
+    element for element (not as a flat array) before it enters the last stage.  Three Adam steps
+    against torch.amp.GradScaler + torch.optim.Adam on an eager copy: the losses must fall alike."""
+    import torch.nn.functional as F
+
+    from pfeife_amd.bench_models.unet_stage import UNetStage, UNetStageConfig
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = UNetStageConfig(in_channels=128, channels=256, temb_dim=256, context_dim=512, heads=4, layers=2, groups=32)
+    torch.manual_seed(0)
+    model = UNetStage(cfg)
+    ref = copy.deepcopy(model).cuda()
+    p0 = {n: p.detach().clone() for n, p in ref.named_parameters()}
+    g = torch.Generator().manual_seed(42)
+    B, hw = 4, 16
+    hidden = torch.randn(B, cfg.in_channels, hw, hw, generator=g).cuda()
+    temb = torch.randn(B, cfg.temb_dim, generator=g).cuda()
+    ctx = torch.randn(B, 77, cfg.context_dim, generator=g).cuda()
+    target = torch.randn(B, cfg.channels, hw, hw, generator=g).cuda()
+    option = PipeOption(device_cnt=1, batch_cnt=1, batch_size=B, mixed_precision="fp16",
+                        optimizer=dict(type="adam", lr=1e-4), loss_scale="dynamic", init_scale=4096.0)
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(h, t, c, y):
+        out = cmodel(h, t, c)
+        loss = F.mse_loss(out.float(), y.float())
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    got = [float(runner.step(hidden, temb, ctx, target)[0]) for _ in range(4)]
+    torch.cuda.synchronize()
+    assert runner.worker.scaler_scale() == 4096.0      # no step overflowed
+    opt = torch.optim.Adam(ref.parameters(), lr=1e-4)
+    scaler = torch.amp.GradScaler("cuda", init_scale=4096.0)
+    want = []
+    for _ in range(4):
+        opt.zero_grad(set_to_none=False)
+        with torch.autocast("cuda", dtype=torch.float16):
+            out = ref(hidden, temb, ctx)
+        loss = F.mse_loss(out.float(), target.float())
+        scaler.scale(loss).backward()
+        scaler.step(opt)
+        scaler.update()
+        want.append(float(loss.detach()))
+    assert want[-1] < 0.97 * want[0]                    # the reference run does train
+    for a, b in zip(got, want):
+        assert abs(a - b) <= 2e-2 * abs(b), (got, want)
+    # the parameters have moved the same way (Adam: about lr per step and element, by the gradient's sign)
+    worst = 0.0
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        d1, d2 = (p.detach() - p0[n]).flatten(), (q.detach() - p0[n]).flatten()
+        firm = d2.abs() > 2e-4                           # elements that moved the same way in most steps
+        if int(firm.sum()) >= 16:
+            worst = max(worst, float(((torch.sign(d1) != torch.sign(d2)) & firm).sum()) / float(firm.sum()))
+    assert worst <= 0.05, worst
+
+
 @pytest.mark.parametrize("opt_type,wd", [("adam", 0.0), ("adam", 0.01), ("adamw", 0.05)])
 def test_fused_adam_matches_torch_optimizer(opt_type, wd):
     """Three training steps with the fused multi-tensor Adam launch against the same steps
