@@ -164,6 +164,216 @@ def test_vit_l_width_fp16_headline_geometry():
         assert w in names, (w, sorted(names))
 
 
+def test_vit_l16_headline_config_trains_like_pytorch():
+    """The headline configuration itself (ViT-L/16, 24 blocks, fp16 autocast, micro-batch 16 x 4, two
+    stages split at block 12, dynamic loss scaling, fused Adam at lr 1e-5, four streams): six
+    optimisation steps against the same steps in plain PyTorch on this GPU (autocast, GradScaler,
+    torch.optim.Adam, gradient accumulation over the four micro-batches).  The loss falls from 7.1 to
+    3.1 in six steps; every step's last micro-batch loss must agree within 1 %."""
+    import torch.nn.functional as F
+
+    from pfeife_amd.bench_models import vit
+    from pfeife_amd.loss import CrossEntropyLoss
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = vit.VIT_L16
+    torch.manual_seed(42)
+    g = torch.Generator().manual_seed(42)
+    model = vit.VisionTransformer(cfg)
+    ref = copy.deepcopy(model).cuda()
+    x = torch.randn(64, cfg.channels, cfg.image_size, cfg.image_size, generator=g).cuda()
+    y = torch.randint(0, cfg.num_classes, (64,), generator=g).cuda()
+    option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=16, split_points=["blocks.12"], mixed_precision="fp16",
+                        optimizer=dict(type="adam", lr=1e-5))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = CrossEntropyLoss(cfg.num_classes)
+
+    def fn(px, labels):
+        loss = crit(cmodel(px), labels)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    got, applied = [], []
+    w = None
+    for _ in range(8):
+        losses = runner.step(x, y)
+        w = runner.worker
+        got.append(float(losses[-1]))
+        applied.append(float(w.scaler_state[3]))
+    torch.cuda.synchronize()
+    assert w.dyn_scale and w.lanes is not None and len(w.lanes) == 4
+    # a step whose gradients overflowed at the initial scale is skipped (same loss again): drop those
+    kept = [got[i] for i in range(len(got)) if i == 0 or applied[i - 1] > (applied[i - 2] if i > 1 else 0.0)][:6]
+    opt = torch.optim.Adam(ref.parameters(), lr=1e-5)
+    scaler = torch.amp.GradScaler("cuda")
+    want = []
+    for _ in range(6):
+        opt.zero_grad(set_to_none=False)
+        for xb, yb in zip(x.chunk(4), y.chunk(4)):
+            with torch.autocast("cuda", dtype=torch.float16):
+                loss = F.cross_entropy(ref(xb).float(), yb)
+            scaler.scale(loss).backward()
+        scaler.step(opt)
+        scaler.update()
+        want.append(float(loss.detach()))
+    assert want[-1] < 0.5 * want[0]
+    assert len(kept) == 6, (got, applied)
+    for a, b in zip(kept, want):
+        assert abs(a - b) <= 1e-2 * abs(b), (kept, want)
+
+
+def test_llama_1b_config_trains_like_pytorch():
+    """The decoder configuration at its own size (16 layers, hidden 2048, 32 heads, SwiGLU 5632, vocabulary
+    32000, 2048 tokens, bf16 autocast, micro-batch 2 x 8, four stages looped over two ranks, fused Adam):
+    four optimisation steps against the same steps in plain PyTorch on this GPU; every step's last
+    micro-batch loss must agree within 0.5 %."""
+    from pfeife_amd.bench_models import llama
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = llama.LLAMA_1B
+    torch.manual_seed(42)
+    g = torch.Generator().manual_seed(42)
+    model = llama.LlamaForCausalLM(cfg)
+    ref = copy.deepcopy(model).cuda()
+    ids = torch.randint(0, cfg.vocab, (16, cfg.max_seq), generator=g).cuda()
+    option = PipeOption(device_cnt=2, batch_cnt=8, batch_size=2, split_points=["layers.4", "layers.8", "layers.12"],
+                        mixed_precision="bf16", optimizer=dict(type="adam", lr=1e-5))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(tok):
+        loss = cmodel(tok, tok)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    got = [float(runner.step(ids)[-1]) for _ in range(4)]
+    torch.cuda.synchronize()
+    assert len(runner.worker.part_graph.nodes) == 4
+    opt = torch.optim.Adam(ref.parameters(), lr=1e-5)
+    want = []
+    for _ in range(4):
+        opt.zero_grad(set_to_none=False)
+        for tok in ids.chunk(8):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                loss = ref(tok, tok)
+            loss.backward()
+        opt.step()
+        want.append(float(loss.detach()))
+    assert want[-1] < want[0] - 0.1
+    for a, b in zip(got, want):
+        assert abs(a - b) <= 5e-3 * abs(b), (got, want)
+
+
+def test_unet_stage_config_trains_like_pytorch():
+    """The UNet stage at its own size (1280 channels at 32x32, 30 transformer blocks, cross attention to 77
+    tokens, fp16 autocast, batch 4, dynamic loss scaling, MSE in user code, fused Adam): five applied
+    optimisation steps against the same steps in plain PyTorch on this GPU; losses within 1 %."""
+    import torch.nn.functional as F
+
+    from pfeife_amd.bench_models import unet_stage
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = unet_stage.SDXL_STAGE
+    torch.manual_seed(42)
+    g = torch.Generator().manual_seed(42)
+    model = unet_stage.UNetStage(cfg)
+    ref = copy.deepcopy(model).cuda()
+    hidden = torch.randn(4, cfg.in_channels, 32, 32, generator=g).cuda()
+    temb = torch.randn(4, cfg.temb_dim, generator=g).cuda()
+    ctx = torch.randn(4, 77, cfg.context_dim, generator=g).cuda()
+    target = torch.randn(4, cfg.channels, 32, 32, generator=g).cuda()
+    option = PipeOption(device_cnt=1, batch_cnt=1, batch_size=4, mixed_precision="fp16", optimizer=dict(type="adam", lr=1e-5))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(h, t, c, y):
+        loss = F.mse_loss(cmodel(h, t, c).float(), y.float())
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    got, applied = [], []
+    for _ in range(8):
+        got.append(float(runner.step(hidden, temb, ctx, target)[0]))
+        applied.append(float(runner.worker.scaler_state[3]))
+    torch.cuda.synchronize()
+    kept = [got[i] for i in range(len(got)) if i == 0 or applied[i - 1] > (applied[i - 2] if i > 1 else 0.0)][:5]
+    opt = torch.optim.Adam(ref.parameters(), lr=1e-5)
+    scaler = torch.amp.GradScaler("cuda")
+    want = []
+    for _ in range(5):
+        opt.zero_grad(set_to_none=False)
+        with torch.autocast("cuda", dtype=torch.float16):
+            out = ref(hidden, temb, ctx)
+        loss = F.mse_loss(out.float(), target.float())
+        scaler.scale(loss).backward()
+        scaler.step(opt)
+        scaler.update()
+        want.append(float(loss.detach()))
+    assert want[-1] < 0.8 * want[0]
+    assert len(kept) == 5, (got, applied)
+    for a, b in zip(kept, want):
+        assert abs(a - b) <= 1e-2 * abs(b), (kept, want)
+
+
+def test_vit_g14_share_config_trains_like_pytorch():
+    """One GPU's share of ViT-g/14 at its own size (10 blocks, hidden 1408, 16 heads of 88, MLP 6144, 257
+    tokens, bf16 autocast, micro-batch 24 x 4, the gradient of the share's output supplied from outside,
+    fused Adam): four optimisation steps against the same steps in plain PyTorch on this GPU.  What is
+    compared is the share's output itself (64 elements of each micro-batch), which moves as the weights do."""
+    from pfeife_amd.bench_models import vit
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = vit.VIT_G14_SHARE
+    torch.manual_seed(42)
+    g = torch.Generator().manual_seed(42)
+    model = vit.BlockStack(cfg)
+    ref = copy.deepcopy(model).cuda()
+    act = torch.randn(96, cfg.tokens, cfg.dim, generator=g).cuda()
+    grad_out = (torch.randn(96, cfg.tokens, cfg.dim, generator=g) * 1e-2).cuda()
+    option = PipeOption(device_cnt=1, batch_cnt=4, batch_size=24, mixed_precision="bf16", optimizer=dict(type="adam", lr=1e-5))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(a, go):
+        out = cmodel(a)
+        out.backward(go.to(out.dtype))
+        return out.detach()[0, 0, :64].float().clone()
+
+    runner.set_exec_fn(fn)
+    got = [torch.stack(runner.step(act, grad_out)).cpu() for _ in range(4)]
+    torch.cuda.synchronize()
+    opt = torch.optim.Adam(ref.parameters(), lr=1e-5)
+    want = []
+    for _ in range(4):
+        opt.zero_grad(set_to_none=False)
+        outs = []
+        for a, go in zip(act.chunk(4), grad_out.chunk(4)):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                out = ref(a)
+            out.backward(go.to(out.dtype))
+            outs.append(out.detach()[0, 0, :64].float().clone())
+        opt.step()
+        want.append(torch.stack(outs).cpu())
+    drift = (want[-1] - want[0]).abs().mean().item()
+    assert drift > 0.02                                   # the outputs do move over the four steps
+    for a, b in zip(got, want):
+        torch.testing.assert_close(a, b, rtol=3e-2, atol=3e-2)
+    # and they move the same way
+    assert ((got[-1] - got[0]) - (want[-1] - want[0])).abs().mean().item() <= 0.35 * drift
+
+
 def test_ragged_batch_on_device():
     """N % batch_cnt != 0: torch.tensor_split gives micro-batches of 3, 3, 2, 2 samples
     (pfeife/batch.py:45); every one gets its own stage programs."""
