@@ -344,7 +344,7 @@ class StageWorker:
         buf = slot.input_buffers.get(placeholder_idx)
         if buf is None:
             return
-        if value.device == buf.device and value.is_contiguous() and value.numel() > 0:
+        if value.device == buf.device and value.is_contiguous() and buf.is_contiguous() and value.numel() > 0:
             rows = value.shape[0] if value.dim() > 0 else 1
             row_bytes = value.numel() * value.element_size() // max(rows, 1)
             self.kernels.split_gather(value, buf, row_bytes, 0, rows)(self.stream())
