@@ -603,6 +603,15 @@ def main():
                                frac=roof.get("frac"), all_gemm_tflops=roof.get("all_gemm_tflops"),
                                loss_scaling=res["loss_scaling"]))
             release(r2)
+            r2 = None
+            if not args.no_eager_baseline and time.perf_counter() - t_start < 240.0:
+                try:   # the same step in plain PyTorch eager, where the leg covers the model family
+                    e2 = torch_eager_gpu(name, device, steps=3, warmup=2)
+                except Exception as e:
+                    e2 = dict(skipped="failed: %s" % (str(e)[:200],))
+                if e2 is not None:
+                    others[-1]["torch_eager_gpu"] = e2
+                    log("[bench] torch eager on this GPU", name, e2)
 
     info = head["info"]
     rec = {
