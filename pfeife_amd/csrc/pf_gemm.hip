@@ -380,6 +380,188 @@ __global__ __launch_bounds__(256) void gemm32_kernel(const pf_gemm_desc p, const
   }
 }
 
+// ---------------------------------------------------------------------------
+// fp32 MFMA kernel (v_mfma_f32_32x32x2_f32): BM x BN tile, TK deep, four wavefronts as 2 x 2, each
+// owning (BM/2) x (BN/2) outputs.  Operand tiles sit in LDS reduction-major ([k][row], the order in
+// which a lane reads its one element per matrix instruction: row = lane % 32, k = lane / 32); the
+// next tile is fetched into registers while the current one is multiplied (two LDS buffers where
+// they fit, else one and a second barrier).  The small tile is 64 deep: its problems leave one
+// workgroup per CU, so a tile's matrix work has to cover the latency of the next tile's loads.
+// Any layout and any size: rows / reduction indices out of range read as zero.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int TK, bool AT, bool BT, bool VEC>
+__global__ __launch_bounds__(256) void gemm32x_kernel(const pf_gemm_desc p, const GemmGrid g) {
+  constexpr int PAD = 4;
+  constexpr int NBUF = (2 * TK * (BM + BN + 2 * PAD) * 4 <= 60 * 1024) ? 2 : 1;
+  constexpr int TMW = BM / 64, TNW = BN / 64;          // 32x32 accumulator tiles per wavefront
+  constexpr int NA = BM * TK / 256 / 4, NB = BN * TK / 256 / 4;   // 4-element loads per thread and tile
+  constexpr int WN = BN / 2, SLD = WN + 8;             // epilogue: floats per staged row of a wavefront's block
+  constexpr int TILE_FLOATS = NBUF * TK * (BM + BN + 2 * PAD), EPI_FLOATS = 4 * 32 * SLD;
+  __shared__ __align__(16) float smem[TILE_FLOATS > EPI_FLOATS ? TILE_FLOATS : EPI_FLOATS];
+  float (*sA)[TK][BM + PAD] = (float (*)[TK][BM + PAD])smem;
+  float (*sB)[TK][BN + PAD] = (float (*)[TK][BN + PAD])(smem + NBUF * TK * (BM + PAD));
+
+  const int t = gemm_tile_id((int)blockIdx.x, g.tiles_m * g.tiles_n, g.per_xcd);
+  if (t < 0) return;
+  int tm, tn;
+  gemm_tile_rc(t, g.tiles_m, g.tiles_n, tm, tn);
+  const int64_t M = p.M, N = p.N, K = p.K;
+  const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+  const int64_t z = blockIdx.y, z1 = z / p.batch2, z2 = z % p.batch2;
+  const float* A = (const float*)p.A + z1 * p.a_stride1 + z2 * p.a_stride2;
+  const float* B = (const float*)p.B + z1 * p.b_stride1 + z2 * p.b_stride2;
+  const int64_t c_base = z1 * p.c_stride1 + z2 * p.c_stride2;
+  const Epi epi = make_epi(p);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm0 = (wave >> 1) * (BM / 2), wn0 = (wave & 1) * (BN / 2);
+
+  // One operand tile -> registers, 4 consecutive elements along the operand's contiguous dimension
+  // (reduction index for a row-major operand, row index for a reduction-strided one).  No branches:
+  // indices are clamped into the operand and out-of-range elements are zeroed afterwards, so all of
+  // a tile's loads are in flight together (a branch around a load makes the compiler wait for it at
+  // the join).  VEC: one 16-byte load (the launcher has checked alignment and that the extent along
+  // the contiguous dimension is a multiple of 4, so a group of 4 is inside or outside as a whole).
+  auto fetch = [&](const float* X, int64_t ld, auto trans_c, int64_t r0, int64_t R, int64_t k0, int rows, int q,
+                   float (&v)[4]) {
+    constexpr bool TR = decltype(trans_c)::value;
+    const int e = tid + q * 256;
+    int r, k;
+    if (TR) { r = (e % (rows / 4)) * 4; k = e / (rows / 4); } else { k = (e % (TK / 4)) * 4; r = e / (TK / 4); }
+    const int64_t gr = r0 + r, gk = k0 + k;
+    if (VEC) {
+      const bool ok = gr < R && gk < K;
+      const int64_t cr = TR ? (gr < R ? gr : R - 4) : (gr < R ? gr : R - 1);
+      const int64_t ck = TR ? (gk < K ? gk : K - 1) : (gk < K ? gk : K - 4);
+      const float4 x = *(const float4*)(X + (TR ? ck * ld + cr : cr * ld + ck));
+      v[0] = ok ? x.x : 0.f; v[1] = ok ? x.y : 0.f; v[2] = ok ? x.z : 0.f; v[3] = ok ? x.w : 0.f;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t er = TR ? gr + j : gr, ek = TR ? gk : gk + j;
+        const bool ok = er < R && ek < K;
+        const int64_t cr = er < R ? er : R - 1, ck = ek < K ? ek : K - 1;
+        const float x = X[TR ? ck * ld + cr : cr * ld + ck];
+        v[j] = ok ? x : 0.f;
+      }
+    }
+  };
+  auto stash = [&](float* S, int ldS, auto trans_c, int rows, int q, const float (&v)[4]) {   // S: [TK][ldS]
+    constexpr bool TR = decltype(trans_c)::value;
+    const int e = tid + q * 256;
+    if (TR) {
+      const int r = (e % (rows / 4)) * 4, k = e / (rows / 4);
+      *(float4*)(S + k * ldS + r) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+      const int k = (e % (TK / 4)) * 4, r = e / (TK / 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) S[(k + j) * ldS + r] = v[j];
+    }
+  };
+  constexpr std::integral_constant<bool, AT> a_trans{};
+  constexpr std::integral_constant<bool, BT> b_trans{};
+
+  float16_t acc[TMW][TNW];
+#pragma unroll
+  for (int i = 0; i < TMW; ++i)
+#pragma unroll
+    for (int j = 0; j < TNW; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Two register sets: while tile `it` is multiplied out of LDS, tile it+1 waits in one set (stored
+  // to LDS at the end of the iteration) and tile it+2 is being fetched into the other, so a load has
+  // two tiles' worth of matrix instructions to arrive.  (Tiles past the end of K are requested too:
+  // the indices are clamped and nothing branches around the loads.)
+  float ra[2][NA][4], rb[2][NB][4];
+  auto fetch_tile = [&](int64_t k0, auto set_c) {
+    constexpr int S = decltype(set_c)::value;
+#pragma unroll
+    for (int q = 0; q < NA; ++q) fetch(A, p.lda, a_trans, m0, M, k0, BM, q, ra[S][q]);
+#pragma unroll
+    for (int q = 0; q < NB; ++q) fetch(B, p.ldb, b_trans, n0, N, k0, BN, q, rb[S][q]);
+  };
+  auto stash_tile = [&](int buf, auto set_c) {
+    constexpr int S = decltype(set_c)::value;
+#pragma unroll
+    for (int q = 0; q < NA; ++q) stash(&sA[buf][0][0], BM + PAD, a_trans, BM, q, ra[S][q]);
+#pragma unroll
+    for (int q = 0; q < NB; ++q) stash(&sB[buf][0][0], BN + PAD, b_trans, BN, q, rb[S][q]);
+  };
+  constexpr std::integral_constant<int, 0> set0{};
+  constexpr std::integral_constant<int, 1> set1{};
+  int cur = 0;
+  fetch_tile(0, set0);
+  stash_tile(0, set0);
+  fetch_tile(TK, set1);
+  __syncthreads();
+  auto body = [&](int64_t k0, auto mine, auto other) {   // tile at k0 is in LDS, `other` holds the next one
+    fetch_tile(k0 + 2 * TK, mine);
+#pragma unroll
+    for (int kk = 0; kk < TK / 2; ++kk) {
+      const int k = 2 * kk + (lane >> 5);
+      float a[TMW], b[TNW];
+#pragma unroll
+      for (int i = 0; i < TMW; ++i) a[i] = sA[cur][k][wm0 + i * 32 + (lane & 31)];
+#pragma unroll
+      for (int j = 0; j < TNW; ++j) b[j] = sB[cur][k][wn0 + j * 32 + (lane & 31)];
+#pragma unroll
+      for (int i = 0; i < TMW; ++i)
+#pragma unroll
+        for (int j = 0; j < TNW; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    if (NBUF == 1) __syncthreads();   // the single buffer is no longer read
+    const int nxt = NBUF == 2 ? cur ^ 1 : 0;
+    if (k0 + TK < K) stash_tile(nxt, other);
+    __syncthreads();   // the next tile is complete (and, with two buffers, this one no longer read)
+    cur = nxt;
+  };
+  for (int64_t k0 = 0; k0 < K; k0 += 2 * TK) {
+    body(k0, set0, set1);
+    if (k0 + TK < K) body(k0 + TK, set1, set0);
+  }
+  // Epilogue.  D layout of v_mfma_f32_32x32x*: lane l holds column l % 32 and rows 8*(r/4) + 4*(l/32) + r%4.
+  // Each wavefront re-lays one 32-row block at a time through a private LDS patch, after which WN/8
+  // adjacent lanes cover a whole row, 8 columns each: every global access of the epilogue moves 8
+  // elements (an element-wise epilogue pays one memory round trip per element and operand).
+  // (the last barrier of the K loop has passed: nobody reads the operand tiles any more)
+  float* stage = smem + wave * (32 * SLD);
+  constexpr int LPR = WN / 8, RPP = 64 / LPR;
+  const int rd_row = lane / LPR, rd_col = (lane % LPR) * 8;
+  const int64_t c8 = n0 + wn0 + rd_col;
+#pragma unroll
+  for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+    for (int j = 0; j < TNW; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        stage[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * SLD + j * 32 + (lane & 31)] = acc[i][j][r];
+#pragma nounroll
+    for (int it = 0; it < 32 / RPP; ++it) {
+      const int rr = it * RPP + rd_row;
+      const int64_t row = m0 + wm0 + i * 32 + rr;
+      const float4 x = *(const float4*)(stage + rr * SLD + rd_col), y = *(const float4*)(stage + rr * SLD + rd_col + 4);
+      if (row >= M || c8 >= N) continue;
+      float v[8] = {x.x, x.y, x.z, x.w, y.x, y.y, y.z, y.w};
+      if (g.vec_epi && c8 + 8 <= N) {
+        epilogue_vec8(epi, c_base, row, c8, v);
+      } else {
+#pragma nounroll
+        for (int k = 0; k < 8; ++k)
+          if (c8 + k < N) epilogue_scalar(epi, c_base, row, c8 + k, v[k]);
+      }
+    }
+  }
+}
+
+// fp32 problems: the matrix-instruction kernel with 128x128 tiles when those fill the GPU, with 64x64
+// tiles otherwise; the plain FMA kernel for problems smaller than one matrix-instruction tile.
+inline int f32_variant(const pf_gemm_desc& d) {
+  if (d.M < 32 || d.N < 32 || d.K < 8) return 0;
+  const int64_t nb = (d.batch1 > 0 ? d.batch1 : 1) * (d.batch2 > 0 ? d.batch2 : 1);
+  const int64_t t128 = ((d.M + 127) / 128) * ((d.N + 127) / 128) * nb;
+  return t128 >= 192 ? 128 : 64;
+}
+
 template <int DT, int BM, int BN, int BK, int WGM, int WGN>
 int launch16(const pf_gemm_desc& d, hipStream_t st) {
   constexpr int NT = 64 * WGM * WGN;
@@ -528,11 +710,38 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
 
   if (d.in_dtype == PF_F32) {
     GemmGrid g;
-    g.tiles_m = (int)tm64;
-    g.tiles_n = (int)tn64;
-    g.per_xcd = (int)((tm64 * tn64 + 7) / 8);
     g.vec_epi = 0;
-    hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(g.per_xcd * 8), (unsigned)nb, 1), dim3(256), 0, st, d, g);
+    const int v32 = f32_variant(d);
+    if (v32 == 0) {
+      g.tiles_m = (int)tm64;
+      g.tiles_n = (int)tn64;
+      g.per_xcd = (int)((tm64 * tn64 + 7) / 8);
+      hipLaunchKernelGGL(gemm32_kernel, dim3((unsigned)(g.per_xcd * 8), (unsigned)nb, 1), dim3(256), 0, st, d, g);
+    } else {
+      g.tiles_m = (int)((d.M + v32 - 1) / v32);
+      g.tiles_n = (int)((d.N + v32 - 1) / v32);
+      g.per_xcd = (int)(((int64_t)g.tiles_m * g.tiles_n + 7) / 8);
+      g.vec_epi = epi_vec_ok(d);
+      const dim3 grid((unsigned)(g.per_xcd * 8), (unsigned)nb, 1);
+      // 16-byte loads need aligned operands whose extent along the contiguous dimension is a multiple of 4
+      const bool vec = pf_aligned(d.A, 16) && pf_aligned(d.B, 16) && d.lda % 4 == 0 && d.ldb % 4 == 0 &&
+                       d.a_stride1 % 4 == 0 && d.a_stride2 % 4 == 0 && d.b_stride1 % 4 == 0 && d.b_stride2 % 4 == 0 &&
+                       (d.a_trans ? d.M : d.K) % 4 == 0 && (d.b_trans ? d.N : d.K) % 4 == 0 && d.K >= 4 && d.M >= 4 && d.N >= 4;
+#define PF_G32(BMN, TK, AT, BT, V) hipLaunchKernelGGL((gemm32x_kernel<BMN, BMN, TK, AT, BT, V>), grid, dim3(256), 0, st, d, g)
+#define PF_G32V(BMN, TK, AT, BT) do { if (vec) PF_G32(BMN, TK, AT, BT, true); else PF_G32(BMN, TK, AT, BT, false); } while (0)
+#define PF_G32L(BMN, TK)                                   \
+  do {                                                     \
+    if (d.a_trans && d.b_trans) PF_G32V(BMN, TK, true, true);   \
+    else if (d.a_trans) PF_G32V(BMN, TK, true, false);          \
+    else if (d.b_trans) PF_G32V(BMN, TK, false, true);          \
+    else PF_G32V(BMN, TK, false, false);                        \
+  } while (0)
+      if (v32 == 128) PF_G32L(128, 16);
+      else PF_G32L(64, 64);
+#undef PF_G32L
+#undef PF_G32V
+#undef PF_G32
+    }
     PF_CHECK_LAUNCH("pf_gemm(f32)");
     return PF_OK;
   }
@@ -618,7 +827,9 @@ extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   if (d.batch1 <= 0) d.batch1 = 1;
   if (d.batch2 <= 0) d.batch2 = 1;
   if (d.in_dtype == PF_F32 || d.K == 0) {
-    snprintf(out, (size_t)cap, "gemm32_kernel");
+    const int v32 = (d.in_dtype == PF_F32 && d.K > 0) ? f32_variant(d) : 0;
+    if (v32) snprintf(out, (size_t)cap, "gemm32x_kernel<%d, %d, %d>", v32, v32, v32 == 128 ? 16 : 64);
+    else snprintf(out, (size_t)cap, "gemm32_kernel");
     return PF_OK;
   }
   const char* at = d.a_trans ? "true" : "false";
