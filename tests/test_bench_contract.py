@@ -49,3 +49,40 @@ def test_only_the_cpu_baseline_leg_imports_the_oracle():
         mod = node.module if isinstance(node, ast.ImportFrom) else ",".join(a.name for a in node.names)
         assert "oracle" not in (mod or "")
     assert users == {"cpu_baseline"}, users
+
+
+def test_the_product_package_never_imports_the_checker_or_scratch_files():
+    """Nothing under pfeife_amd/ (nor the `pfeife` alias package) imports `oracle` or reads `_work/`;
+    `__graft_entry__.py` imports the oracle in smoke() only."""
+    bad = []
+    for top in ("pfeife_amd", "pfeife"):
+        for dirpath, _, files in os.walk(os.path.join(ROOT, top)):
+            for f in files:
+                if not f.endswith(".py"):
+                    continue
+                path = os.path.join(dirpath, f)
+                src = open(path).read()
+                tree = ast.parse(src)
+                for node in ast.walk(tree):
+                    mods = []
+                    if isinstance(node, ast.ImportFrom) and node.module:
+                        mods = [node.module]
+                    elif isinstance(node, ast.Import):
+                        mods = [a.name for a in node.names]
+                    if any(m == "oracle" or m.startswith("oracle.") for m in mods):
+                        bad.append(path)
+                if "_work/" in src or "_work\\\\" in src:
+                    bad.append(path + " (_work)")
+    assert not bad, bad
+    tree = ast.parse(open(os.path.join(ROOT, "__graft_entry__.py")).read())
+    users = set()
+    for fn in [n for n in tree.body if isinstance(n, ast.FunctionDef)]:
+        for node in ast.walk(fn):
+            mods = []
+            if isinstance(node, ast.ImportFrom) and node.module:
+                mods = [node.module]
+            elif isinstance(node, ast.Import):
+                mods = [a.name for a in node.names]
+            if any(m == "oracle" or m.startswith("oracle.") for m in mods):
+                users.add(fn.name)
+    assert users <= {"smoke", "build"}, users
