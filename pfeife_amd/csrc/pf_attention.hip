@@ -899,6 +899,182 @@ __global__ __launch_bounds__(NT) void attn_dkv_short_kernel(const AttnArgs a, in
   }
 }
 
+// dQ, dK and dV of one head in ONE workgroup of eight wavefronts (heads of up to 256 queries and 256
+// keys, head dim <= 64): Q, dO, K and V are loaded into LDS once (4 x 32 KB at 197 tokens), every
+// wavefront first forms delta and dQ for its 32 queries (sweeping the keys), then, after one barrier,
+// dK and dV for its 32 keys (sweeping the queries); against the two-kernel form this saves a launch and
+// one load of the head.  Same arithmetic, in the same order, as attn_dq_short_kernel and
+// attn_dkv_short_kernel.
+template <int DT, int HD>
+__global__ __launch_bounds__(512) void attn_bwd_short_fused_kernel(const AttnArgs a, float* delta_out, int rows_q, int rows_k) {
+  constexpr int NC = HD / 16, NO = HD / 32, LD = HD + 8, NT = 512;
+  extern __shared__ __align__(16) uint16_t smem[];
+  uint16_t* sK = smem;
+  uint16_t* sV = sK + rows_k * LD;
+  uint16_t* sQ = sV + rows_k * LD;
+  uint16_t* sDO = sQ + rows_q * LD;
+  float* sLse = (float*)(sDO + rows_q * LD);
+  float* sDelta = sLse + rows_q;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  const uint16_t* OO = a.o + b * a.o_sb + h * a.o_sh;
+  const float sc = a.scale * LOG2E;
+  const int shift = a.Tk - a.Tq;
+
+  // delta = rowsum(dO * O) and lse of this lane's query row: requested before the head is loaded
+  const int q0 = wave * 32, qi = q0 + (lane & 31);
+  const bool qok = qi < a.Tq;
+  const uint16_t* DOg = a.d_o + b * a.do_sb + h * a.do_sh;
+  float dlt = 0.f;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int h0 = c * 16 + (lane >> 5) * 8;
+    const uint4 dof = load_row8(DOg, a.do_st, qi, a.Tq, h0, a.hd);
+    const uint4 of = load_row8(OO, a.o_st, qi, a.Tq, h0, a.hd);
+    float x[8], y[8];
+    unpack8<DT>(dof, x);
+    unpack8<DT>(of, y);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) dlt += x[k] * y[k];
+  }
+  dlt += __shfl_xor(dlt, 32, 64);
+  const float lse2 = qok ? a.lse[(int64_t)bh * a.Tq + qi] * LOG2E : INFINITY;
+  load_heads<HD, NT>(a.k + b * a.k_sb + h * a.k_sh, a.k_st, a.v + b * a.v_sb + h * a.v_sh, a.v_st, a.Tk, a.hd, rows_k, sK,
+                     sV, tid);
+  load_heads<HD, NT>(a.q + b * a.q_sb + h * a.q_sh, a.q_st, DOg, a.do_st, a.Tq, a.hd, rows_q, sQ, sDO, tid);
+  if (q0 < rows_q && (lane >> 5) == 0) {
+    // rows past the end: Q and dO rows are zero, lse = +inf makes their P exactly zero
+    sLse[qi] = lse2;
+    sDelta[qi] = qok ? dlt : 0.f;
+    if (qok) delta_out[(int64_t)bh * a.Tq + qi] = dlt;
+  }
+  __syncthreads();
+
+  // ---- dQ for queries q0 .. q0+31
+  if (q0 < a.Tq) {
+    uint4 qf[NC], dof[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int off = qi * LD + c * 16 + (lane >> 5) * 8;
+      qf[c] = *(const uint4*)(sQ + off);
+      dof[c] = *(const uint4*)(sDO + off);
+    }
+    float16_t acc[NO];
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[o][r] = 0.f;
+    const int k_end = a.causal ? min(a.Tk, min(q0 + 31, a.Tq - 1) + shift + 1) : a.Tk;
+    for (int k0 = 0; k0 < k_end; k0 += 32) {
+      float16_t s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int off = (k0 + (lane & 31)) * LD + c * 16 + (lane >> 5) * 8;
+        s = M32<DT>::run(*(const uint4*)(sK + off), qf[c], s);
+        dp = M32<DT>::run(*(const uint4*)(sV + off), dof[c], dp);
+      }
+      const bool masked = (k0 + 32 > a.Tk) || (a.causal && k0 + 31 > q0 + shift);
+      if (masked) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kj = k0 + acc_row(r, lane);
+          const bool ok = kj < a.Tk && (!a.causal || kj <= qi + shift);
+          const float p = ok ? __builtin_amdgcn_exp2f(s[r] * sc - lse2) : 0.f;
+          s[r] = p * (dp[r] - dlt);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(s[r] * sc - lse2) * (dp[r] - dlt);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const uint4 dsf = pack8<DT>(s, 8 * j);
+#pragma unroll
+        for (int o = 0; o < NO; ++o) acc[o] = M32<DT>::run(frag_tr<LD>(sK, k0 + 16 * j, o * 32, lane), dsf, acc[o]);
+      }
+    }
+    if (qok) {
+      uint16_t* DQ = a.dq + b * a.dq_sb + h * a.dq_sh + (int64_t)qi * a.dq_st;
+#pragma unroll
+      for (int o = 0; o < NO; ++o)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+          if (h0 < a.hd)
+            *(uint2*)(DQ + h0) = make_uint2(M32<DT>::pack(acc[o][4 * g] * a.scale, acc[o][4 * g + 1] * a.scale),
+                                            M32<DT>::pack(acc[o][4 * g + 2] * a.scale, acc[o][4 * g + 3] * a.scale));
+        }
+    }
+  }
+
+  // ---- dK, dV for keys kw0 .. kw0+31 (sLse / sDelta were complete at the barrier above)
+  const int kw0 = wave * 32, kj = kw0 + (lane & 31);
+  if (kw0 >= a.Tk) return;
+  const bool kok = kj < a.Tk;
+  uint4 kf[NC], vf[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int off = kj * LD + c * 16 + (lane >> 5) * 8;   // rows up to rows_k are in LDS (zero past Tk)
+    kf[c] = *(const uint4*)(sK + off);
+    vf[c] = *(const uint4*)(sV + off);
+  }
+  float16_t dk[NO], dv[NO];
+#pragma unroll
+  for (int o = 0; o < NO; ++o)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[o][r] = dv[o][r] = 0.f;
+  int q_begin = 0;
+  if (a.causal) q_begin = max(0, kw0 - shift) / 32 * 32;
+  for (int qs = q_begin; qs < a.Tq; qs += 32) {
+    const bool masked = a.causal && (kw0 + 31 > qs + shift);
+    float16_t s, dp;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int off = (qs + (lane & 31)) * LD + c * 16 + (lane >> 5) * 8;
+      s = M32<DT>::run(*(const uint4*)(sQ + off), kf[c], s);
+      dp = M32<DT>::run(*(const uint4*)(sDO + off), vf[c], dp);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int ql = qs + acc_row(r, lane);
+      float p = __builtin_amdgcn_exp2f(s[r] * sc - sLse[ql]);
+      if (masked && kj > ql + shift) p = 0.f;
+      s[r] = p;
+      dp[r] = p * (dp[r] - sDelta[ql]);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const uint4 pf = pack8<DT>(s, 8 * j);
+      const uint4 dsf = pack8<DT>(dp, 8 * j);
+#pragma unroll
+      for (int o = 0; o < NO; ++o) {
+        dv[o] = M32<DT>::run(frag_tr<LD>(sDO, qs + 16 * j, o * 32, lane), pf, dv[o]);
+        dk[o] = M32<DT>::run(frag_tr<LD>(sQ, qs + 16 * j, o * 32, lane), dsf, dk[o]);
+      }
+    }
+  }
+  if (kok) {
+    uint16_t* DK = a.dk + b * a.dk_sb + h * a.dk_sh + (int64_t)kj * a.dk_st;
+    uint16_t* DV = a.dv + b * a.dv_sb + h * a.dv_sh + (int64_t)kj * a.dv_st;
+#pragma unroll
+    for (int o = 0; o < NO; ++o)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int h0 = o * 32 + 8 * g + 4 * (lane >> 5);
+        if (h0 < a.hd) {
+          *(uint2*)(DK + h0) = make_uint2(M32<DT>::pack(dk[o][4 * g] * a.scale, dk[o][4 * g + 1] * a.scale),
+                                          M32<DT>::pack(dk[o][4 * g + 2] * a.scale, dk[o][4 * g + 3] * a.scale));
+          *(uint2*)(DV + h0) = make_uint2(M32<DT>::pack(dv[o][4 * g], dv[o][4 * g + 1]),
+                                          M32<DT>::pack(dv[o][4 * g + 2], dv[o][4 * g + 3]));
+        }
+      }
+  }
+}
+
 bool strides_ok(const void* p, int64_t sb, int64_t sh, int64_t st) {
   return pf_aligned(p, 16) && sb % 8 == 0 && sh % 8 == 0 && st % 8 == 0;
 }
@@ -1034,8 +1210,18 @@ extern "C" int pf_attention_bwd(const pf_attn_desc* d, void* stream) {
   const dim3 gq((unsigned)((d->Tq + 127) / 128), (unsigned)(d->B * d->H));
   const dim3 gk((unsigned)((d->Tk + 127) / 128), (unsigned)(d->B * d->H));
   if (d->Tq <= SHORT_T && d->Tk <= SHORT_T) {
-    // dQ first: it also leaves delta = rowsum(dO * O) for the dK/dV kernel
     const int rows_k = (d->Tk + 31) / 32 * 32, rows_q = (d->Tq + 31) / 32 * 32;
+    if (d->hd <= 64 && d->Tq <= 256 && d->Tk <= 256 && (d->Tq > 128 || d->Tk > 128)) {
+      // one workgroup per head forms dQ, dK and dV from a single load of the head
+      const size_t lds = (size_t)2 * (rows_k + rows_q) * (64 + 8) * 2 + (size_t)rows_q * 8;
+      const dim3 gf(1, (unsigned)(d->B * d->H));
+      if (d->dtype == PF_F16) rc = launch_short(attn_bwd_short_fused_kernel<PF_F16, 64>, gf, 512, lds, st, a, d->delta, rows_q, rows_k);
+      else rc = launch_short(attn_bwd_short_fused_kernel<PF_BF16, 64>, gf, 512, lds, st, a, d->delta, rows_q, rows_k);
+      if (rc != PF_OK) return rc;
+      PF_CHECK_LAUNCH("pf_attention_bwd");
+      return PF_OK;
+    }
+    // dQ first: it also leaves delta = rowsum(dO * O) for the dK/dV kernel
     auto lds_q = [rows_k](int HD) { return (size_t)2 * rows_k * (HD + 8) * 2; };
     auto lds_k = [rows_q](int HD) { return (size_t)2 * rows_q * (HD + 8) * 2 + (size_t)rows_q * 8; };
     PF_ATTN_SHORT(attn_dq_short_kernel, 512, rc, d->Tq, d->B * d->H, lds_q, st, d->dtype, d->hd, a, d->delta, rows_k);
