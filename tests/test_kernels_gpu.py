@@ -571,6 +571,8 @@ def test_deferred_reductions_match_immediate(hip):
     dict(B=2, H=3, Tq=200, Tk=160, hd=64, causal=0, packed=False),   # one-workgroup backward, more queries than keys
     dict(B=1, H=2, Tq=150, Tk=250, hd=64, causal=1, packed=False),   # one-workgroup backward, causal with more keys
     dict(B=1, H=2, Tq=256, Tk=256, hd=40, causal=1, packed=False),   # one-workgroup backward at its largest head
+    dict(B=1, H=3, Tq=200, Tk=40, hd=64, causal=0, packed=False),    # one-workgroup backward, two key tiles only
+    dict(B=1, H=2, Tq=33, Tk=250, hd=16, causal=0, packed=False),    # one-workgroup backward, two query tiles only
     dict(B=1, H=2, Tq=330, Tk=40, hd=88, causal=0, packed=False),    # the same at head dim 88, ragged query blocks
     dict(B=1, H=2, Tq=160, Tk=170, hd=96, causal=0, packed=False),   # head dim 96: six key tiles in one 4-wavefront workgroup
 ])
