@@ -187,10 +187,11 @@ class PartialRunner:
         get_logger().info(self.worker.memory_report())
 
     def train(self):
-        pass
+        """No-op, as in the reference (pfeife/mp/partial/module.py:175-177): stage programs are built
+        from the graph TorchDynamo captured, and a captured dropout with p > 0 is refused at lowering."""
 
     def eval(self):
-        pass
+        """No-op, as in the reference (pfeife/mp/partial/module.py:179-181)."""
 
     # -- helpers --------------------------------------------------------------------
     def _exec_loop(self, batch_idx):
