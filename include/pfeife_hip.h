@@ -131,6 +131,12 @@ typedef struct pf_gemm_desc {
                       harnesses): 1..3 direct-to-LDS kernel with 256x256 / 256x128 / 128x128
                       tiles, 11..14 register-staged kernel with 128x128 (8 wavefronts),
                       128x128, 128x64, 64x64 tiles; PF_ERR_INVALID if it cannot run the problem */
+  float* colsum_ws; /* optional, with dact on the direct-to-LDS kernel (pf_gemm_variant ends in ", 5>"): the
+                       launch also leaves the column sums of the 16-bit values it stores in C as partial
+                       rows, ws[tile_row * N + column] for tile_row < ceil(M / BM) (BM: the variant's first
+                       tile dimension): the bias gradient of the layer whose pre-activation gradient C is
+                       (aten.sum of the reference's autograd, pfeife/mp/worker.py:1585-1587), finished by
+                       pf_colreduce_finalize(_batch).  PF_ERR_UNSUPPORTED on any other kernel path. */
 } pf_gemm_desc;
 
 int pf_gemm(const pf_gemm_desc* desc, void* stream);

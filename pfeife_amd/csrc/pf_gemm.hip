@@ -663,6 +663,14 @@ int resolve_variant(const pf_gemm_desc& d) { return d.variant == V_AUTO ? choose
 template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
   const int v = resolve_variant(d);
+  if (d.colsum_ws != nullptr) {   // only the GELU' class of the direct-to-LDS kernel sums its columns
+    const bool xk = v == V_X256 || v == V_X256x128 || v == V_X128 || v == V_X192x256;
+    if (!xk || d.a_trans || d.b_trans || !x_supports(d, v) || epi_class(d, epi_vec_ok(d)) != EC_DACT16 ||
+        !pf_aligned(d.colsum_ws, 16)) {
+      pf_set_error("pf_gemm: colsum_ws needs a 16-bit product with the GELU' epilogue on the direct-to-LDS kernel");
+      return PF_ERR_UNSUPPORTED;
+    }
+  }
   switch (v) {
     case V_X256: case V_X256x128: case V_X128: case V_X192x256: {
       const int xt = v;   // variant ids 1..5 are the PF_XT_* tile ids
@@ -710,6 +718,10 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
   PF_REQUIRE(tm64 * tn64 < (1ll << 30), "pf_gemm: problem too large for one launch");
 
   if (d.in_dtype == PF_F32) {
+    if (d.colsum_ws != nullptr) {
+      pf_set_error("pf_gemm: colsum_ws needs a 16-bit product with the GELU' epilogue on the direct-to-LDS kernel");
+      return PF_ERR_UNSUPPORTED;
+    }
     GemmGrid g;
     g.vec_epi = 0;
     const int v32 = f32_variant(d);

@@ -24,6 +24,7 @@ struct Epi {
   const void* residual;
   void* C;
   int64_t ldc, ld_aux_out, ld_aux_in, ld_res;
+  float* colsum_ws;
 };
 
 __device__ __forceinline__ Epi make_epi(const pf_gemm_desc& p) {
@@ -32,6 +33,7 @@ __device__ __forceinline__ Epi make_epi(const pf_gemm_desc& p) {
   e.in_dtype = p.in_dtype; e.c_dtype = p.c_dtype; e.bias_dtype = p.bias_dtype; e.res_dtype = p.res_dtype;
   e.bias = p.bias; e.aux_out = p.aux_out; e.aux_in = p.aux_in; e.residual = p.residual; e.C = p.C;
   e.ldc = p.ldc; e.ld_aux_out = p.ld_aux_out; e.ld_aux_in = p.ld_aux_in; e.ld_res = p.ld_res;
+  e.colsum_ws = p.colsum_ws;
   return e;
 }
 

@@ -413,6 +413,7 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
         }
       }
     };
+    float8_t csum = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // EC_DACT16: column sums of the stored values
     fetch(0);
 #pragma nounroll
     for (int hb = 0; hb < NHB; ++hb) {
@@ -492,7 +493,44 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
           __builtin_amdgcn_raw_buffer_store_b128(lo, rs_c, (int)oc, 0, 0);
           __builtin_amdgcn_raw_buffer_store_b128(hi, rs_c, (int)(oc + 16), 0, 0);
         } else {
-          __builtin_amdgcn_raw_buffer_store_b128(pack16<DT>(v), rs_c, (int)oc, 0, 0);
+          const v4i_t packed = pack16<DT>(v);
+          if constexpr (EC == EC_DACT16) {   // sums run over the ROUNDED values, rows past M excluded
+            const float keep = (row0 + (int64_t)rowk < M) ? 1.f : 0.f;
+            csum += unpack16<DT>(packed) * keep;
+          }
+          __builtin_amdgcn_raw_buffer_store_b128(packed, rs_c, (int)oc, 0, 0);
+        }
+      }
+    }
+    if constexpr (EC == EC_DACT16) {
+      if (epi.colsum_ws != nullptr) {   // uniform over the grid
+        // lanes l, l + LPR, l + 2 LPR, ... hold the same 8 columns (different rows)
+#pragma unroll
+        for (int off = LPR; off < 64; off <<= 1)
+#pragma unroll
+          for (int k = 0; k < 8; ++k) csum[k] += __shfl_xor(csum[k], off, 64);
+        // wavefronts of one block column add up in wavefront-row order through LDS (every wavefront
+        // is done with its own epilogue patch at the barrier; the patch of partial sums lies below
+        // the first wavefront's operand buffers, which the last, unused prefetch may still be filling)
+        float* red = (float*)smem;
+        static_assert(NW * WN * 4 <= HB * SLD * 4, "partial column sums overlap the operand buffers");
+        lds_barrier();
+        if (lane < LPR) {
+#pragma unroll
+          for (int k = 0; k < 8; ++k) red[wave * WN + lane * 8 + k] = csum[k];
+        }
+        lds_barrier();
+        if (wave / WGN == 0 && lane < LPR && c8 < N) {
+          float t[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) t[k] = 0.f;
+#pragma unroll
+          for (int w = 0; w < WGM; ++w)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) t[k] += red[(w * WGN + wave % WGN) * WN + lane * 8 + k];
+          float* dst = epi.colsum_ws + (int64_t)tm * N + c8;
+          *(float4*)dst = make_float4(t[0], t[1], t[2], t[3]);
+          *(float4*)(dst + 4) = make_float4(t[4], t[5], t[6], t[7]);
         }
       }
     }

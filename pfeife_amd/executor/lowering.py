@@ -23,6 +23,8 @@ parameter gradients are accumulated in fp32.
 import math
 import operator
 
+import os
+
 import torch
 import torch.nn.functional as F
 
@@ -841,8 +843,16 @@ def lower_linear(L, node):
                     if pm is None:
                         raise Unsupported("accumulating into a non-matrix gradient")
                     kw2.update(residual=prev, ld_res=pm[2])
-                B.emit(B.k.gemm(dy, wb, dst, ldc=dm[2], **kw2))
+                launch = B.k.gemm(dy, wb, dst, ldc=dm[2], **kw2)
+                B.emit(launch)
                 B.commit(x, dst)
+                if ("dact" in kw2 and hasattr(B.k, "gemm_attach_colsum") and dm[2] == K
+                        and os.environ.get("PFEIFE_EPILOGUE_COLSUM", "1") != "0"):
+                    # dst now holds the gradient of the producing layer's pre-activation: its column sums
+                    # are that layer's bias gradient, and the product's epilogue can leave them behind
+                    cs = B.k.gemm_attach_colsum(launch, B.temp)
+                    if cs is not None:
+                        B.register_lp(dst, dst, colsum=cs)
             else:
                 # target is not a plain matrix (e.g. a permuted view): go through a temp
                 tmp = B.temp(tuple(x.shape), x.dtype)

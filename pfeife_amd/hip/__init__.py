@@ -58,6 +58,7 @@ class GemmDesc(Structure):
         ("aux_in", c_void_p), ("ld_aux_in", c_int64),
         ("residual", c_void_p), ("ld_res", c_int64),
         ("res_dtype", c_int32), ("variant", c_int32),
+        ("colsum_ws", c_void_p),
     ]
 
 
@@ -305,6 +306,25 @@ class HipKernels:
         launch.flops = 2.0 * M * N * K * batch[0] * batch[1]
         launch.desc = d
         return launch
+
+    def gemm_attach_colsum(self, launch, alloc):
+        """Make a prepared product with a fused GELU' epilogue on the direct-to-LDS kernel also leave the
+        column sums of what it stores (the bias gradient of the layer whose pre-activation gradient it
+        writes) as partial rows.  alloc(shape, dtype) -> workspace tensor that outlives the launch.
+        -> (workspace, offset, partial rows, row stride) for the deferred finish, or None when the
+        launch runs on another kernel."""
+        v = getattr(launch, "variant", "")
+        d = getattr(launch, "desc", None)
+        if d is None or not (v.startswith("gemm16x_kernel<") and v.endswith(", false, false, 5>")):
+            return None
+        if d.batch1 * d.batch2 != 1 or d.colsum_ws:
+            return None
+        bm = int(v.split("<")[1].split(",")[1])
+        nb = (d.M + bm - 1) // bm
+        ws = alloc((nb, d.N), torch.float32)
+        d.colsum_ws = ws.data_ptr()
+        launch.colsum_ws = ws
+        return ws, 0, nb, d.N
 
     GEMM_GROUP_MAX = 4
 

@@ -169,6 +169,39 @@ def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
     close(r["c"], rt, at * 2)
 
 
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("variant,bm", [(1, 256), (2, 256), (3, 128), (4, 192)])
+def test_gemm_gelu_grad_epilogue_leaves_column_sums(hip, dtype, variant, bm):
+    """The GELU' epilogue of the direct-to-LDS kernel can also leave the column sums of the values it
+    stores (the bias gradient of the layer whose pre-activation gradient it writes) as one partial row
+    per tile row: their sum must equal the column sums of the stored 16-bit matrix (fp32 adds of the
+    same numbers in another order), ragged in M and N; the output itself must not change."""
+    M, N, K = 1000, 1160, 320
+    x, w = rnd((M, K), dtype, 1).cuda(), rnd((N, K), dtype, 2, 0.1).cuda()
+    pre = rnd((M, N), dtype, 6).cuda()
+    kw = dict(M=M, N=N, K=K, lda=K, ldb=K, ldc=N, dact=1, ld_aux_in=N, variant=variant)
+    plain = torch.zeros(M, N, dtype=dtype, device="cuda")
+    hip.gemm(x, w, plain, aux_in=pre, **kw)(torch.cuda.current_stream().cuda_stream)
+    out = torch.zeros(M, N, dtype=dtype, device="cuda")
+    launch = hip.gemm(x, w, out, aux_in=pre, **kw)
+    cs = hip.gemm_attach_colsum(launch, lambda shape, dt: torch.full(shape, float("nan"), dtype=dt, device="cuda"))
+    assert cs is not None and launch.variant.endswith(", 5>")
+    ws, off, nb, stride = cs
+    assert (off, nb, stride) == (0, (M + bm - 1) // bm, N) and tuple(ws.shape) == (nb, N)
+    launch(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(out, plain)
+    got = ws.double().sum(0).cpu()
+    want = out.double().sum(0).cpu()
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-4)
+    # any other kernel path refuses the request loudly
+    other = hip.gemm(x, w, torch.zeros(M, N, dtype=dtype, device="cuda"), M=M, N=N, K=K, lda=K, ldb=K, ldc=N, variant=variant)
+    assert hip.gemm_attach_colsum(other, lambda shape, dt: torch.zeros(shape, dtype=dt, device="cuda")) is None
+    other.desc.colsum_ws = ws.data_ptr()
+    with pytest.raises(RuntimeError, match="colsum_ws"):
+        other(torch.cuda.current_stream().cuda_stream)
+
+
 def test_gemm_full_size_vit_l(hip, oracle):
     # qkv projection of ViT-L/16 at micro-batch 16: [3152 x 1024] . [1024 x 3072]
     M, N, K = 3152, 3072, 1024
