@@ -52,7 +52,7 @@ def test_only_the_cpu_baseline_leg_imports_the_oracle():
 
 
 def test_the_product_package_never_imports_the_checker_or_scratch_files():
-    """Nothing under pfeife_amd/ (nor the `pfeife` alias package) imports `oracle` or reads `_work/`;
+    """Nothing under pfeife_amd/ (nor the `pfeife` alias package) imports `oracle` or reads the scratch folder;
     `__graft_entry__.py` imports the oracle in smoke() only."""
     bad = []
     for top in ("pfeife_amd", "pfeife"):
