@@ -420,10 +420,10 @@ class StageWorker:
                 self.kernels.scale_by_state(g, self.scaler_state, buf, g.numel())(self.stream())
             else:
                 # the kernel walks both operands as flat arrays: anything with strides of its own (an output
-                # kept channels-last in memory, a permuted gradient) goes through a stride-aware copy first;
-                # the scale stays on the device (a 0-dim view of the scaler state, no host read)
-                buf.copy_(g)
-                buf.mul_(self.scaler_state[0])
+                # kept channels-last in memory, a permuted gradient) goes through a stride-aware copy.
+                # The product is formed in fp32 (the scale itself, 65536 by default, is not an fp16 number)
+                # and the scale stays on the device (a 0-dim view of the scaler state, no host read).
+                buf.copy_(g.to(device=buf.device, dtype=torch.float32) * self.scaler_state[0])
             return
         scale = self.option.loss_scale
         if g.device == buf.device and g.is_contiguous() and buf.is_contiguous() and g.dtype.is_floating_point:

@@ -716,7 +716,7 @@ def test_unet_stage_dynamic_loss_scale_with_a_tensor_valued_loss_gradient():
     ctx = torch.randn(B, 77, cfg.context_dim, generator=g).cuda()
     target = torch.randn(B, cfg.channels, hw, hw, generator=g).cuda()
     option = PipeOption(device_cnt=1, batch_cnt=1, batch_size=B, mixed_precision="fp16",
-                        optimizer=dict(type="adam", lr=1e-4), loss_scale="dynamic", init_scale=4096.0)
+                        optimizer=dict(type="adam", lr=1e-4), loss_scale="dynamic")   # initial scale 65536
     runner = _fresh_runner(option)
     model.cuda()
     cmodel = torch.compile(model, backend=partial_compiler)
@@ -730,9 +730,9 @@ def test_unet_stage_dynamic_loss_scale_with_a_tensor_valued_loss_gradient():
     runner.set_exec_fn(fn)
     got = [float(runner.step(hidden, temb, ctx, target)[0]) for _ in range(4)]
     torch.cuda.synchronize()
-    assert runner.worker.scaler_scale() == 4096.0      # no step overflowed
+    assert runner.worker.scaler_scale() == 65536.0     # no step overflowed (65536 itself is not an fp16 number)
     opt = torch.optim.Adam(ref.parameters(), lr=1e-4)
-    scaler = torch.amp.GradScaler("cuda", init_scale=4096.0)
+    scaler = torch.amp.GradScaler("cuda")
     want = []
     for _ in range(4):
         opt.zero_grad(set_to_none=False)
