@@ -863,6 +863,56 @@ def test_dynamic_loss_scale_matches_torch_gradscaler_and_adam():
                                    msg=n)
 
 
+def test_dynamic_loss_scale_with_an_optimizer_that_keeps_pytorchs_step():
+    """Dynamic loss scaling with SGD + momentum (no fused step: the overflow flag is read once on the host
+    and PyTorch's own step() runs or is skipped), fp32 model: five steps, the second with an overflowing
+    loss, against torch.amp.GradScaler + torch.optim.SGD; parameters and scale must agree."""
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=2, mlp_dim=128, num_classes=10)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(8, 3, 32, 32, generator=g).cuda()
+    y = torch.randint(0, 10, (8,), generator=g).cuda()
+    torch.manual_seed(0)
+    model = VisionTransformer(cfg)
+    ref = copy.deepcopy(model).cuda()
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=4, split_points=["blocks.1"],
+                        optimizer=dict(type="sgd", lr=0.05, momentum=0.9), loss_scale="dynamic", init_scale=256.0,
+                        growth_interval=2)
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+    poison = [False]
+
+    def fn(px, labels):
+        loss = crit(cmodel(px).float(), labels)
+        (loss * float("inf") if poison[0] else loss).backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    ropt = torch.optim.SGD(ref.parameters(), lr=0.05, momentum=0.9)
+    scaler = torch.amp.GradScaler("cuda", init_scale=256.0, growth_interval=2)
+    for step in range(5):
+        poison[0] = step == 1
+        runner.step(x, y)
+        ropt.zero_grad(set_to_none=False)
+        for xs, ys in zip(x.chunk(2), y.chunk(2)):
+            loss = crit(ref(xs), ys)
+            scaler.scale(loss * float("inf") if poison[0] else loss).backward()
+        scaler.step(ropt)
+        scaler.update()
+        torch.cuda.synchronize()
+        assert runner.worker.scaler_scale() == float(scaler.get_scale()), step
+        for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+            torch.testing.assert_close(p.detach(), q.detach(), rtol=2e-4, atol=2e-5,
+                                       msg=lambda m: "%s step %d: %s" % (n, step, m))
+    assert type(runner.worker.optimizer) is torch.optim.SGD
+    assert float(runner.worker.scaler_state[3]) == 4.0        # four completed steps, one skipped
+
+
 def test_fp16_defaults_to_dynamic_loss_scaling():
     """mixed_precision="fp16" without an explicit loss_scale runs the device-side scaler (the
     reference wraps fp16 training in a GradScaler, pfeife/mp/worker.py:133-145)."""
