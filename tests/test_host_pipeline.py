@@ -328,3 +328,43 @@ def test_print_graph_lists_stages_and_edges(capsys):
     # the parameters are split over the stages without overlap
     total = sum(pg.stage_summary(i)["weight"] for i in range(4))
     assert total == sum(p.numel() * 4 for p in model.parameters())
+
+
+def test_weights_tied_across_two_stages_accumulate_both_contributions():
+    """An embedding table that is also the output projection (first and last stage, different pipeline
+    ranks): its gradient is the sum of both stages' contributions over all micro-batches."""
+    import copy
+
+    from oracle.kernels_oracle import OracleKernels
+    from pfeife_amd.bench_models.llama import LlamaConfig, LlamaForCausalLM
+    from pfeife_amd.mp import PartialRunner, initialize_pfeife, net_states, partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = LlamaConfig(vocab=256, dim=64, layers=4, heads=4, ffn=176, max_seq=32)
+    torch.manual_seed(0)
+    model = LlamaForCausalLM(cfg)
+    model.lm_head.weight = model.embed.weight
+    ref = copy.deepcopy(model)
+    assert ref.lm_head.weight is ref.embed.weight
+    torch._dynamo.reset()
+    net_states._reset_state_for_tests()
+    initialize_pfeife(device="cpu")
+    option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=2, split_points=["layers.2"],
+                        optimizer=dict(type="sgd", lr=0.0))
+    runner = PartialRunner(option, kernels=OracleKernels("cpu"))
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(tok):
+        loss = cmodel(tok, tok)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    ids = torch.randint(0, cfg.vocab, (8, 32), generator=torch.Generator().manual_seed(1))
+    losses = runner.step(ids)
+    for chunk, got in zip(ids.chunk(4), losses):
+        want = ref(chunk, chunk)
+        want.backward()
+        assert abs(float(got) - float(want.detach())) <= 1e-5 * abs(float(want.detach()))
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n

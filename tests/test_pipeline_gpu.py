@@ -374,6 +374,56 @@ def test_vit_g14_share_config_trains_like_pytorch():
     assert ((got[-1] - got[0]) - (want[-1] - want[0])).abs().mean().item() <= 0.35 * drift
 
 
+def test_weights_tied_across_stages_train_like_pytorch():
+    """A decoder whose embedding table is also its output projection, split so that the two uses sit on
+    different pipeline ranks (the streams per rank are switched off for such a model): bf16 autocast, four
+    Adam steps against plain PyTorch; losses within 0.5 %, the tied weight moves the same way."""
+    from pfeife_amd.bench_models.llama import LlamaConfig, LlamaForCausalLM
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = LlamaConfig(vocab=512, dim=256, layers=4, heads=4, ffn=688, max_seq=128)
+    torch.manual_seed(0)
+    model = LlamaForCausalLM(cfg)
+    model.lm_head.weight = model.embed.weight
+    ref = copy.deepcopy(model).cuda()
+    w0 = ref.embed.weight.detach().clone()
+    ids = torch.randint(0, cfg.vocab, (8, 128), generator=torch.Generator().manual_seed(1)).cuda()
+    option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=2, split_points=["layers.2"], mixed_precision="bf16",
+                        optimizer=dict(type="adam", lr=1e-3))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+
+    def fn(tok):
+        loss = cmodel(tok, tok)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    got = [float(runner.step(ids)[-1]) for _ in range(4)]
+    torch.cuda.synchronize()
+    assert runner.worker.lanes is None                   # a parameter shared by two ranks: one stream
+    assert model.lm_head.weight is model.embed.weight
+    opt = torch.optim.Adam(ref.parameters(), lr=1e-3)
+    want = []
+    for _ in range(4):
+        opt.zero_grad(set_to_none=False)
+        for tok in ids.chunk(4):
+            with torch.autocast("cuda", dtype=torch.bfloat16):
+                loss = ref(tok, tok)
+            loss.backward()
+        opt.step()
+        want.append(float(loss.detach()))
+    assert want[-1] < want[0] - 0.05
+    for a, b in zip(got, want):
+        assert abs(a - b) <= 5e-3 * abs(b), (got, want)
+    d1, d2 = (model.embed.weight.detach() - w0).flatten(), (ref.embed.weight.detach() - w0).flatten()
+    firm = d2.abs() > 2e-3
+    assert int(firm.sum()) > 1000
+    assert float(((torch.sign(d1) != torch.sign(d2)) & firm).sum()) / float(firm.sum()) <= 0.02
+
+
 def test_ragged_batch_on_device():
     """N % batch_cnt != 0: torch.tensor_split gives micro-batches of 3, 3, 2, 2 samples
     (pfeife/batch.py:45); every one gets its own stage programs."""
