@@ -424,6 +424,48 @@ def test_weights_tied_across_stages_train_like_pytorch():
     assert float(((torch.sign(d1) != torch.sign(d2)) & firm).sum()) / float(firm.sum()) <= 0.02
 
 
+def test_batch_shape_that_changes_between_steps():
+    """An epoch's short last batch and back: eight SGD + momentum steps alternating 8- and 6-sample
+    batches (stage programs and their captured graphs exist per shape), fp32, against PyTorch."""
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=2, mlp_dim=128, num_classes=10)
+    g = torch.Generator().manual_seed(42)
+    xa, ya = torch.randn(8, 3, 32, 32, generator=g).cuda(), torch.randint(0, 10, (8,), generator=g).cuda()
+    xb, yb = torch.randn(6, 3, 32, 32, generator=g).cuda(), torch.randint(0, 10, (6,), generator=g).cuda()
+    torch.manual_seed(0)
+    model = VisionTransformer(cfg)
+    ref = copy.deepcopy(model).cuda()
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=4, split_points=["blocks.1"],
+                        optimizer=dict(type="sgd", lr=0.05, momentum=0.9))
+    runner = _fresh_runner(option)
+    model.cuda()
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+
+    def fn(px, labels):
+        loss = crit(cmodel(px).float(), labels)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    ropt = torch.optim.SGD(ref.parameters(), lr=0.05, momentum=0.9)
+    for step in range(8):
+        x, y = (xa, ya) if step % 3 != 2 else (xb, yb)
+        got = runner.step(x, y)
+        ropt.zero_grad(set_to_none=False)
+        for (xs, ys), a in zip(zip(x.chunk(2), y.chunk(2)), got):
+            loss = crit(ref(xs), ys)
+            loss.backward()
+            assert abs(float(a) - float(loss.detach())) <= 1e-4 * abs(float(loss.detach())) + 1e-6, step
+        ropt.step()
+        torch.cuda.synchronize()
+        for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+            torch.testing.assert_close(p.detach(), q.detach(), rtol=1e-4, atol=2e-5, msg=lambda m: "%s step %d: %s" % (n, step, m))
+
+
 def test_ragged_batch_on_device():
     """N % batch_cnt != 0: torch.tensor_split gives micro-batches of 3, 3, 2, 2 samples
     (pfeife/batch.py:45); every one gets its own stage programs."""
