@@ -340,11 +340,20 @@ def torch_eager_gpu(name, device, steps=5, warmup=2):
     from pfeife_amd.bench_models import unet_stage
 
     family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
-    if family not in ("vit", "llama", "unet"):
+    if family not in ("vit", "llama", "unet", "vit_share"):
         return None
     torch.manual_seed(42)
     g = torch.Generator().manual_seed(42)
-    if family == "unet":
+    if family == "vit_share":
+        cfg = getattr(vit, cfg_name)
+        model = vit.BlockStack(cfg).to(device)
+        x = torch.randn(batch, cfg.tokens, cfg.dim, generator=g).to(device)
+        y = (torch.randn(batch, cfg.tokens, cfg.dim, generator=g) * 1e-2).to(device)
+
+        def loss_of(xb, yb):   # the supplied upstream gradient, written as a loss: d(sum(out * g))/d(out) = g
+            out = model(xb)
+            return (out.float() * yb.float()).sum()
+    elif family == "unet":
         cfg = getattr(unet_stage, cfg_name)
         model = unet_stage.UNetStage(cfg).to(device)
         x = torch.randn(batch, cfg.in_channels, 32, 32, generator=g).to(device)
