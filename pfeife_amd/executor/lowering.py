@@ -317,6 +317,7 @@ class BwdCtx:
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
         self._dw = []       # held-back weight-gradient products: (launch, accumulator, tiles)
+        self._dw_big = []   # issued ones that fill the device alone: (launch, the same on 256x256 tiles, accumulator, tiles)
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
         self._lp = {}
@@ -343,10 +344,34 @@ class BwdCtx:
             self.emit(launch)
             return
         tiles = self._tiles(launch)
-        if any(g.data_ptr() == grad.data_ptr() for _, g, _ in self._dw):
+        if any(g.data_ptr() == grad.data_ptr() for _, g, _ in self._dw + [(None, g2, None) for _, _, g2, _ in self._dw_big]):
             self.flush_dw()          # two products into one accumulator keep their order
         if tiles >= self.FULL_GRID:
+            # Fills the device on its own with small tiles.  Four such products whose 256x256 tiles fill it
+            # TOGETHER (a decoder's four 2048x2048 attention projections: 64 tiles each) run faster as one
+            # launch on the large tile, which moves half the operand bytes per FLOP through LDS.  Each is
+            # issued where it stands and remembered; only when the set is complete do its members give
+            # way to the one launch, at the place of the last (a set that never completes costs nothing).
             self.emit(launch)
+            d = launch.desc
+            t256 = ((d.M + 255) // 256) * ((d.N + 255) // 256)
+            retile = getattr(self.k, "gemm_retiled", None) if os.environ.get("PFEIFE_DW_RETILE", "1") != "0" else None
+            big = retile(launch, 1) if (retile is not None and t256 * 2 <= self.FULL_GRID
+                                        and not launch.variant.startswith("gemm16x_kernel<%d, 256, 256" % d.in_dtype)) else None
+            if big is None or not groupable(big):
+                self._dw_big = []
+                return
+            if self._dw_big and (self._dw_big[0][1].variant != big.variant
+                                 or sum(t for _, _, _, t in self._dw_big) + t256 > self.FULL_GRID):
+                self._dw_big = []
+            self._dw_big.append((launch, big, grad, t256))
+            if sum(t for _, _, _, t in self._dw_big) >= self.FULL_GRID - 16:
+                for member, _, _, _ in self._dw_big:
+                    del self.out[next(i for i in range(len(self.out) - 1, -1, -1) if self.out[i] is member)]
+                self.emit(self.k.gemm_group([b for _, b, _, _ in self._dw_big]))
+                self._dw_big = []
+            elif len(self._dw_big) == self.k.GEMM_GROUP_MAX:
+                self._dw_big = []
             return
         held = sum(t for _, _, t in self._dw)
         if self._dw and (self._dw[0][0].variant != launch.variant or held + tiles > self.FULL_GRID
@@ -358,6 +383,7 @@ class BwdCtx:
             self.flush_dw()
 
     def flush_dw(self):
+        self._dw_big = []
         if len(self._dw) == 1:
             self.emit(self._dw[0][0])
         elif self._dw:

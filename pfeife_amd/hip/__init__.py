@@ -326,6 +326,21 @@ class HipKernels:
         launch.colsum_ws = ws
         return ws, 0, nb, d.N
 
+    def gemm_retiled(self, launch, variant):
+        """The same product pinned to another kernel variant (see `pf_gemm_desc.variant`), or None when
+        that variant cannot run it."""
+        d = GemmDesc()
+        ctypes.memmove(ctypes.byref(d), ctypes.byref(launch.desc), ctypes.sizeof(GemmDesc))
+        d.variant = int(variant)
+        name = ctypes.create_string_buffer(128)
+        if self.lib.pf_gemm_variant(byref(d), name, 128) != 0:
+            return None
+        new = self._prep("pf_gemm", (byref(d),), (d, launch))
+        new.variant = name.value.decode()
+        new.flops = launch.flops
+        new.desc = d
+        return new
+
     GEMM_GROUP_MAX = 4
 
     @staticmethod

@@ -846,3 +846,45 @@ def test_gemm_grouped_weight_gradients_bit_exact(hip, dtype):
         torch.testing.assert_close(c1.double(), ref, rtol=2e-3, atol=2e-2)
     with pytest.raises(RuntimeError):
         hip.gemm_group([groups[0][0]])
+
+
+def test_weight_gradients_that_fill_the_device_together_share_a_launch_on_large_tiles(hip, monkeypatch):
+    """Four 2048x2048 weight-gradient products (a decoder layer's attention projections) each fill the
+    device on 128x128 tiles; the backward builder replaces them by ONE launch on 256x256 tiles once the
+    fourth arrives, leaves a set that never completes where it stood, and the values are those of the
+    four separate launches, bit for bit.  PFEIFE_DW_RETILE=0 keeps the separate launches."""
+    from types import SimpleNamespace
+    from pfeife_amd.executor.lowering import BwdCtx
+    from pfeife_amd.hip import dtype_code
+    K, M, N = 4096, 2048, 2048
+    probs = [(rnd((K, M), BF16, 50 + i).cuda(), rnd((K, N), BF16, 60 + i).cuda(), rnd((M, N), F32, 70 + i).cuda())
+             for i in range(4)]
+
+    def build(n):
+        prog = SimpleNamespace(bwd=[])
+        B = BwdCtx(SimpleNamespace(kernels=hip), prog)
+        outs = []
+        for dy, x, c0 in probs[:n]:
+            c = c0.clone()
+            B.emit_dw(hip.gemm(dy, x, c, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1), c)
+            outs.append(c)
+        B.flush_dw()
+        return prog.bwd, outs
+
+    s = torch.cuda.current_stream().cuda_stream
+    one, c_one = build(4)
+    assert len(one) == 1 and one[0].variant.startswith("gemm16x_group_kernel<%d, 256, 256" % dtype_code(BF16))
+    three, c_three = build(3)
+    assert len(three) == 3 and all(l.variant.startswith("gemm16x_kernel<") for l in three)
+    monkeypatch.setenv("PFEIFE_DW_RETILE", "0")
+    four, c_four = build(4)
+    assert len(four) == 4
+    for l in one + three + four:
+        l(s)
+    torch.cuda.synchronize()
+    for i, (dy, x, c0) in enumerate(probs):
+        assert torch.equal(c_one[i], c_four[i])
+        if i < 3:
+            assert torch.equal(c_three[i], c_four[i])
+    torch.testing.assert_close(c_one[0].double(), probs[0][2].double() + probs[0][0].double().t() @ probs[0][1].double(),
+                               rtol=2e-3, atol=5e-2)
