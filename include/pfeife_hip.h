@@ -140,9 +140,11 @@ typedef struct pf_gemm_desc {
 } pf_gemm_desc;
 
 int pf_gemm(const pf_gemm_desc* desc, void* stream);
+#define PF_GEMM_GROUP_MAX 8
 /* n products in as few launches as possible.  Runs of consecutive descriptors that are weight
  * gradients (a_trans = b_trans = 1, 16-bit operands, fp32 C with beta = 1, no epilogue operands,
- * no batch) and resolve to the same kernel instantiation share ONE launch (up to 4 per launch):
+ * no batch) and resolve to the same kernel instantiation share ONE launch (up to PF_GEMM_GROUP_MAX
+ * per launch):
  * dW of a 1024x1024 weight covers only 64 of the 256 CUs on its own.  Everything else is issued
  * as by pf_gemm, in order.  The products of one call must not depend on each other's results.
  * torch.autograd issues the same products one by one (pfeife/mp/worker.py:1585-1587). */

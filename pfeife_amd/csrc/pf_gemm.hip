@@ -811,12 +811,12 @@ extern "C" int pf_gemm_grouped(const pf_gemm_desc* descs, int n, void* stream) {
     if (groupable(descs[i], v0)) {
       run = 1;
       int v = 0;
-      while (i + run < n && run < 4 && descs[i + run].in_dtype == descs[i].in_dtype && groupable(descs[i + run], v) &&
+      while (i + run < n && run < PF_GEMM_GROUP_MAX && descs[i + run].in_dtype == descs[i].in_dtype && groupable(descs[i + run], v) &&
              v == v0)
         ++run;
     }
     if (run >= 2) {
-      pf_gemm_desc d[4];
+      pf_gemm_desc d[PF_GEMM_GROUP_MAX];
       for (int k = 0; k < run; ++k) {
         d[k] = descs[i + k];
         d[k].batch1 = d[k].batch2 = 1;

@@ -583,7 +583,7 @@ __global__ PF_X_BOUNDS void gemm16x_kernel(const pf_gemm_desc p, const GemmGrid 
 // [start[i], start[i+1]).  Weight-gradient products are independent of everything that follows
 // them in a backward job; small ones (64 tiles for a 1024x1024 weight) are launched together so
 // that they fill the 256 CUs.
-constexpr int GEMM_GROUP_MAX = 4;
+constexpr int GEMM_GROUP_MAX = PF_GEMM_GROUP_MAX;   // 8 problems: 2.3 KB of kernel arguments
 struct GemmGroup {
   pf_gemm_desc p[GEMM_GROUP_MAX];
   GemmGrid g[GEMM_GROUP_MAX];

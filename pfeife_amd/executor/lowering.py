@@ -317,7 +317,8 @@ class BwdCtx:
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
         self._dw = []       # held-back weight-gradient products: (launch, accumulator, tiles)
-        self._dw_big = []   # issued ones that fill the device alone: (launch, the same on 256x256 tiles, accumulator, tiles)
+        self._dw_big = []   # issued ones that may yet share a launch on 256x256 tiles:
+                            # (issued launch, its products on that tile, their accumulators, tiles)
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
         self._lp = {}
@@ -344,34 +345,13 @@ class BwdCtx:
             self.emit(launch)
             return
         tiles = self._tiles(launch)
-        if any(g.data_ptr() == grad.data_ptr() for _, g, _ in self._dw + [(None, g2, None) for _, _, g2, _ in self._dw_big]):
+        if any(g.data_ptr() == grad.data_ptr() for _, g, _ in self._dw) or \
+                any(g.data_ptr() == grad.data_ptr() for _, _, gs, _ in self._dw_big for g in gs):
             self.flush_dw()          # two products into one accumulator keep their order
+            self._dw_big = []
         if tiles >= self.FULL_GRID:
-            # Fills the device on its own with small tiles.  Four such products whose 256x256 tiles fill it
-            # TOGETHER (a decoder's four 2048x2048 attention projections: 64 tiles each) run faster as one
-            # launch on the large tile, which moves half the operand bytes per FLOP through LDS.  Each is
-            # issued where it stands and remembered; only when the set is complete do its members give
-            # way to the one launch, at the place of the last (a set that never completes costs nothing).
             self.emit(launch)
-            d = launch.desc
-            t256 = ((d.M + 255) // 256) * ((d.N + 255) // 256)
-            retile = getattr(self.k, "gemm_retiled", None) if os.environ.get("PFEIFE_DW_RETILE", "1") != "0" else None
-            big = retile(launch, 1) if (retile is not None and t256 * 2 <= self.FULL_GRID
-                                        and not launch.variant.startswith("gemm16x_kernel<%d, 256, 256" % d.in_dtype)) else None
-            if big is None or not groupable(big):
-                self._dw_big = []
-                return
-            if self._dw_big and (self._dw_big[0][1].variant != big.variant
-                                 or sum(t for _, _, _, t in self._dw_big) + t256 > self.FULL_GRID):
-                self._dw_big = []
-            self._dw_big.append((launch, big, grad, t256))
-            if sum(t for _, _, _, t in self._dw_big) >= self.FULL_GRID - 16:
-                for member, _, _, _ in self._dw_big:
-                    del self.out[next(i for i in range(len(self.out) - 1, -1, -1) if self.out[i] is member)]
-                self.emit(self.k.gemm_group([b for _, b, _, _ in self._dw_big]))
-                self._dw_big = []
-            elif len(self._dw_big) == self.k.GEMM_GROUP_MAX:
-                self._dw_big = []
+            self._offer_big(launch, [(launch, grad)])
             return
         held = sum(t for _, _, t in self._dw)
         if self._dw and (self._dw[0][0].variant != launch.variant or held + tiles > self.FULL_GRID
@@ -382,12 +362,47 @@ class BwdCtx:
         if held + tiles >= self.FULL_GRID - 32:
             self.flush_dw()
 
+    def _offer_big(self, issued, members):
+        """`issued` (one launch, already in the job) computes `members`: (product, accumulator) pairs.
+        Products that fill the device on 128x128 tiles, alone or a few together, run faster on 256x256
+        tiles, which move half the operand bytes per FLOP through LDS, but then cover only part of it (a
+        decoder's 2048x2048 attention projections and ViT-L's 1024x4096 MLP weights: 64 tiles each).  So
+        every such launch is issued where it stands and remembered; once the remembered products give
+        nearly every CU a 256x256 tile they all give way to ONE launch on that tile, at the place of the
+        last.  A set that never completes costs nothing, and the sums are the same bit for bit (the tile
+        does not change the order in which a product is summed)."""
+        retile = getattr(self.k, "gemm_retiled", None)
+        if retile is None or os.environ.get("PFEIFE_DW_RETILE", "1") == "0":
+            return
+        bigs, t256 = [], 0
+        for launch, _ in members:
+            d = launch.desc
+            big = launch if launch.variant.startswith("gemm16x_kernel<%d, 256, 256" % d.in_dtype) else retile(launch, 1)
+            if big is None or not self.k.gemm_groupable(big):
+                return
+            bigs.append(big)
+            t256 += ((d.M + 255) // 256) * ((d.N + 255) // 256)
+        if t256 * 2 > self.FULL_GRID:
+            return                   # covers most of the device on the large tile by itself
+        if self._dw_big and (self._dw_big[0][1][0].variant != bigs[0].variant
+                             or sum(t for _, _, _, t in self._dw_big) + t256 > self.FULL_GRID
+                             or sum(len(b) for _, b, _, _ in self._dw_big) + len(bigs) > self.k.GEMM_GROUP_MAX):
+            self._dw_big = []
+        self._dw_big.append((issued, bigs, [g for _, g in members], t256))
+        if sum(t for _, _, _, t in self._dw_big) >= self.FULL_GRID - 16 and len(self._dw_big) >= 2:
+            for old, _, _, _ in self._dw_big:
+                del self.out[next(i for i in range(len(self.out) - 1, -1, -1) if self.out[i] is old)]
+            self.emit(self.k.gemm_group([b for _, bs, _, _ in self._dw_big for b in bs]))
+            self._dw_big = []
+
     def flush_dw(self):
-        self._dw_big = []
         if len(self._dw) == 1:
             self.emit(self._dw[0][0])
+            self._offer_big(self._dw[0][0], [(self._dw[0][0], self._dw[0][1])])
         elif self._dw:
-            self.emit(self.k.gemm_group([l for l, _, _ in self._dw]))
+            group = self.k.gemm_group([l for l, _, _ in self._dw])
+            self.emit(group)
+            self._offer_big(group, [(l, g) for l, g, _ in self._dw])
         self._dw = []
 
     def register_lp(self, full, copy, colsum=None):

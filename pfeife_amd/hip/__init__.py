@@ -341,7 +341,7 @@ class HipKernels:
         new.desc = d
         return new
 
-    GEMM_GROUP_MAX = 4
+    GEMM_GROUP_MAX = 8      # PF_GEMM_GROUP_MAX
 
     @staticmethod
     def gemm_groupable(launch):

@@ -848,6 +848,48 @@ def test_gemm_grouped_weight_gradients_bit_exact(hip, dtype):
         hip.gemm_group([groups[0][0]])
 
 
+def test_weight_gradients_of_mixed_sizes_regroup_on_large_tiles(hip, monkeypatch):
+    """An encoder's weight gradients in backward order (two 1024x4096 MLP weights that fill the device
+    alone on 128x128 tiles, then the 1024x1024 projection and the 3072x1024 qkv weight that are held
+    back to fill it together, then the next layer's MLP weight): 64 + 64 + (16 + 48) + 64 tiles of
+    256x256, so the fifth product completes the set and the job holds ONE launch.  Token count 1576:
+    the reduction ends inside a tile.  Values equal those of the launches it replaced, bit for bit."""
+    from types import SimpleNamespace
+    from pfeife_amd.executor.lowering import BwdCtx
+    from pfeife_amd.hip import dtype_code
+    K = 1576
+    shapes = [(1024, 4096), (4096, 1024), (1024, 1024), (3072, 1024), (1024, 4096), (4096, 1024)]
+    probs = [(rnd((K, M), F16, 80 + i).cuda(), rnd((K, N), F16, 90 + i).cuda(), rnd((M, N), F32, 100 + i).cuda())
+             for i, (M, N) in enumerate(shapes)]
+
+    def build():
+        prog = SimpleNamespace(bwd=[])
+        B = BwdCtx(SimpleNamespace(kernels=hip), prog)
+        outs = []
+        for dy, x, c0 in probs:
+            c = c0.clone()
+            M, N = c.shape
+            B.emit_dw(hip.gemm(dy, x, c, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1), c)
+            outs.append(c)
+        B.flush_dw()
+        return prog.bwd, outs
+
+    new, c_new = build()
+    assert [l.variant.split("<")[0] for l in new] == ["gemm16x_group_kernel", "gemm16x_kernel"]
+    assert new[0].variant.startswith("gemm16x_group_kernel<%d, 256, 256" % dtype_code(F16))
+    monkeypatch.setenv("PFEIFE_DW_RETILE", "0")
+    old, c_old = build()
+    assert len(old) == 5       # projection and qkv share a launch on 128x128 tiles
+    s = torch.cuda.current_stream().cuda_stream
+    for l in new + old:
+        l(s)
+    torch.cuda.synchronize()
+    for a, b in zip(c_new, c_old):
+        assert torch.equal(a, b)
+    dy, x, c0 = probs[3]
+    torch.testing.assert_close(c_new[3].double(), c0.double() + dy.double().t() @ x.double(), rtol=2e-3, atol=2e-2)
+
+
 def test_weight_gradients_that_fill_the_device_together_share_a_launch_on_large_tiles(hip, monkeypatch):
     """Four 2048x2048 weight-gradient products (a decoder layer's attention projections) each fill the
     device on 128x128 tiles; the backward builder replaces them by ONE launch on 256x256 tiles once the
