@@ -317,7 +317,7 @@ class BwdCtx:
         self._pending = {}
         self.reduces = []   # deferred column reductions, finished by one batched launch at the end
         self._dw = []       # held-back weight-gradient products: (launch, accumulator, tiles)
-        self._dw_big = []   # issued ones that may yet share a launch on 256x256 tiles:
+        self._dw_big = []   # open sets of issued ones that may yet share a launch on 256x256 tiles, each a list of
                             # (issued launch, its products on that tile, their accumulators, tiles)
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
@@ -328,6 +328,7 @@ class BwdCtx:
 
     # -- weight-gradient products that share a launch ---------------------------------------------
     FULL_GRID = 256     # workgroups that fill the device (one tile per CU)
+    OPEN_SETS = 4       # sets of issued weight-gradient products that may yet share a launch on 256x256 tiles
 
     @staticmethod
     def _tiles(launch):
@@ -346,7 +347,7 @@ class BwdCtx:
             return
         tiles = self._tiles(launch)
         if any(g.data_ptr() == grad.data_ptr() for _, g, _ in self._dw) or \
-                any(g.data_ptr() == grad.data_ptr() for _, _, gs, _ in self._dw_big for g in gs):
+                any(g.data_ptr() == grad.data_ptr() for entries in self._dw_big for _, _, gs, _ in entries for g in gs):
             self.flush_dw()          # two products into one accumulator keep their order
             self._dw_big = []
         if tiles >= self.FULL_GRID:
@@ -382,18 +383,28 @@ class BwdCtx:
                 return
             bigs.append(big)
             t256 += ((d.M + 255) // 256) * ((d.N + 255) // 256)
-        if t256 * 2 > self.FULL_GRID:
-            return                   # covers most of the device on the large tile by itself
-        if self._dw_big and (self._dw_big[0][1][0].variant != bigs[0].variant
-                             or sum(t for _, _, _, t in self._dw_big) + t256 > self.FULL_GRID
-                             or sum(len(b) for _, b, _, _ in self._dw_big) + len(bigs) > self.k.GEMM_GROUP_MAX):
-            self._dw_big = []
-        self._dw_big.append((issued, bigs, [g for _, g in members], t256))
-        if sum(t for _, _, _, t in self._dw_big) >= self.FULL_GRID - 16 and len(self._dw_big) >= 2:
-            for old, _, _, _ in self._dw_big:
+        if t256 > self.FULL_GRID - 32:
+            return                   # nothing worth its launch fits beside it
+        # best fit over a few open sets: the fullest one that still takes it (a decoder's 5632x2048 MLP
+        # weights, 176 tiles each, are each completed by one of the 64-tile attention projections)
+        mine = None
+        for entries in self._dw_big:
+            held = sum(t for _, _, _, t in entries)
+            if entries[0][1][0].variant == bigs[0].variant and held + t256 <= self.FULL_GRID \
+                    and sum(len(b) for _, b, _, _ in entries) + len(bigs) <= self.k.GEMM_GROUP_MAX \
+                    and (mine is None or held > sum(t for _, _, _, t in mine)):
+                mine = entries
+        if mine is None:
+            mine = []
+            self._dw_big.append(mine)
+            if len(self._dw_big) > self.OPEN_SETS:
+                self._dw_big.pop(0)  # the oldest stays as it was issued
+        mine.append((issued, bigs, [g for _, g in members], t256))
+        if sum(t for _, _, _, t in mine) >= self.FULL_GRID - 56 and len(mine) >= 2:
+            for old, _, _, _ in mine:
                 del self.out[next(i for i in range(len(self.out) - 1, -1, -1) if self.out[i] is old)]
-            self.emit(self.k.gemm_group([b for _, bs, _, _ in self._dw_big for b in bs]))
-            self._dw_big = []
+            self.emit(self.k.gemm_group([b for _, bs, _, _ in mine for b in bs]))
+            self._dw_big.remove(mine)
 
     def flush_dw(self):
         if len(self._dw) == 1:
