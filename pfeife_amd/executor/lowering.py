@@ -379,8 +379,8 @@ class BwdCtx:
         for launch, _ in members:
             d = launch.desc
             big = launch if launch.variant.startswith("gemm16x_kernel<%d, 256, 256" % d.in_dtype) else retile(launch, 1)
-            if big is None or not self.k.gemm_groupable(big):
-                return
+            if d.M < 256 or d.N < 256 or big is None or not self.k.gemm_groupable(big):
+                return               # less than one full tile either way: stays on the small tile
             bigs.append(big)
             t256 += ((d.M + 255) // 256) * ((d.N + 255) // 256)
         if t256 > self.FULL_GRID - 32:
