@@ -398,13 +398,35 @@ class BwdCtx:
             mine = []
             self._dw_big.append(mine)
             if len(self._dw_big) > self.OPEN_SETS:
-                self._dw_big.pop(0)  # the oldest stays as it was issued
+                self._close_set(self._dw_big[0])     # the oldest has waited long enough
         mine.append((issued, bigs, [g for _, g in members], t256))
-        if sum(t for _, _, _, t in mine) >= self.FULL_GRID - 56 and len(mine) >= 2:
-            for old, _, _, _ in mine:
-                del self.out[next(i for i in range(len(self.out) - 1, -1, -1) if self.out[i] is old)]
-            self.emit(self.k.gemm_group([b for _, bs, _, _ in mine for b in bs]))
-            self._dw_big.remove(mine)
+        if sum(t for _, _, _, t in mine) >= self.FULL_GRID - 56:
+            self._close_set(mine)
+
+    def _close_set(self, entries):
+        """Two or more remembered launches that cover half the device or more on 256x256 tiles give way to
+        one launch on that tile, here; anything less stays as it was issued."""
+        self._dw_big.remove(entries)
+        if len(entries) >= 2 and sum(t for _, _, _, t in entries) >= self.FULL_GRID // 2:
+            for old, _, _, _ in entries:   # blanked, not deleted: positions in the list stay valid until compact()
+                self.out[next(i for i in range(len(self.out) - 1, -1, -1) if self.out[i] is old)] = None
+            self.emit(self.k.gemm_group([b for _, bs, _, _ in entries for b in bs]))
+
+    def compact(self, ranges):
+        """Drop the blanked launches; `ranges` ((name, first, end) over the list) follow."""
+        new, n = [], 0
+        for launch in self.out:
+            new.append(n)
+            n += launch is not None
+        new.append(n)
+        self.out[:] = [launch for launch in self.out if launch is not None]
+        ranges[:] = [(name, new[a], new[b]) for name, a, b in ranges]
+
+    def close_dw(self):
+        """End of the job: nothing more will arrive."""
+        self.flush_dw()
+        while self._dw_big:
+            self._close_set(self._dw_big[0])
 
     def flush_dw(self):
         if len(self._dw) == 1:
@@ -686,11 +708,12 @@ class Lowerer:
             fn(B)
             prog.bwd_ranges.append((name, first, len(prog.bwd)))
         first = len(prog.bwd)
-        B.flush_dw()
+        B.close_dw()
         if B.reduces:
             prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
         if prog.bwd_ranges and len(prog.bwd) > first:   # held-back tail: charged to the job's last node
             prog.bwd_ranges.append((prog.bwd_ranges[-1][0], first, len(prog.bwd)))
+        B.compact(prog.bwd_ranges)
         prog.input_grads = []
         for v in prog.inputs:
             if isinstance(v, Val) and v.req_grad and v.param is None:

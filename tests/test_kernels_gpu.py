@@ -871,7 +871,10 @@ def test_weight_gradients_of_mixed_sizes_regroup_on_large_tiles(hip, monkeypatch
             M, N = c.shape
             B.emit_dw(hip.gemm(dy, x, c, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1), c)
             outs.append(c)
-        B.flush_dw()
+        B.close_dw()
+        ranges = [("all", 0, len(prog.bwd))]
+        B.compact(ranges)
+        assert ranges == [("all", 0, len(prog.bwd))] and None not in prog.bwd
         return prog.bwd, outs
 
     new, c_new = build()
@@ -893,7 +896,7 @@ def test_weight_gradients_of_mixed_sizes_regroup_on_large_tiles(hip, monkeypatch
 def test_weight_gradients_that_fill_the_device_together_share_a_launch_on_large_tiles(hip, monkeypatch):
     """Four 2048x2048 weight-gradient products (a decoder layer's attention projections) each fill the
     device on 128x128 tiles; the backward builder replaces them by ONE launch on 256x256 tiles once the
-    fourth arrives, leaves a set that never completes where it stood, and the values are those of the
+    fourth arrives (at the end of a job, with what has arrived if that covers half the device), and the values are those of the
     four separate launches, bit for bit.  PFEIFE_DW_RETILE=0 keeps the separate launches."""
     from types import SimpleNamespace
     from pfeife_amd.executor.lowering import BwdCtx
@@ -910,14 +913,18 @@ def test_weight_gradients_that_fill_the_device_together_share_a_launch_on_large_
             c = c0.clone()
             B.emit_dw(hip.gemm(dy, x, c, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1), c)
             outs.append(c)
-        B.flush_dw()
+        B.close_dw()
+        ranges = [("all", 0, len(prog.bwd))]
+        B.compact(ranges)
+        assert ranges == [("all", 0, len(prog.bwd))] and None not in prog.bwd
         return prog.bwd, outs
 
     s = torch.cuda.current_stream().cuda_stream
     one, c_one = build(4)
     assert len(one) == 1 and one[0].variant.startswith("gemm16x_group_kernel<%d, 256, 256" % dtype_code(BF16))
-    three, c_three = build(3)
-    assert len(three) == 3 and all(l.variant.startswith("gemm16x_kernel<") for l in three)
+    three, c_three = build(3)    # end of the job: three cover 192 CUs together, still better than one after another
+    assert len(three) == 1 and three[0].variant.startswith("gemm16x_group_kernel<")
+    assert [l.variant.split("<")[0] for l in build(1)[0]] == ["gemm16x_kernel"]
     monkeypatch.setenv("PFEIFE_DW_RETILE", "0")
     four, c_four = build(4)
     assert len(four) == 4
