@@ -370,8 +370,8 @@ class BwdCtx:
         decoder's 2048x2048 attention projections and ViT-L's 1024x4096 MLP weights: 64 tiles each).  So
         every such launch is issued where it stands and remembered; once the remembered products give
         nearly every CU a 256x256 tile they all give way to ONE launch on that tile, at the place of the
-        last.  A set that never completes costs nothing, and the sums are the same bit for bit (the tile
-        does not change the order in which a product is summed)."""
+        last.  Members of a set that is dropped stay as they were issued, and the sums are the same bit
+        for bit either way (the tile does not change the order in which a product is summed)."""
         retile = getattr(self.k, "gemm_retiled", None)
         if retile is None or os.environ.get("PFEIFE_DW_RETILE", "1") == "0":
             return
