@@ -274,7 +274,7 @@ def cpu_baseline(name):
     import torch.nn.functional as F
 
     from oracle.stage_oracle import run_pipeline_step
-    from pfeife_amd.bench_models import llama, vit
+    from pfeife_amd.bench_models import llama, unet_stage, vit
 
     family, cfg_name, batch, batch_cnt, splits, device_cnt, mixed = WORKLOADS[name]
     cores = os.cpu_count() or 1
@@ -284,7 +284,7 @@ def cpu_baseline(name):
     torch.set_num_threads(cores)
     torch.manual_seed(42)
     g = torch.Generator().manual_seed(42)
-    cnt = 2
+    cnt, passes = 2, 2
     if family == "vit":
         cfg = getattr(vit, cfg_name)
         model = vit.VisionTransformer(cfg)
@@ -303,7 +303,25 @@ def cpu_baseline(name):
         loss_fn = lambda o, t: (o * t).sum()
         unit, per_sample = "samples/s", 1
     elif family == "unet":
-        raise RuntimeError("no CPU baseline leg for the UNet stage workload (run with --no-cpu-baseline)")
+        cfg = getattr(unet_stage, cfg_name)
+        stage = unet_stage.UNetStage(cfg)
+        mb, cnt, passes = 1, 1, 1     # one sample, one pass (2e13 FLOPs: tens of seconds on the host cores)
+        temb = torch.randn(mb, cfg.temb_dim, generator=g)
+        ctx = torch.randn(mb, 77, cfg.context_dim, generator=g)
+
+        class OneInput(nn.Module):     # the stage executor hands one tensor from stage to stage
+            def __init__(self):
+                super().__init__()
+                self.stage = stage
+
+            def forward(self, hidden):
+                return self.stage(hidden, temb, ctx)
+
+        stages = [OneInput()]
+        x = torch.randn(mb * cnt, cfg.in_channels, 32, 32, generator=g)
+        y = torch.randn(mb * cnt, cfg.channels, 32, 32, generator=g)
+        loss_fn = lambda o, t: F.mse_loss(o.float(), t.float())
+        unit, per_sample = "samples/s", 1
     else:
         cfg = getattr(llama, cfg_name)
         model = llama.LlamaForCausalLM(cfg)
@@ -314,12 +332,16 @@ def cpu_baseline(name):
         loss_fn = lambda lg, t: F.cross_entropy(lg[:, :-1].reshape(-1, lg.shape[-1]), t[:, 1:].reshape(-1))
         unit, per_sample = "samples/s (sequences of 2048 tokens; measured tokens/s / 2048)", T / float(cfg.max_seq)
     times = []
-    for _ in range(2):  # first pass warms the allocator and the thread pool
+    for _ in range(passes):  # with two passes the first warms the allocator and the thread pool
         t0 = time.perf_counter()
         run_pipeline_step(stages, loss_fn, x, y, cnt, device_cnt=device_cnt)
         times.append(time.perf_counter() - t0)
     sps = mb * cnt * per_sample / times[-1]
     return dict(value=round(sps, 4), unit=unit, cores=cores, kind="port",
+                # the CPU sample is SMALLER than the GPU step: do not divide `value` fields by each other
+                # without these (GPU step: the workload's micro_batch x batch_cnt, with the optimizer step)
+                micro_batch=mb, batch_cnt=cnt, optimizer_step=False, precision="fp32",
+                gpu_step_micro_batch=batch // batch_cnt, gpu_step_batch_cnt=batch_cnt,
                 sample="%s fp32 on CPU: %d micro-batches x %d samples, %d stages, forward+backward+grad-accumulate "
                        "(no optimizer step), oracle stage executor; %.1f s%s" % (
                            cfg_name, cnt, mb, len(stages), times[-1],
@@ -420,6 +442,26 @@ def torch_eager_gpu(name, device, steps=5, warmup=2):
                            "on" if mixed == "fp16" else "off", last))
 
 
+def unet_stage_forward_flops(cfg, hw=32, ctx_tokens=77):
+    """Algorithmic forward FLOPs per sample of bench_models/unet_stage.UNetStage, layer by layer
+    (2 x rows x in x out per linear layer / convolution tap, 4 x Tq x Tk x dim per attention)."""
+    T, c, cin = hw * hw, cfg.channels, cfg.in_channels
+    lin = lambda rows, i, o: 2.0 * rows * i * o
+
+    def resnet(ci, co):
+        f = lin(T, 9 * ci, co) + lin(T, 9 * co, co) + lin(1, cfg.temb_dim, co)   # conv1, conv2 (3x3), time embedding
+        return f + (lin(T, ci, co) if ci != co else 0.0)                          # 1x1 shortcut
+
+    def block():
+        self_attn = 4 * lin(T, c, c) + 4.0 * T * T * c                            # q, k, v, out + QK^T, PV
+        cross = 2 * lin(T, c, c) + 2 * lin(ctx_tokens, cfg.context_dim, c) + 4.0 * T * ctx_tokens * c
+        ff = lin(T, c, 2 * cfg.ff_mult * c) + lin(T, cfg.ff_mult * c, c)          # GEGLU projection, output
+        return self_attn + cross + ff
+
+    transformer = 2 * lin(T, c, c) + cfg.layers * block()                         # proj_in, proj_out + blocks
+    return resnet(cin, c) + resnet(c, c) + 2 * transformer + resnet(c, c) + transformer + resnet(c, c)
+
+
 def model_flops_per_step(info):
     cfg, samples = info["cfg"], info["batch"]
     if info["family"] in ("vit", "vit_share"):
@@ -430,7 +472,7 @@ def model_flops_per_step(info):
             extra = 2 * (T - 1) * (cfg.channels * cfg.patch_size ** 2) * d + 2 * d * cfg.num_classes
         return 3.0 * samples * (L * per_block + extra)
     if info["family"] == "unet":
-        return None
+        return 3.0 * samples * unet_stage_forward_flops(cfg)
     T, d, ff, L, V = cfg.max_seq, cfg.dim, cfg.ffn, cfg.layers, cfg.vocab
     per_tok = L * (8 * d * d + 6 * d * ff + 4 * T * d) + 2 * d * V
     return 3.0 * samples * T * per_tok
@@ -587,7 +629,10 @@ def main():
     cpu = None
     if not args.no_cpu_baseline:
         log("[bench] timing the CPU baseline ...")
-        cpu = cpu_baseline(args.workload)
+        try:
+            cpu = cpu_baseline(args.workload)
+        except Exception as e:   # report, do not lose the headline line
+            cpu = dict(skipped="failed: %s" % (str(e)[:200],))
         log("[bench] cpu baseline", cpu)
 
     # the other single-GPU configurations, for a bounded number of steps each (reported next to the

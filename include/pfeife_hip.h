@@ -128,8 +128,9 @@ typedef struct pf_gemm_desc {
   int64_t ld_res;
   int32_t res_dtype;
   int32_t variant; /* 0: automatic tile choice; otherwise one kernel variant by id (tuning
-                      harnesses): 1..3 direct-to-LDS kernel with 256x256 / 256x128 / 128x128
-                      tiles, 11..14 register-staged kernel with 128x128 (8 wavefronts),
+                      harnesses): 1..6 direct-to-LDS kernel with 256x256 / 256x128 / 128x128 /
+                      192x256 tiles and the two-workgroups-per-CU 128x128 / 256x128 tiles
+                      (32-deep stages), 11..14 register-staged kernel with 128x128 (8 wavefronts),
                       128x128, 128x64, 64x64 tiles; PF_ERR_INVALID if it cannot run the problem */
   float* colsum_ws; /* optional, with dact on the direct-to-LDS kernel (pf_gemm_variant ends in ", 5>"): the
                        launch also leaves the column sums of the 16-bit values it stores in C as partial

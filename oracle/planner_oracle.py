@@ -14,6 +14,11 @@ Restates
     sum over the rank's job list that starts at the rank's weights, adds a stage's activation
     memory at its forward, releases it at its backward, and peaks by the stage's temporary memory.
 
+  * `PipeSchedSet._build_set`   (pfeife/schedule/scheduler.py:130-151): the (loop_batch,
+    prefetch_fwd) pairs valued per stage count, and the stage counts of
+    `PipeGraphGenerator.gen_graph` (pfeife/schedule/planner.py:667-670): `loop_cnt * device_cnt`,
+    else 1x, 2x, 3x `device_cnt`; pinned by hand-enumerated sets in tests/test_planner.py.
+
 What pins it (tests/test_planner.py): closed forms of the one-forward-one-backward pipeline
 with equal stages ((B + D - 1)(f + b) + optimizer), the single-stage sum, a hand-worked
 two-stage case with unequal stages and a transfer time, and a hand-worked memory trace.
@@ -106,4 +111,33 @@ def brute_force_points(candidates, n_cuts, value_fn):
         v = value_fn(list(pts))
         if best is None or v < best[0]:
             best = (v, list(pts))
+    return best
+
+
+def sched_set(device_cnt, batch_cnt, node_cnt):
+    """[(loop_batch, prefetch_fwd)] of pfeife/schedule/scheduler.py:130-151, in its order."""
+    out = []
+    if node_cnt > device_cnt:
+        for loop_batch in range(device_cnt, batch_cnt + 1):
+            if loop_batch > device_cnt and batch_cnt % loop_batch != 0:
+                continue
+            for prefetch_fwd in range(0, device_cnt):
+                out.append((loop_batch, prefetch_fwd))
+    else:
+        for prefetch_fwd in range(0, device_cnt):
+            out.append((batch_cnt, prefetch_fwd))
+    return out
+
+
+def brute_force_plan(candidates, stage_counts, variants_of, value_fn):
+    """The best of ALL (stage count, schedule variant, increasing split points): variants_of(cnt) ->
+    [(loop_batch, prefetch_fwd)], value_fn(points, cnt, loop_batch, prefetch_fwd) -> time or None
+    (None: the variant cannot be run)."""
+    best = None
+    for cnt in stage_counts:
+        for lb, pf in variants_of(cnt):
+            for pts in itertools.combinations(candidates, cnt - 1):
+                v = value_fn(list(pts), cnt, lb, pf)
+                if v is not None and (best is None or v < best[0]):
+                    best = (v, list(pts), cnt, lb, pf)
     return best

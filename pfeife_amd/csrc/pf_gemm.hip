@@ -15,11 +15,22 @@
 //   the parity path, not the throughput path).
 #include "pf_gemm_common.h"
 
-// direct-to-LDS kernels, one translation unit per operand dtype
-int pf_gemm_x_f16(const pf_gemm_desc& d, int tile, hipStream_t st);
-int pf_gemm_x_bf16(const pf_gemm_desc& d, int tile, hipStream_t st);
-int pf_gemm_xgroup_f16(const pf_gemm_desc* d, int n, int tile, hipStream_t st);
-int pf_gemm_xgroup_bf16(const pf_gemm_desc* d, int n, int tile, hipStream_t st);
+// direct-to-LDS kernels, one object file per (operand dtype id, tile id): pf_gemm_x_inst.hip
+#define PF_X_DECL(DT, XT)                                              \
+  int pf_gemm_x_##DT##_##XT(const pf_gemm_desc& d, hipStream_t st);    \
+  int pf_gemm_xgroup_##DT##_##XT(const pf_gemm_desc* d, int n, hipStream_t st);
+#define PF_X_DECL_DT(DT) PF_X_DECL(DT, 1) PF_X_DECL(DT, 2) PF_X_DECL(DT, 3) PF_X_DECL(DT, 4) PF_X_DECL(DT, 5) PF_X_DECL(DT, 6)
+PF_X_DECL_DT(1)
+PF_X_DECL_DT(2)
+#undef PF_X_DECL_DT
+#undef PF_X_DECL
+static_assert(PF_F16 == 1 && PF_BF16 == 2 && PF_XT_COUNT == 7, "the table below is written out for these ids");
+typedef int (*pf_x_fn)(const pf_gemm_desc&, hipStream_t);
+typedef int (*pf_xgroup_fn)(const pf_gemm_desc*, int, hipStream_t);
+#define PF_X_ROW(P, DT) {nullptr, P##DT##_1, P##DT##_2, P##DT##_3, P##DT##_4, P##DT##_5, P##DT##_6}
+static const pf_x_fn pf_x_table[3][PF_XT_COUNT] = {{}, PF_X_ROW(pf_gemm_x_, 1), PF_X_ROW(pf_gemm_x_, 2)};
+static const pf_xgroup_fn pf_xgroup_table[3][PF_XT_COUNT] = {{}, PF_X_ROW(pf_gemm_xgroup_, 1), PF_X_ROW(pf_gemm_xgroup_, 2)};
+#undef PF_X_ROW
 
 namespace {
 
@@ -604,9 +615,11 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
 }
 
 // Variant ids (pf_gemm_desc.variant; 0 = automatic):
-//   1..4   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128 / 192x256
+//   1..6   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128 / 192x256 / 128x128d / 256x128d
 //   11..14 register-staged kernel: 128x128 by 8 wavefronts, 128x128, 128x64, 64x64 by 4
-enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_X192x256 = 4, V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
+enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_X192x256 = 4, V_X128D = 5, V_X256x128D = 6,
+       V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
+inline bool is_x_variant(int v) { return v >= V_X256 && v <= V_X256x128D; }
 
 // Register-staged tiles: 128x128 with two workgroups resident per CU is the largest that keeps
 // accumulators, two sets of staging registers and fragments in the register file; smaller tiles
@@ -627,7 +640,7 @@ int choose_staged(const pf_gemm_desc& d) {
 // reduction-contiguous or both reduction-strided; a ragged reduction tail is zero-filled by the
 // hardware range check only in the second case (whole k-rows fall outside the operand).
 bool x_supports(const pf_gemm_desc& d, int xt) {
-  const int bk = (xt == PF_XT_256x256 || xt == PF_XT_192x256) ? 32 : 64;
+  const int bk = x_tile_bk(xt);
   if (xt == PF_XT_192x256 && d.a_trans) return false;   // no reduction-strided 192-row tile
   if (d.a_trans != d.b_trans) return false;
   if (!d.a_trans && d.K % bk != 0) return false;
@@ -658,27 +671,46 @@ int choose_variant(const pf_gemm_desc& d) {
   return best < 0 ? choose_staged(d) : best;
 }
 
-int resolve_variant(const pf_gemm_desc& d) { return d.variant == V_AUTO ? choose_variant(d) : d.variant; }
+// PF_GEMM_TILE_MAP="3:5,1:6": the automatic choice's tile 3 runs as tile 5, tile 1 as tile 6 (where the
+// replacement supports the problem); a measurement aid, read once.
+int remap_variant(const pf_gemm_desc& d, int v) {
+  static int map[PF_XT_COUNT];
+  static std::once_flag once;
+  std::call_once(once, [] {
+    for (int i = 0; i < PF_XT_COUNT; ++i) map[i] = i;
+    const char* e = getenv("PF_GEMM_TILE_MAP");
+    while (e && *e) {
+      int a = 0, b = 0, used = 0;
+      if (sscanf(e, "%d:%d%n", &a, &b, &used) == 2 && a > 0 && a < PF_XT_COUNT && b > 0 && b < PF_XT_COUNT) map[a] = b;
+      e += used > 0 ? used : 1;
+      while (*e == ',' || *e == ' ') ++e;
+    }
+  });
+  if (!is_x_variant(v)) return v;
+  const int w = map[v];
+  return (w != v && x_supports(d, w)) ? w : v;
+}
+
+int resolve_variant(const pf_gemm_desc& d) { return d.variant == V_AUTO ? remap_variant(d, choose_variant(d)) : d.variant; }
 
 template <int DT>
 int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
   const int v = resolve_variant(d);
   if (d.colsum_ws != nullptr) {   // only the GELU' class of the direct-to-LDS kernel sums its columns
-    const bool xk = v == V_X256 || v == V_X256x128 || v == V_X128 || v == V_X192x256;
-    if (!xk || d.a_trans || d.b_trans || !x_supports(d, v) || epi_class(d, epi_vec_ok(d)) != EC_DACT16 ||
+    if (!is_x_variant(v) || d.a_trans || d.b_trans || !x_supports(d, v) || epi_class(d, epi_vec_ok(d)) != EC_DACT16 ||
         !pf_aligned(d.colsum_ws, 16)) {
       pf_set_error("pf_gemm: colsum_ws needs a 16-bit product with the GELU' epilogue on the direct-to-LDS kernel");
       return PF_ERR_UNSUPPORTED;
     }
   }
   switch (v) {
-    case V_X256: case V_X256x128: case V_X128: case V_X192x256: {
-      const int xt = v;   // variant ids 1..5 are the PF_XT_* tile ids
+    case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128D: case V_X256x128D: {
+      const int xt = v;   // variant ids 1..6 are the PF_XT_* tile ids
       if (!x_supports(d, xt)) {
         pf_set_error("pf_gemm: variant %d needs both operands stored alike and (unless transposed) K a multiple of the stage depth", v);
         return PF_ERR_INVALID;
       }
-      return DT == PF_F16 ? pf_gemm_x_f16(d, xt, st) : pf_gemm_x_bf16(d, xt, st);
+      return pf_x_table[DT][xt](d, st);
     }
     case V_R128W8: return launch16<DT, 128, 128, 64, 4, 2>(d, st);
     case V_R128: return launch16<DT, 128, 128, 64, 2, 2>(d, st);
@@ -796,7 +828,7 @@ bool groupable(const pf_gemm_desc& d, int& variant) {
   const int64_t a_bytes = (d.K + 256) * d.lda * 2, b_bytes = (d.K + 256) * d.ldb * 2;
   if (a_bytes >= (1ll << 31) || b_bytes >= (1ll << 31)) return false;
   variant = resolve_variant(d);
-  if (variant != V_X256 && variant != V_X256x128 && variant != V_X128) return false;
+  if (!is_x_variant(variant) || variant == V_X192x256) return false;
   if (!x_supports(d, variant)) return false;
   return epi_class(d, epi_vec_ok(d)) == EC_ACC32;
 }
@@ -821,8 +853,7 @@ extern "C" int pf_gemm_grouped(const pf_gemm_desc* descs, int n, void* stream) {
         d[k] = descs[i + k];
         d[k].batch1 = d[k].batch2 = 1;
       }
-      const int rc = descs[i].in_dtype == PF_F16 ? pf_gemm_xgroup_f16(d, run, v0, (hipStream_t)stream)
-                                                 : pf_gemm_xgroup_bf16(d, run, v0, (hipStream_t)stream);
+      const int rc = pf_xgroup_table[descs[i].in_dtype][v0](d, run, (hipStream_t)stream);
       if (rc != PF_OK) return rc;
       i += run;
     } else {
@@ -849,9 +880,14 @@ extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   const char* bt = d.b_trans ? "true" : "false";
   const int v = resolve_variant(d);
   switch (v) {
-    case V_X256: case V_X256x128: case V_X128: case V_X192x256: {
+    case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128D: case V_X256x128D: {
       static const char* shapes[PF_XT_COUNT] = {"", "256, 256, 32, 2, 2, 5", "256, 128, 64, 2, 2, 3", "128, 128, 64, 2, 2, 3",
-                                                "192, 256, 32, 2, 2, 5"};
+                                                "192, 256, 32, 2, 2, 5", "128, 128, 32, 2, 2, 4", "256, 128, 32, 2, 2, 3"};
+      if (!x_supports(d, v)) {   // a pinned tile that cannot run this product: say so here, not at launch time
+        pf_set_error("pf_gemm_variant: variant %d needs both operands stored alike, K >= %d and (unless both are "
+                     "reduction-strided) K a multiple of %d", v, x_tile_bk(v), x_tile_bk(v));
+        return PF_ERR_INVALID;
+      }
       int ec = epi_class(d, epi_vec_ok(d));
       if (d.a_trans && ec != EC_ACC32 && ec != EC_STORE32) ec = EC_GENERIC;
       snprintf(out, (size_t)cap, "gemm16x_kernel<%d, %s, %s, %s, %d>", d.in_dtype, shapes[v], at, bt, ec);

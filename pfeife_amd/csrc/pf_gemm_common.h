@@ -1,6 +1,7 @@
 // Pieces shared by the GEMM translation units: launch geometry, the runtime-configured
 // epilogue, the XCD-aware workgroup -> tile order, MFMA wrappers, raw buffer access.
 #pragma once
+#include <cstdlib>
 #include <mutex>
 #include <type_traits>
 
@@ -175,7 +176,20 @@ __device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t b
 // Tile shapes of the direct-to-LDS kernel (BM x BN; reduction depth per stage, stages):
 //   256x256 (32 deep, 5 stages): one 128x128 block per wavefront, the least operand traffic per FLOP
 //   256x128 (64 deep, 3 stages), 128x128 (64 deep, 3 stages): more workgroups for smaller outputs
-enum { PF_XT_256x256 = 1, PF_XT_256x128 = 2, PF_XT_128x128 = 3, PF_XT_192x256 = 4, PF_XT_COUNT = 5 };
+//   128x128 (32 deep, 4 stages; 64 KB) and 256x128 (32 deep, 3 stages; 72 KB): "d" tiles, small enough
+//   in LDS and registers for TWO workgroups per CU, so that workgroups of kernels launched on
+//   different streams share a CU and one's prologue and epilogue run under the other's reduction loop
+enum { PF_XT_256x256 = 1, PF_XT_256x128 = 2, PF_XT_128x128 = 3, PF_XT_192x256 = 4, PF_XT_128x128d = 5,
+       PF_XT_256x128d = 6, PF_XT_COUNT = 7 };
+// BM, BN, reduction depth per stage, stages of each tile id
+template <int XT> struct XTile;
+template <> struct XTile<PF_XT_256x256> { static constexpr int BM = 256, BN = 256, BK = 32, ST = 5; };
+template <> struct XTile<PF_XT_256x128> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3; };
+template <> struct XTile<PF_XT_128x128> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3; };
+template <> struct XTile<PF_XT_192x256> { static constexpr int BM = 192, BN = 256, BK = 32, ST = 5; };
+template <> struct XTile<PF_XT_128x128d> { static constexpr int BM = 128, BN = 128, BK = 32, ST = 4; };
+template <> struct XTile<PF_XT_256x128d> { static constexpr int BM = 256, BN = 128, BK = 32, ST = 3; };
+inline int x_tile_bk(int xt) { return (xt == PF_XT_256x128 || xt == PF_XT_128x128) ? 64 : 32; }
 
 // Epilogue classes with straight-line code (which operands exist, and their dtypes, fixed at
 // compile time).  Everything else takes EC_GENERIC: one rolled loop with runtime switches.

@@ -1,5 +1,5 @@
 // The direct-to-LDS 16-bit MFMA kernel and its launchers.  Included by one translation unit per
-// operand dtype (the instantiations take minutes to compile; separate units build in parallel).
+// operand dtype and tile shape (the instantiations take minutes to compile; separate units build in parallel).
 #pragma once
 #include "pf_gemm_common.h"
 
@@ -723,26 +723,16 @@ int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
   return PF_ERR_INVALID;
 }
 
-template <int DT>
-int gemm_x_group_launch(const pf_gemm_desc* d, int n, int tile, hipStream_t st) {
-  switch (tile) {
-    case PF_XT_256x256: return launch16x_group<DT, 256, 256, 32, 2, 2, 5>(d, n, st);
-    case PF_XT_256x128: return launch16x_group<DT, 256, 128, 64, 2, 2, 3>(d, n, st);
-    case PF_XT_128x128: return launch16x_group<DT, 128, 128, 64, 2, 2, 3>(d, n, st);
-    default: pf_set_error("pf_gemm_grouped: unknown direct-to-LDS tile %d", tile); return PF_ERR_INVALID;
-  }
+// one tile shape per translation unit (see pf_gemm_x_inst.hip)
+template <int DT, int XT>
+int gemm_x_group_launch(const pf_gemm_desc* d, int n, hipStream_t st) {
+  using T = XTile<XT>;
+  return launch16x_group<DT, T::BM, T::BN, T::BK, 2, 2, T::ST>(d, n, st);
 }
-
-// tile: one of the PF_XT_* shapes (see pf_gemm_x_tiles)
-template <int DT>
-int gemm_x_launch(const pf_gemm_desc& d, int tile, hipStream_t st) {
-  switch (tile) {
-    case PF_XT_256x256: return launch16x<DT, 256, 256, 32, 2, 2, 5>(d, st);
-    case PF_XT_256x128: return launch16x<DT, 256, 128, 64, 2, 2, 3>(d, st);
-    case PF_XT_128x128: return launch16x<DT, 128, 128, 64, 2, 2, 3>(d, st);
-    case PF_XT_192x256: return launch16x<DT, 192, 256, 32, 2, 2, 5>(d, st);
-    default: pf_set_error("pf_gemm: unknown direct-to-LDS tile %d", tile); return PF_ERR_INVALID;
-  }
+template <int DT, int XT>
+int gemm_x_launch(const pf_gemm_desc& d, hipStream_t st) {
+  using T = XTile<XT>;
+  return launch16x<DT, T::BM, T::BN, T::BK, 2, 2, T::ST>(d, st);
 }
 
 }  // namespace

@@ -8,7 +8,9 @@ ONCE as a single stage for one micro-batch (the same launch lists a real stage r
 the lowerer says which launches belong to which graph node, and the launches are timed on
 the device with events recorded between the nodes (HIP events on the worker's stream; wall
 clock for a host kernel table, whose launches are synchronous).  Memory figures are the
-sizes of the buffers the lowering allocated, not allocator watermarks.
+sizes of the buffers the lowering allocated, not allocator watermarks.  While the profile runs
+the single-stage copy's buffers (one micro-batch of activations, a gradient buffer and a 16-bit
+shadow per parameter) exist next to the model; they are released before it returns.
 """
 import time
 from dataclasses import dataclass, field
@@ -134,7 +136,8 @@ def profile_graph(kernels, device, compute_dtype, gm, live_args, repeats=3, stre
                 pos = b
             if cuda:
                 evs = [torch.cuda.Event(enable_timing=True) for _ in range(len(marks) + 1)]
-                so = torch.cuda.current_stream(device)
+                # the events go to the stream the launches go to (`s` is its raw handle)
+                so = torch.cuda.ExternalStream(s, device=device) if s else torch.cuda.current_stream(device)
                 for (name, a, b), ev in zip(marks, evs):
                     ev.record(so)
                     for launch in launches[a:b]:
@@ -193,3 +196,10 @@ def profile_graph(kernels, device, compute_dtype, gm, live_args, repeats=3, stre
     finally:
         for p, g in saved_grads:
             p.grad = g
+        # the single-stage copy holds a second set of activations, gradient buffers and 16-bit
+        # shadows: give them back before the real stages are built
+        prog = out_grads = ins = None
+        L = params = pool = None
+        if device.type == "cuda":
+            torch.cuda.synchronize(device)
+            torch.cuda.empty_cache()

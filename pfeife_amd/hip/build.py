@@ -19,14 +19,17 @@ OBJ_DIR = os.path.join(HERE, "build")
 SOURCES = [
     "pf_runtime.cpp",
     "pf_gemm.hip",
-    "pf_gemm_x_f16.hip",
-    "pf_gemm_x_bf16.hip",
     "pf_attention.hip",
     "pf_norm.hip",
     "pf_elementwise.hip",
     "pf_softmax_loss.hip",
     "pf_batch.hip",
 ]
+
+# the direct-to-LDS MFMA kernel: one object per (operand dtype id, tile id), all from one source
+# (ids as in csrc/pf_gemm_common.h: dtypes PF_F16 = 1, PF_BF16 = 2; tiles PF_XT_* = 1..6)
+GEMM_X_SOURCE = "pf_gemm_x_inst.hip"
+GEMM_X_PAIRS = [(dt, xt) for xt in (1, 2, 3, 4, 5, 6) for dt in (1, 2)]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -44,9 +47,10 @@ COMMON_FLAGS = [
 ]
 
 
-def _compile_one(src):
-    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
-    cmd = [HIPCC, "-x", "hip"] + COMMON_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+def _compile_one(job):
+    src, defines, stem = job
+    obj = os.path.join(OBJ_DIR, stem + ".o")
+    cmd = [HIPCC, "-x", "hip"] + COMMON_FLAGS + defines + ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature and says so once per pass
     err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
@@ -60,14 +64,17 @@ def build(verbose=True, jobs=None):
     if not os.path.exists(HIPCC):
         raise RuntimeError("hipcc not found at %s (set HIPCC)" % HIPCC)
     os.makedirs(OBJ_DIR, exist_ok=True)
-    jobs = jobs or min(len(SOURCES), max(1, os.cpu_count() or 2))
+    work = [(GEMM_X_SOURCE, ["-DPF_X_DT=%d" % dt, "-DPF_X_TILE=%d" % xt], "pf_gemm_x_%d_%d" % (dt, xt))
+            for dt, xt in GEMM_X_PAIRS]   # the long ones first
+    work += [(src, [], os.path.splitext(src)[0]) for src in SOURCES]
+    jobs = jobs or min(len(work), max(1, os.cpu_count() or 2))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        results = list(pool.map(_compile_one, SOURCES))
+        results = list(pool.map(_compile_one, work))
     objs = [o for o, _ in results]
     if verbose:
-        for (_, warn), src in zip(results, SOURCES):
+        for (_, warn), job in zip(results, work):
             if warn.strip():
-                print("[pfeife_amd.hip.build] %s:\n%s" % (src, warn), file=sys.stderr)
+                print("[pfeife_amd.hip.build] %s:\n%s" % (job[2], warn), file=sys.stderr)
     tmp = LIB_PATH + ".tmp"
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + objs
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -186,6 +186,16 @@ class PartialRunner:
     def log_memory_usage(self):
         get_logger().info(self.worker.memory_report())
 
+    def scaler_state_dict(self):
+        """State of the dynamic loss scaler (torch.amp.GradScaler.state_dict() layout) for a
+        checkpoint; the reference keeps its GradScaler inside the worker and saves nothing
+        (pfeife/mp/worker.py:133-145).  `optimizer.state_dict()` already carries the count of
+        completed steps in its `step` entries."""
+        return self.worker.scaler_state_dict()
+
+    def load_scaler_state_dict(self, state):
+        self.worker.load_scaler_state_dict(state)
+
     def train(self):
         """No-op, as in the reference (pfeife/mp/partial/module.py:175-177): stage programs are built
         from the graph TorchDynamo captured, and a captured dropout with p > 0 is refused at lowering."""

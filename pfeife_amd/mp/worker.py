@@ -65,6 +65,8 @@ class StageWorker:
         self.graphs_ready = False
         self.steps_done = 0
         self.begin_graph = None
+        self.plan = None           # the auto-partitioner's choice (split points + schedule variant), if it ran
+        self.profile = None
         # One stream per pipeline rank ("lane"): the jobs of different ranks are independent by
         # construction of the schedule (that is what lets the reference run them on different
         # GPUs), so on one GPU they run side by side and fill the CUs and launch gaps that a
@@ -114,6 +116,10 @@ class StageWorker:
         loop_batch = opt.loop_batch if opt.loop_batch is not None else device_cnt
         loop_batch = max(1, min(loop_batch, opt.batch_cnt))
         prefetch = opt.prefetch_fwd if opt.prefetch_fwd is not None else 0
+        plan = getattr(self, "plan", None)
+        if plan is not None and plan.sched_params.node_cnt == node_cnt:
+            # the auto-partitioner valued its split under one schedule variant: run that one
+            loop_batch, prefetch = plan.sched_params.loop_batch, plan.sched_params.prefetch_fwd
         for st in pg.nodes.values():
             st.rank = st.idx % device_cnt
         self.sched_params = PipeSchedParams(device_cnt, opt.batch_cnt, node_cnt, loop_batch, prefetch)
@@ -312,6 +318,9 @@ class StageWorker:
         self._job_events = {}
         self._loss_events = {}
         self.optimizer = None
+        self.plan = self.profile = None
+        self._steps_owner = None
+        self._host_steps_stale = False
         self.params = ParamStore(self.kernels, self.device)
         self.pool = BufferPool(self.device)
         self.lowerer = Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
@@ -553,6 +562,8 @@ class StageWorker:
     def _fused_adam_step(self, opt, scaled=False):
         cache = self.__dict__.setdefault("_adam_tables", {})
         s = self.stream()
+        rebuilt = False
+        groups = []
         for gi, g in enumerate(opt.param_groups):
             params = [p for p in g["params"] if p.grad is not None]
             if not params:
@@ -570,20 +581,83 @@ class StageWorker:
                                                 [opt.state[p]["exp_avg"] for p in params],
                                                 [opt.state[p]["exp_avg_sq"] for p in params])
                 ent = cache[gi] = (sig, table)
-            step = int(opt.state[params[0]]["step"].item()) + 1
+                rebuilt = True
+            groups.append((g, params, ent[1]))
+        if scaled and rebuilt:
+            self._seed_device_step_count(opt, groups)
+        for g, params, (table, n_items, max_n) in groups:
             b1, b2 = g["betas"]
-            table, n_items, max_n = ent[1]
             if scaled:
-                # skipped on overflow; the bias corrections use the device's count of completed steps
-                # (the host-side `step` entries below count attempted steps)
+                # skipped on overflow; the bias corrections use the device's count of completed steps.
+                # The host-side `step` entries are brought up to date from that count when somebody
+                # reads them (sync_optimizer_steps: optimizer.state_dict() calls it)
                 self.kernels.adam_step_scaled(table, n_items, max_n, float(g["lr"]), float(b1), float(b2),
                                               float(g["eps"]), float(g["weight_decay"]),
                                               type(opt) is torch.optim.AdamW, self.scaler_state, s)
+                self._host_steps_stale = True
             else:
+                step = int(opt.state[params[0]]["step"].item()) + 1
                 self.kernels.adam_step(table, n_items, max_n, float(g["lr"]), float(b1), float(b2), float(g["eps"]),
                                        float(g["weight_decay"]), step, type(opt) is torch.optim.AdamW, s)
-            for p in params:
-                opt.state[p]["step"] += 1
+                for p in params:
+                    opt.state[p]["step"] += 1
+
+    def _seed_device_step_count(self, opt, groups):
+        """The fused step under dynamic loss scaling takes Adam's bias corrections from the device's
+        count of completed steps (scaler_state[3]).  Whenever the optimizer's state tensors are new
+        to this worker (first step, `load_state_dict`), that count is set from the optimizer's own
+        `step` entries, so a resumed optimizer continues at step k + 1 against its warm moments.
+        One counter serves every parameter: an optimizer whose parameters disagree is refused."""
+        if getattr(self, "_host_steps_stale", False) and getattr(self, "_steps_owner", None) is opt:
+            self.sync_optimizer_steps()
+        steps = {int(float(opt.state[p]["step"])) for _, params, _ in groups for p in params}
+        if len(steps) > 1:
+            raise RuntimeError("fused Adam step with dynamic loss scaling: the optimizer's parameters are at "
+                               "different step counts %s; one device-side counter serves them all" % sorted(steps))
+        k = float(steps.pop()) if steps else 0.0
+        if float(self.scaler_state[3].item()) != k:
+            self.scaler_state[3:4].fill_(k)
+        if getattr(self, "_steps_owner", None) is not opt:
+            self._steps_owner = opt
+            if hasattr(opt, "register_state_dict_pre_hook"):
+                opt.register_state_dict_pre_hook(lambda o: self.sync_optimizer_steps())
+
+    def sync_optimizer_steps(self):
+        """Writes the device's count of completed optimizer steps into the optimizer's `step`
+        entries (one host read).  torch.amp.GradScaler leaves `step` untouched on a skipped step;
+        so does this, which is why the entries cannot simply be bumped on the host."""
+        opt = getattr(self, "_steps_owner", None)
+        if opt is None or not self.dyn_scale or not getattr(self, "_host_steps_stale", False):
+            return
+        done = float(self.scaler_state[3].item())
+        for g in opt.param_groups:
+            for p in g["params"]:
+                st = opt.state.get(p)
+                if st and "step" in st:
+                    if torch.is_tensor(st["step"]):
+                        st["step"].fill_(done)
+                    else:
+                        st["step"] = done
+        self._host_steps_stale = False
+
+    def scaler_state_dict(self):
+        """The dynamic loss scaler's state in torch.amp.GradScaler.state_dict()'s layout (empty
+        for a static scale), for checkpoints."""
+        if not self.dyn_scale:
+            return {}
+        st = self.scaler_state.tolist()
+        o = self.option
+        return {"scale": st[0], "growth_factor": o.growth_factor, "backoff_factor": o.backoff_factor,
+                "growth_interval": o.growth_interval, "_growth_tracker": int(st[1])}
+
+    def load_scaler_state_dict(self, state):
+        if not self.dyn_scale:
+            if state:
+                raise RuntimeError("this worker runs with a static loss scale; there is no scaler state to load")
+            return
+        self.scaler_state[0:1].fill_(float(state["scale"]))
+        self.scaler_state[1:2].fill_(float(state.get("_growth_tracker", 0)))
+        self.scaler_state[2:3].fill_(0.0)
 
     # -- reporting -----------------------------------------------------------------------
     def memory_report(self):

@@ -6,7 +6,14 @@ Counterpart of the search branch of `PipeGraphGenerator.gen_graph`
 (pfeife/graph/pipe_graph.py:177-314) as the objective:
 
   * the stage count is `loop_cnt * device_cnt` when `loop_cnt` is given, else the best of
-    1x, 2x and 3x `device_cnt` (a count needs at least `count + 4` compute nodes);
+    1x, 2x and 3x `device_cnt` (a count needs at least `count + 4` compute nodes; a looped
+    count the user did not ask for is skipped when its stages would average 3 ms or less);
+  * for every stage count the schedule variants of `PipeSchedSet` (`loop_batch` x
+    `prefetch_fwd`, pfeife/schedule/scheduler.py:118-151) are searched, except that a
+    `loop_batch` / `prefetch_fwd` the user fixed in the option is kept (planner.py:706-714).  Every
+    variant is valued: the reference leaves a stage count at the first variant that improves the
+    best time by less than 1 % (planner.py:778-787), a shortcut for its far costlier valuation
+    that can miss the optimum by more than that;
   * a candidate split is valued by the expected time of one optimisation step: the jobs
     (stage, micro-batch, direction) run in each rank's schedule order, a job starts when its
     rank is free and the jobs it depends on have finished (plus the transfer time of the
@@ -26,12 +33,13 @@ import math
 from dataclasses import dataclass, field
 from typing import List, Optional
 
-from .scheduler import PipeSchedParams
+from .scheduler import PipeSchedParams, PipeSchedSet
 
 HBM_BYTES = 288 * 1024 ** 3       # MI355X
 RESERVE_MEM_RATIO = 0.9           # part of a rank's memory the plan may use
 ADAM_BYTES_PER_PARAM_BYTE = 7.0   # 28 bytes moved per fp32 parameter
 OPTIM_GBS = 4800.0                # measured rate of the fused Adam step
+FWD_AVG_MIN = 3.0                 # ms: looped stage counts nobody asked for need stages longer than this
 
 
 @dataclass
@@ -277,8 +285,23 @@ def search_points(model, sched, cand, max_mem=None, beam=8, exhaustive_limit=200
     return best[0], list(best[1]), len(seen)
 
 
+def schedule_variants(option, device_cnt, batch_cnt, node_cnt):
+    """(loop_batch, prefetch_fwd) pairs to value for `node_cnt` stages: the reference's set, narrowed
+    to what the user fixed; when the set is empty (fewer micro-batches than ranks) the manual-split
+    defaults are used (`loop_batch = device_cnt` clamped to `batch_cnt`, no prefetch)."""
+    pairs = PipeSchedSet.variants(device_cnt, batch_cnt, node_cnt)
+    if option.loop_batch is not None:
+        pairs = [(lb, pf) for lb, pf in pairs if lb == option.loop_batch]
+    if option.prefetch_fwd is not None:
+        pairs = [(lb, pf) for lb, pf in pairs if pf == option.prefetch_fwd]
+    if not pairs:
+        lb = option.loop_batch if option.loop_batch is not None else device_cnt
+        pairs = [(max(1, min(lb, batch_cnt)), option.prefetch_fwd if option.prefetch_fwd is not None else 0)]
+    return pairs
+
+
 def plan_split(prof, option, device_cnt, max_mem=None, link=None, beam=8):
-    """-> Plan with the best split points over the stage counts tried."""
+    """-> Plan with the best (split points, schedule variant) over the stage counts tried."""
     model = CostModel(prof, link)
     batch_cnt = option.batch_cnt
     if max_mem is None:
@@ -287,19 +310,36 @@ def plan_split(prof, option, device_cnt, max_mem=None, link=None, beam=8):
     counts = [option.loop_cnt * device_cnt] if option.loop_cnt else [i * device_cnt for i in range(1, 4)]
     best = None
     evaluated = 0
-    for cnt in counts:
+    total_ms = model.fwd[-1] + model.bwd[-1]
+    for loop_idx, cnt in enumerate(counts):
         if cnt + 4 > prof.n or cnt - 1 > len(cand):
             break
-        loop_batch = option.loop_batch if option.loop_batch is not None else device_cnt
-        loop_batch = max(1, min(loop_batch, batch_cnt))
-        prefetch = option.prefetch_fwd if option.prefetch_fwd is not None else 0
-        sched = PipeSchedParams(device_cnt, batch_cnt, cnt, loop_batch, prefetch)
-        v, pts, n = search_points(model, sched, cand, max_mem, beam=beam)
-        evaluated += n
-        if pts is None or not math.isfinite(v):
-            continue
-        if best is None or v < best[0] - 1e-9:
-            best = (v, pts, sched)
+        if loop_idx != 0 and not option.loop_cnt and total_ms / cnt <= FWD_AVG_MIN:
+            continue   # stages too short to be worth another loop (planner.py:724-737)
+        for loop_batch, prefetch in schedule_variants(option, device_cnt, batch_cnt, cnt):
+            sched = PipeSchedParams(device_cnt, batch_cnt, cnt, loop_batch, prefetch)
+            try:
+                v, pts, n = search_points(model, sched, cand, max_mem, beam=beam)
+            except RuntimeError:   # a variant whose rank lists cannot be merged into one order
+                continue
+            evaluated += n
+            if pts is None or not math.isfinite(v):
+                continue
+            if best is None or v < best[0] - 1e-9:
+                best = (v, pts, sched)
+    if best is None:
+        # too few compute nodes (or cut positions) for device_cnt stages: fewer stages, down to one,
+        # with every legal position as a candidate
+        every = [i for i in range(1, prof.n) if (prof.cut_ok[i] if prof.cut_ok else True)]
+        for cnt in range(min(device_cnt, len(every) + 1, prof.n), 0, -1):
+            ranks = min(device_cnt, cnt)
+            lb, pf = schedule_variants(option, ranks, batch_cnt, cnt)[0]
+            sched = PipeSchedParams(ranks, batch_cnt, cnt, max(1, min(lb, batch_cnt)), pf)
+            v, pts, n = search_points(model, sched, every, max_mem[:ranks], beam=beam)
+            evaluated += n
+            if pts is not None and math.isfinite(v):
+                best = (v, pts, sched)
+                break
     if best is None:
         raise RuntimeError("auto-partitioner: no split of the graph's %d compute nodes into %s stages fits"
                            % (prof.n, counts))

@@ -85,6 +85,30 @@ class PipeSchedParams:
     __repr__ = __str__
 
 
+class PipeSchedSet:
+    """The schedule variants the auto-partitioner values for one stage count
+    (pfeife/schedule/scheduler.py:118-151): a looped pipeline (more stages than ranks) tries every
+    `loop_batch` from `device_cnt` to `batch_cnt` that is `device_cnt` itself or divides
+    `batch_cnt`, each with `prefetch_fwd` 0 .. device_cnt - 1; a plain pipeline takes
+    `loop_batch = batch_cnt` with the same prefetch range."""
+
+    def __init__(self, device_cnt, batch_cnt, node_cnt):
+        self.device_cnt, self.batch_cnt, self.node_cnt = int(device_cnt), int(batch_cnt), int(node_cnt)
+        self.scheds: List[PipeSchedParams] = [
+            PipeSchedParams(self.device_cnt, self.batch_cnt, self.node_cnt, lb, pf)
+            for lb, pf in self.variants(self.device_cnt, self.batch_cnt, self.node_cnt)]
+
+    @staticmethod
+    def variants(device_cnt, batch_cnt, node_cnt):
+        """-> [(loop_batch, prefetch_fwd)] in the order the reference builds its set."""
+        D, B, S = int(device_cnt), int(batch_cnt), int(node_cnt)
+        if S > D:
+            loops = [lb for lb in range(D, B + 1) if lb == D or B % lb == 0]
+        else:
+            loops = [B]
+        return [(lb, pf) for lb in loops for pf in range(D)]
+
+
 class Scheduler:
     """Expands rank_works into RECV/COMPUTE/SEND job triples per rank."""
 

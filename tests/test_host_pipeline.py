@@ -251,6 +251,25 @@ def test_dynamic_loss_scale_skips_overflowing_steps():
     runner.step(x, y)                                   # two clean steps: scale doubles
     assert w.scaler_scale() == 256.0
     assert float(w.scaler_state[3]) == 3.0
+    # the scaler's state travels in torch.amp.GradScaler's layout and loads back
+    saved = runner.scaler_state_dict()
+    assert saved == {"scale": 256.0, "growth_factor": 2.0, "backoff_factor": 0.5, "growth_interval": 2,
+                     "_growth_tracker": 0}
+    ref_scaler = torch.amp.GradScaler("cpu")
+    ref_scaler.load_state_dict(saved)                   # torch accepts it as its own
+    assert ref_scaler.get_growth_interval() == 2
+    runner.step(x, y)                                   # one clean step: tracker 1
+    assert runner.scaler_state_dict()["_growth_tracker"] == 1
+    runner.load_scaler_state_dict(dict(saved, scale=64.0))
+    assert w.scaler_scale() == 64.0 and runner.scaler_state_dict()["_growth_tracker"] == 0
+
+
+def test_static_loss_scale_has_no_scaler_state():
+    runner = make_runner(PipeOption(device_cnt=1, batch_cnt=1, batch_size=2))
+    assert runner.scaler_state_dict() == {}
+    runner.load_scaler_state_dict({})
+    with pytest.raises(RuntimeError, match="static loss scale"):
+        runner.load_scaler_state_dict({"scale": 2.0})
 
 
 def test_failed_step_releases_parked_micro_batches():

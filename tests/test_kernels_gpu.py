@@ -123,7 +123,8 @@ def test_gemm_epilogues(hip, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32"), (2, "256, 128, 64"), (3, "128, 128, 64"), (4, "192, 256, 32")])
+@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 5"), (2, "256, 128, 64, 2, 2, 3"), (3, "128, 128, 64, 2, 2, 3"),
+                                          (4, "192, 256, 32, 2, 2, 5"), (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3")])
 def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
     """Every straight-line epilogue class of the direct-to-LDS kernel on every tile shape, ragged in M
     (and in N against the 256- and 192-wide tiles), against the oracle; the launch names the class."""
@@ -138,8 +139,7 @@ def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
         dev = {k: (None if v is None else v.cuda()) for k, v in tensors.items()}
         cpu = {k: (None if v is None else v.clone()) for k, v in tensors.items()}
         launch = hip.gemm(**dev, variant=variant, **kw)
-        assert launch.variant == "gemm16x_kernel<%d, %s, 2, 2, %d, false, false, %d>" % (
-            dt, tile, 3 if tile.endswith("64") else 5, ec), launch.variant
+        assert launch.variant == "gemm16x_kernel<%d, %s, false, false, %d>" % (dt, tile, ec), launch.variant
         launch(torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
         oracle.gemm(**cpu, **kw)()
@@ -170,7 +170,31 @@ def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("variant,bm", [(1, 256), (2, 256), (3, 128), (4, 192)])
+@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 5"), (2, "256, 128, 64, 2, 2, 3"), (3, "128, 128, 64, 2, 2, 3"),
+                                          (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3")])
+def test_gemm_direct_to_lds_weight_gradient_tiles(hip, oracle, dtype, variant, tile):
+    """The reduction-strided (weight-gradient) form of every tile that has one: dW += dY^T X with a
+    ragged reduction length (not a multiple of any stage depth) and ragged M and N, fp32 accumulate
+    and fp32 store, against the oracle."""
+    rows, M, N = 1000, 1160, 520
+    dt = {F16: 1, BF16: 2}[dtype]
+    dy, x = rnd((rows, M), dtype, 1), rnd((rows, N), dtype, 2, 0.1)
+    for ec, beta in ((4, 1), (1, 0)):
+        print("gemm variant", variant, "transposed class", ec, flush=True)
+        c0 = rnd((M, N), F32, 3)
+        dev = dict(a=dy.cuda(), b=x.cuda(), c=c0.clone().cuda())
+        cpu = dict(a=dy, b=x, c=c0.clone())
+        kw = dict(M=M, N=N, K=rows, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=beta)
+        launch = hip.gemm(**dev, variant=variant, **kw)
+        assert launch.variant == "gemm16x_kernel<%d, %s, true, true, %d>" % (dt, tile, ec), launch.variant
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        oracle.gemm(**cpu, **kw)()
+        close((dev["c"].cpu(), cpu["c"]), 1e-3, 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("variant,bm", [(1, 256), (2, 256), (3, 128), (4, 192), (5, 128), (6, 256)])
 def test_gemm_gelu_grad_epilogue_leaves_column_sums(hip, dtype, variant, bm):
     """The GELU' epilogue of the direct-to-LDS kernel can also leave the column sums of the values it
     stores (the bias gradient of the layer whose pre-activation gradient it writes) as one partial row

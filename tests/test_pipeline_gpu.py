@@ -955,6 +955,74 @@ def test_dynamic_loss_scale_matches_torch_gradscaler_and_adam():
                                    msg=n)
 
 
+def test_resumed_adam_under_dynamic_loss_scale_continues_its_step_count():
+    """An optimizer whose state was loaded (`load_state_dict`, step = k, warm moments) continues at
+    step k + 1 under the fused Adam step with dynamic loss scaling: one clean step, one overflowing
+    step and one more clean step against torch.amp.GradScaler + torch.optim.Adam resumed from the
+    same state; `optimizer.state_dict()` reports performed steps (a skipped step is not counted)."""
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=2, mlp_dim=128, num_classes=10)
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(8, 3, 32, 32, generator=g).cuda()
+    y = torch.randint(0, 10, (8,), generator=g).cuda()
+    crit = nn.CrossEntropyLoss()
+    torch.manual_seed(0)
+    model = VisionTransformer(cfg).cuda()
+    # warm state: seven plain Adam steps in PyTorch
+    warm = torch.optim.Adam(model.parameters(), lr=1e-2)
+    for _ in range(7):
+        warm.zero_grad()
+        crit(model(x), y).backward()
+        warm.step()
+    saved = copy.deepcopy(warm.state_dict())
+    assert float(saved["state"][0]["step"]) == 7.0
+    ref = copy.deepcopy(model)
+    ropt = torch.optim.Adam(ref.parameters(), lr=1e-2)
+    ropt.load_state_dict(copy.deepcopy(saved))
+    opt = torch.optim.Adam(model.parameters(), lr=1e-2)
+    opt.load_state_dict(copy.deepcopy(saved))
+
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=4, split_points=["blocks.1"], loss_scale="dynamic",
+                        init_scale=1024.0, growth_interval=100)
+    runner = _fresh_runner(option)
+    runner.optimizer = opt
+    cmodel = torch.compile(model, backend=partial_compiler)
+    poison = [False]
+
+    def fn(px, labels):
+        loss = crit(cmodel(px).float(), labels)
+        (loss * float("inf") if poison[0] else loss).backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    scaler = torch.amp.GradScaler("cuda", init_scale=1024.0, growth_interval=100)
+    for step in range(3):
+        poison[0] = step == 1
+        runner.step(x, y)
+        ropt.zero_grad(set_to_none=False)
+        for xs, ys in zip(x.chunk(2), y.chunk(2)):
+            loss = crit(ref(xs), ys)
+            scaler.scale(loss * float("inf") if poison[0] else loss).backward()
+        scaler.step(ropt)
+        scaler.update()
+        torch.cuda.synchronize()
+        assert runner.worker._fused_adam_applicable(opt)
+        assert float(runner.worker.scaler_state[3]) == 7.0 + (1, 1, 2)[step]
+        for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+            real = ropt.state[q]["exp_avg_sq"] > 1e-10
+            # a restart of the bias corrections at t = 1 against the warm moments would move every
+            # parameter by several times the tolerance
+            torch.testing.assert_close(p.detach()[real], q.detach()[real], rtol=2e-4, atol=2e-5,
+                                       msg=lambda m: "%s step %d: %s" % (n, step, m))
+    mine, theirs = opt.state_dict(), ropt.state_dict()
+    for idx in theirs["state"]:
+        assert float(mine["state"][idx]["step"]) == float(theirs["state"][idx]["step"]) == 9.0
+    assert runner.scaler_state_dict()["scale"] == float(scaler.get_scale()) == 512.0
+
+
 def test_dynamic_loss_scale_with_an_optimizer_that_keeps_pytorchs_step():
     """Dynamic loss scaling with SGD + momentum (no fused step: the overflow flag is read once on the host
     and PyTorch's own step() runs or is skipped), fp32 model: five steps, the second with an overflowing
