@@ -266,6 +266,49 @@ def hbm_kernel_rates(runner, reps=3):
     return out
 
 
+def gemm_ceiling(kernels, mixed, reps=20):
+    """Off-path record: what the step's matrix-product kernel reaches on shapes that take the
+    step's shape losses away, so that kernel loss and shape loss can be told apart.  Times (hipGraph
+    replays, HIP events) the 256x256-tile direct-to-LDS kernel on 8192^3, one of the step's own
+    products ([3152 x 1024] . [1024 x 4096], the MLP's first layer, plain 16-bit store) and the same
+    product with a four times longer reduction, plus the 128x128 tile on the step's dominant
+    shape ([3152 x 4096] . [4096 x 1024]) and on that shape with 16 times the rows."""
+    import torch
+
+    dt = {"fp16": torch.float16, "bf16": torch.bfloat16}.get(mixed)
+    if dt is None:
+        return None
+    st = torch.cuda.Stream()
+    s = st.cuda_stream
+    out = []
+    for label, M, N, K, variant in (("8192^3, 256x256 tile", 8192, 8192, 8192, 1),
+                                    ("step shape 3152x4096x1024, 256x256 tile", 3152, 4096, 1024, 1),
+                                    ("same with K x4 (3152x4096x4096), 256x256 tile", 3152, 4096, 4096, 1),
+                                    ("step shape 3152x1024x4096, 128x128 tile", 3152, 1024, 4096, 3),
+                                    ("same with M x16 (50432x1024x4096), 128x128 tile", 50432, 1024, 4096, 3),
+                                    ("same with M x16 (50432x1024x4096), 256x256 tile", 50432, 1024, 4096, 1)):
+        x = torch.randn(M, K, device="cuda", dtype=dt)
+        w = torch.randn(N, K, device="cuda", dtype=dt) * 0.03
+        c = torch.empty(M, N, device="cuda", dtype=dt)
+        n = 4 if M * N * K > 1e11 else 16
+        chain = [kernels.gemm(x, w, c, M=M, N=N, K=K, lda=K, ldb=K, ldc=N, variant=variant) for _ in range(n)]
+        graph = kernels.capture(chain, s)
+        graph(s)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record(st)
+        for _ in range(reps):
+            graph(s)
+        ev1.record(st)
+        ev1.synchronize()
+        us = 1e3 * ev0.elapsed_time(ev1) / (reps * n)
+        kernels.destroy_graph(graph)
+        tf = 2.0 * M * N * K / us / 1e6
+        out.append(dict(shape=label, kernel=chain[0].variant, avg_launch_us=round(us, 2), tflops=round(tf, 1),
+                        frac=round(tf / PEAK_TFLOPS[mixed], 4)))
+        del x, w, c, chain
+    return out
+
+
 def cpu_baseline(name):
     """The oracle's restatement of the reference's stage execution on the host
     cores, fp32, on a bounded sample of the workload (about 10-20 s of CPU work in all)."""
@@ -539,6 +582,10 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
                100 * r["frac"], PEAK_HBM_GBS, "" if r["on_path"] else "  [off-path micro-benchmark]",
                "" if "frac_of_copy" not in r else "  copy of the same bytes: %.1f us (kernel at %.0f%% of it)"
                % (r["copy_same_bytes_us"], 100 * r["frac_of_copy"])))
+    ceiling = gemm_ceiling(w.kernels, info["mixed"]) if (roofline and hbm) else None
+    for r in ceiling or []:
+        log("[bench] gemm ceiling [off-path] %-52s %8.1f us/launch %7.1f TFLOP/s (%.0f%% of peak)  %s"
+            % (r["shape"], r["avg_launch_us"], r["tflops"], 100 * r["frac"], r["kernel"]))
     flops_step = model_flops_per_step(info)
     cfg = info["cfg"]
     plan = getattr(w, "plan", None)
@@ -547,6 +594,7 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
                   % (plan.split_points, plan.expect_ms)) if plan is not None else str(info["splits"])
     lanes = "%d streams (%s)" % (len(w.lanes), w.lane_mode) if w.lanes else "one stream"
     res = dict(value=value, ms=ms, host_ms=host_ms, roof=roof, hbm=rates, info=info, loss_scaling=scaling,
+               gemm_ceiling=ceiling,
                model_tflops=None if flops_step is None else round(flops_step / (ms * 1e-3) / 1e12, 2),
                workload="%s: %s micro-batch %d x %d, %d stages split at %s, schedule drawn for %d ranks, "
                         "all stages on one GPU on %s, Adam" % (
@@ -684,6 +732,7 @@ def main():
         "config": {"workload": head["workload"], "global_batch": info["batch"], "batch_cnt": info["batch_cnt"]},
         "roofline": head["roof"],
         "hbm_kernels": head["hbm"],
+        "gemm_ceiling": head["gemm_ceiling"],
         "cpu_baseline": cpu,
         "torch_eager_gpu": eager,
         "model_tflops": head["model_tflops"],

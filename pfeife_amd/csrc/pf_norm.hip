@@ -334,14 +334,15 @@ __global__ __launch_bounds__(256) void norm_bwd_kernel(const void* dy, int dy_dt
     for (int i = 0; i < NV; ++i) {
       __syncthreads();
 #pragma unroll
-      for (int k = 0; k < W; ++k) red[wave][lane * W + k] = which == 0 ? pg[i][k] : (which == 1 ? pb[i][k] : ps[i < NS ? i : 0][k]);
+      // value k of lane l sits at [k * 64 + l]: consecutive lanes hit consecutive banks
+      for (int k = 0; k < W; ++k) red[wave][k * 64 + lane] = which == 0 ? pg[i][k] : (which == 1 ? pb[i][k] : ps[i < NS ? i : 0][k]);
       __syncthreads();
       if (wave == 0) {
         const int64_t c = ((int64_t)lane + i * 64) * W;
         if (c < d) {
 #pragma unroll
           for (int k = 0; k < W; ++k) {
-            const float s = red[0][lane * W + k] + red[1][lane * W + k] + red[2][lane * W + k] + red[3][lane * W + k];
+            const float s = red[0][k * 64 + lane] + red[1][k * 64 + lane] + red[2][k * 64 + lane] + red[3][k * 64 + lane];
             wrow[which * d + c + k] = s;
           }
         }
@@ -404,13 +405,13 @@ __global__ __launch_bounds__(256) void colsum_kernel(const void* x, int x_dt, in
     }
   }
 #pragma unroll
-  for (int k = 0; k < W; ++k) red[wave][lane * W + k] = s[k];
+  for (int k = 0; k < W; ++k) red[wave][k * 64 + lane] = s[k];   // lane-contiguous: no bank conflicts
   __syncthreads();
   if (wave == 0 && c < cols) {
 #pragma unroll
     for (int k = 0; k < W; ++k)
       ws[(int64_t)blockIdx.y * cols + c + k] =
-          red[0][lane * W + k] + red[1][lane * W + k] + red[2][lane * W + k] + red[3][lane * W + k];
+          red[0][k * 64 + lane] + red[1][k * 64 + lane] + red[2][k * 64 + lane] + red[3][k * 64 + lane];
   }
 }
 

@@ -1742,6 +1742,34 @@ def lower_dropout(L, node):
     return Val(x.buf, req_grad=x.req_grad, kind="view", base=x, view_fn=lambda t: t)
 
 
+def lower_pad(L, node):
+    """F.pad(x, pad, "constant", value) of a tensor that needs no gradient (label shifting:
+    pfeife's language-model scripts let the model library pad the labels with -100 and slice
+    them by one).  The padded buffer is filled once, when the program is built; a step only copies
+    x into its interior."""
+    x = L.arg(node.args[0])
+    pad = tuple(_kw(node, 1, "pad"))
+    mode = _kw(node, 2, "mode", "constant")
+    value = _kw(node, 3, "value", None)
+    if not isinstance(x, Val) or x.req_grad:
+        raise Unsupported("pad of a tensor that needs a gradient")
+    if mode != "constant" or len(pad) % 2 or len(pad) // 2 > x.buf.dim() or any(p < 0 for p in pad):
+        raise Unsupported("pad mode %s / widths %s" % (mode, pad))
+    shape = list(x.shape)
+    region = []
+    for i in range(len(pad) // 2):
+        dim = x.buf.dim() - 1 - i
+        shape[dim] += pad[2 * i] + pad[2 * i + 1]
+        region.append((dim, pad[2 * i], x.shape[dim]))
+    out = torch.full(shape, 0 if value is None else value, dtype=x.dtype, device=L.device)
+    L.cur.fwd_bytes += out.numel() * out.element_size()
+    inner = out
+    for dim, start, n in region:
+        inner = inner.narrow(dim, start, n)
+    L.copy(x.buf, inner)
+    return Val(out, req_grad=False)
+
+
 def lower_cross_entropy(L, node):
     logits = L.arg(node.args[0])
     target = L.arg(node.args[1])
@@ -1769,9 +1797,14 @@ def lower_cross_entropy(L, node):
         if g.dtype != torch.float32:
             raise Unsupported("loss gradient must be fp32")
         dst, prev = B.grad_target(logits)
-        if prev is not None or not dst.is_contiguous():
-            raise Unsupported("cross entropy backward into an already written gradient")
-        B.emit(B.k.cross_entropy_bwd(logits.buf, tgt, row_lse, g, loss2, dst, rows, classes, ignore_index))
+        if prev is None and dst.is_contiguous() and dst.dtype == logits.dtype:
+            B.emit(B.k.cross_entropy_bwd(logits.buf, tgt, row_lse, g, loss2, dst, rows, classes, ignore_index))
+        else:
+            # the logits already have a gradient (they are also returned to user code, as model
+            # libraries' output records do): form this one aside and add it
+            tmp = B.temp(logits.shape, logits.dtype)
+            B.emit(B.k.cross_entropy_bwd(logits.buf, tgt, row_lse, g, loss2, tmp, rows, classes, ignore_index))
+            B.merge(tmp, dst, prev)
         B.commit(logits, dst)
 
     if logits.req_grad:
@@ -1975,11 +2008,24 @@ def lower_rope(L, node, x_node, cos_node, sin_node, half):
     if x.buf.dim() != 4 or x.shape[-1] != 2 * half or x.buf.stride(3) != 1:
         raise Unsupported("rotary embedding on a tensor of shape %s" % (x.shape,))
     Bn, H, T, D = x.shape                      # [B, H, T, D] view of a token-major projection
-    for t in (cos, sin):
-        if t.dtype != torch.float32 or t.buf.dim() != 2 or t.shape != (T, D) or t.buf.stride(1) != 1:
-            raise Unsupported("rotary tables must be fp32 [T, D], got %s %s" % (t.shape, t.dtype))
+
+    def table(t):
+        """[T, D] fp32 view of a rotary table given as [T, D] or with broadcast dimensions in front
+        ([1, 1, T, D] / [B, 1, T, D] with the same positions for every batch entry, the form model
+        libraries hand over after `unsqueeze(1)`)."""
         if t.req_grad:
             raise Unsupported("trainable rotary tables")
+        b = t.buf
+        if b.dtype == torch.float32 and b.dim() > 2 and tuple(b.shape[-2:]) == (T, D) and b.stride(-1) == 1:
+            lead = b.reshape(-1, T, D)
+            if lead.shape[0] == 1 or bool((lead == lead[:1]).all()):   # build-time check (one host read)
+                b = lead[0]
+        if b.dtype != torch.float32 or b.dim() != 2 or tuple(b.shape) != (T, D) or b.stride(1) != 1:
+            raise Unsupported("rotary tables must be fp32 [T, D] (or that with broadcast dimensions in front), "
+                              "got %s %s" % (t.shape, t.dtype))
+        return Val(b, req_grad=False, name=t.name)
+
+    cos, sin = table(cos), table(sin)
     out_dtype = L.cd if L.mixed else x.dtype
     y = L.alloc((Bn, T, H, D), out_dtype)       # token-major like the projections
     yv = y.permute(0, 2, 1, 3)
@@ -2039,6 +2085,7 @@ FUNCTION_HANDLERS = {
     F.silu: lower_act_maybe_gate,
     F.relu: lower_unary_act, torch.relu: lower_unary_act,
     F.dropout: lower_dropout,
+    F.pad: lower_pad, torch._C._nn.pad: lower_pad,
     F.cross_entropy: lower_cross_entropy,
     F.embedding: lower_embedding,
     operator.add: lower_add, operator.iadd: lower_add, torch.add: lower_add,

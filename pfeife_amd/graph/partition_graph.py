@@ -190,7 +190,8 @@ def is_static_placeholder(node: fx.Node, example):
     if isinstance(example, torch.nn.Parameter):
         return True
     name = node.name
-    return torch.is_tensor(example) and ("_parameters_" in name or "_buffers_" in name)
+    # (constants the canonicalisation pass evaluated at compile time arrive as placeholders too)
+    return torch.is_tensor(example) and ("_parameters_" in name or "_buffers_" in name or name.startswith("pf_folded_"))
 
 
 def partition_module(gm: fx.GraphModule, stage_of: Dict[fx.Node, int], example_inputs=None,

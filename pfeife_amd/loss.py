@@ -21,6 +21,23 @@ def _kernels_for(t):
     return k
 
 
+_scratch = {}
+
+
+def _scratch_buffer(name, shape, dtype, device):
+    """Per-shape work buffers of the loss kernels, allocated once: every micro-batch's loss is
+    evaluated on the same stream in turn, and each buffer's last reader (the backward kernel, or the
+    copy of the gradient into the stage's own buffer) is enqueued before the next micro-batch's
+    writer, so a training loop makes no allocator call and no fill here."""
+    key = (name, tuple(shape), dtype, str(device))
+    t = _scratch.get(key)
+    if t is None:
+        if len(_scratch) > 64:
+            _scratch.clear()
+        t = _scratch[key] = torch.empty(shape, dtype=dtype, device=device)
+    return t
+
+
 class _CrossEntropyFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, target, ignore_index):
@@ -28,21 +45,24 @@ class _CrossEntropyFn(torch.autograd.Function):
         logits = logits.contiguous()
         target = target.contiguous()
         rows, classes = logits.shape
-        row_loss = torch.empty(rows, dtype=torch.float32, device=logits.device)
+        row_loss = _scratch_buffer("row_loss", (rows,), torch.float32, logits.device)
+        # saved for backward: per call, a second loss may be evaluated before the first one's backward
         row_lse = torch.empty(rows, dtype=torch.float32, device=logits.device)
-        loss = torch.empty(2, dtype=torch.float32, device=logits.device)
+        loss = torch.empty(2, dtype=torch.float32, device=logits.device)   # {mean loss, 1 / counted rows}
         k.run("cross_entropy_fwd", logits, target, row_loss, row_lse, loss, rows, classes, ignore_index)
         ctx.save_for_backward(logits, target, row_lse, loss)
         ctx.ignore_index = ignore_index
-        return loss[0].clone()
+        return loss[0]      # a view of this call's own result pair: no copy kernel
 
     @staticmethod
     def backward(ctx, grad_out):
         logits, target, row_lse, loss = ctx.saved_tensors
         k = _kernels_for(logits)
         rows, classes = logits.shape
-        dlogits = torch.empty_like(logits)
-        g = grad_out.detach().to(torch.float32).contiguous()
+        dlogits = _scratch_buffer("dlogits", logits.shape, logits.dtype, logits.device)
+        g = grad_out.detach()
+        if g.dtype != torch.float32 or not g.is_contiguous():
+            g = g.to(torch.float32).contiguous()
         k.run("cross_entropy_bwd", logits, target, row_lse, g, loss, dlogits, rows, classes, ctx.ignore_index)
         return dlogits, None, None
 

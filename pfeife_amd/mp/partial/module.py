@@ -30,7 +30,8 @@ import torch.nn as nn
 
 from ...batch import split_args_kwargs
 from ...executor.values import Val
-from ...graph.partition_graph import compute_nodes, partition_by_split_points
+from ...graph.canonicalize import canonicalize
+from ...graph.partition_graph import compute_nodes, is_static_placeholder, partition_by_split_points
 from ...option import PipeOption
 from ...utils import get_logger, to_device
 from ..net_states import get_state
@@ -255,6 +256,7 @@ class PartialModule(nn.Module):
                   % (len(self._all_modules) + 1, len(gm.graph.nodes), self.should_pp))
             gm.graph.print_tabular()
         self.partition_graph = None
+        self._canonical, self._folded = False, []
         # TorchDynamo recompiles when a micro-batch arrives with a new shape (ragged last chunk);
         # a structurally identical graph is the same pipeline, run by the module that owns the programs
         self.alias_of = None
@@ -289,6 +291,15 @@ class PartialModule(nn.Module):
         ex = self.example_inputs if self.example_inputs is not None else list(args)
         # module state is identified on the real call arguments (they are the live tensors)
         live = list(args)
+        if not self._canonical:
+            # library spellings (decomposed norms, eager attention, mask / rotary-table bookkeeping)
+            # -> the lowering's vocabulary; constants it evaluated become extra static inputs
+            live, info = canonicalize(self.gm, live, worker.device, is_static_placeholder)
+            self._canonical, self._folded = True, live[len(args):]
+            if any(info.values()):
+                get_logger().info("graph canonicalised: %s", info)
+        else:
+            live = live + self._folded
         points = option.split_points
         plan = None
         if self.alias_of is not None:
