@@ -451,7 +451,8 @@ def torch_eager_gpu(name, device, steps=5, warmup=2):
             return model(xb, yb)
     dtype = {"fp16": torch.float16, "bf16": torch.bfloat16}.get(mixed)
     opt = torch.optim.Adam(model.parameters(), lr=1e-5)
-    scaler = torch.amp.GradScaler("cuda", enabled=mixed == "fp16")
+    # the reference builds its GradScaler for every mixed precision (pfeife/mp/worker.py:135)
+    scaler = torch.amp.GradScaler("cuda", enabled=mixed in ("fp16", "bf16"))
     xs, ys = x.chunk(batch_cnt), y.chunk(batch_cnt)
 
     def step():
@@ -482,7 +483,7 @@ def torch_eager_gpu(name, device, steps=5, warmup=2):
                 sample="%s in PyTorch %s eager on this GPU: autocast %s, %d micro-batches x %d with gradient "
                        "accumulation, GradScaler %s, torch.optim.Adam; last loss %.4f" % (
                            cfg_name, torch.__version__, mixed, batch_cnt, batch // batch_cnt,
-                           "on" if mixed == "fp16" else "off", last))
+                           "on" if mixed in ("fp16", "bf16") else "off", last))
 
 
 def unet_stage_forward_flops(cfg, hw=32, ctx_tokens=77):

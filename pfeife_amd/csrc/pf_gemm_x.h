@@ -727,12 +727,12 @@ int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
 template <int DT, int XT>
 int gemm_x_group_launch(const pf_gemm_desc* d, int n, hipStream_t st) {
   using T = XTile<XT>;
-  return launch16x_group<DT, T::BM, T::BN, T::BK, 2, 2, T::ST>(d, n, st);
+  return launch16x_group<DT, T::BM, T::BN, T::BK, T::WGM, T::WGN, T::ST>(d, n, st);
 }
 template <int DT, int XT>
 int gemm_x_launch(const pf_gemm_desc& d, hipStream_t st) {
   using T = XTile<XT>;
-  return launch16x<DT, T::BM, T::BN, T::BK, 2, 2, T::ST>(d, st);
+  return launch16x<DT, T::BM, T::BN, T::BK, T::WGM, T::WGN, T::ST>(d, st);
 }
 
 }  // namespace

@@ -22,7 +22,6 @@ parameter gradients are accumulated in fp32.
 """
 import math
 import operator
-
 import os
 
 import torch
@@ -31,6 +30,10 @@ import torch.nn.functional as F
 from .values import Val, as_matrix, collapse_for_copy, dense_like, is_dense
 
 ACT_NONE, ACT_GELU, ACT_GELU_TANH, ACT_SILU, ACT_RELU = 0, 1, 2, 3, 4
+# kernel variant (pf_gemm_desc.variant) that regrouped weight-gradient products are pinned to: the 256x256
+# tile the automatic choice itself uses (eight wavefronts), so that products that chose it on their own and
+# products moved onto it share launches
+BIG_TILE_VARIANT = int(os.environ.get("PFEIFE_BIG_TILE", "7"))
 
 
 class Unsupported(RuntimeError):
@@ -378,7 +381,7 @@ class BwdCtx:
         bigs, t256 = [], 0
         for launch, _ in members:
             d = launch.desc
-            big = launch if launch.variant.startswith("gemm16x_kernel<%d, 256, 256" % d.in_dtype) else retile(launch, 1)
+            big = launch if launch.variant.startswith("gemm16x_kernel<%d, 256, 256" % d.in_dtype) else retile(launch, BIG_TILE_VARIANT)
             if d.M < 256 or d.N < 256 or big is None or not self.k.gemm_groupable(big):
                 return               # less than one full tile either way: stays on the small tile
             bigs.append(big)

@@ -90,11 +90,13 @@ class PipeOption:
         # before the optimizer step (the reference's GradScaler scales at every stage, so its
         # stage i of L sees S^(L-i)).  "dynamic": torch.amp.GradScaler's rule (worker.py:133-145)
         # kept on the device: overflowing steps are skipped and halve the scale, `growth_interval`
-        # clean steps double it.  A number: that static scale.  Default: dynamic for fp16 mixed
-        # precision (where the reference's scaler matters), 1.0 otherwise.
+        # clean steps double it.  A number: that static scale.  Default: dynamic for every mixed
+        # precision, fp16 and bf16 alike, as the reference builds its GradScaler
+        # (`enabled=mixed_precision is not None`, worker.py:135): a bf16 step whose gradients are
+        # not finite is skipped too.  1.0 without mixed precision.
         ls = get("loss_scale", None)
         if ls is None:
-            ls = "dynamic" if self.mixed_precision is torch.float16 else 1.0
+            ls = "dynamic" if self.mixed_precision in (torch.float16, torch.bfloat16) else 1.0
         self.loss_scale = "dynamic" if isinstance(ls, str) and ls.lower() == "dynamic" else float(ls)
         self.init_scale = float(get("init_scale", 65536.0))
         self.growth_factor = float(get("growth_factor", 2.0))

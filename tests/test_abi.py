@@ -60,7 +60,7 @@ def test_pinned_gemm_variant_that_cannot_run_the_product_is_refused():
         d.ldc, d.batch1, d.batch2, d.alpha = d.N, 1, 1, 1.0
         return d
 
-    for v, bk in ((1, 32), (2, 64), (3, 64), (4, 32), (5, 32), (6, 32)):
+    for v, bk in ((1, 32), (2, 64), (3, 64), (4, 32), (5, 32), (6, 32), (7, 32), (8, 64), (9, 64)):
         assert lib.pf_gemm_variant(ctypes.byref(desc(256, variant=v)), name, 128) == 0, v
         assert name.value.decode().startswith("gemm16x_kernel<1, "), name.value
         assert lib.pf_gemm_variant(ctypes.byref(desc(bk // 2, variant=v)), name, 128) == -1, v   # shorter than a stage

@@ -26,12 +26,14 @@ def _check(model, ref, losses, want, mixed):
     ltol = 1e-5 if mixed is None else 2e-2
     for a, b in zip(losses, want):
         assert abs(float(a) - float(b)) <= ltol * abs(float(b)), (float(a), float(b))
-    scale = max(float(q.grad.abs().max()) for q in ref.parameters())
     for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
         gp, gq = p.grad.float(), q.grad.float()
         assert torch.isfinite(gp).all(), n
-        if float(gq.abs().max()) <= 1e-6 * scale:
-            continue     # a gradient that is zero by construction (key bias): rounding noise on both sides
+        if n.endswith("k_proj.bias"):
+            # zero by construction (softmax is invariant to a shift of every score of a row, which is
+            # all a key bias does): both sides hold rounding noise only
+            assert float(gp.abs().max()) <= 1e-2 * max(float(x.grad.abs().max()) for x in ref.parameters()), n
+            continue
         if mixed is None:
             assert (gp - gq).abs().max() <= 1e-4 * gq.abs().max() + 1e-7, (n, float((gp - gq).abs().max()))
         else:

@@ -264,6 +264,43 @@ def test_dynamic_loss_scale_skips_overflowing_steps():
     assert w.scaler_scale() == 64.0 and runner.scaler_state_dict()["_growth_tracker"] == 0
 
 
+def test_bf16_step_with_non_finite_gradients_is_skipped():
+    """bf16 mixed precision runs the dynamic scaler by default, as the reference's GradScaler does
+    for every mixed precision (pfeife/mp/worker.py:135): a step whose gradients are not finite
+    changes no parameter and halves the scale; the next clean step is applied."""
+    from pfeife_amd.mp import partial_compiler
+
+    torch.manual_seed(0)
+    model = VisionTransformer(CFG)
+    option = PipeOption(device_cnt=2, batch_cnt=2, batch_size=2, split_points=["blocks.2"], mixed_precision="bf16",
+                        optimizer=dict(type="sgd", lr=0.1))
+    assert option.loss_scale == "dynamic"
+    runner = make_runner(option)
+    cmodel = torch.compile(model, backend=partial_compiler)
+    crit = nn.CrossEntropyLoss()
+    poison = [True]
+
+    def fn(x, y):
+        loss = crit(cmodel(x).float(), y)
+        (loss * float("inf") if poison[0] else loss).backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    x, y = torch.randn(4, 3, 32, 32, generator=g), torch.randint(0, 10, (4,), generator=g)
+    before = {n: p.detach().clone() for n, p in model.named_parameters()}
+    runner.step(x, y)
+    w = runner.worker
+    assert w.dyn_scale and w.scaler_scale() == 32768.0 and float(w.scaler_state[3]) == 0.0
+    for n, p in model.named_parameters():
+        assert torch.equal(p.detach(), before[n]), n
+    poison[0] = False
+    runner.step(x, y)
+    assert float(w.scaler_state[3]) == 1.0 and w.scaler_scale() == 32768.0
+    assert any(not torch.equal(p.detach(), before[n]) for n, p in model.named_parameters())
+    assert all(torch.isfinite(p.grad).all() for p in model.parameters())
+
+
 def test_static_loss_scale_has_no_scaler_state():
     runner = make_runner(PipeOption(device_cnt=1, batch_cnt=1, batch_size=2))
     assert runner.scaler_state_dict() == {}

@@ -124,7 +124,8 @@ def test_gemm_epilogues(hip, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 5"), (2, "256, 128, 64, 2, 2, 3"), (3, "128, 128, 64, 2, 2, 3"),
-                                          (4, "192, 256, 32, 2, 2, 5"), (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3")])
+                                          (4, "192, 256, 32, 2, 2, 5"), (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3"),
+                                          (7, "256, 256, 32, 2, 4, 5"), (8, "128, 128, 64, 2, 4, 3"), (9, "256, 128, 64, 2, 4, 3")])
 def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
     """Every straight-line epilogue class of the direct-to-LDS kernel on every tile shape, ragged in M
     (and in N against the 256- and 192-wide tiles), against the oracle; the launch names the class."""
@@ -171,7 +172,8 @@ def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 5"), (2, "256, 128, 64, 2, 2, 3"), (3, "128, 128, 64, 2, 2, 3"),
-                                          (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3")])
+                                          (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3"), (7, "256, 256, 32, 2, 4, 5"),
+                                          (8, "128, 128, 64, 2, 4, 3"), (9, "256, 128, 64, 2, 4, 3")])
 def test_gemm_direct_to_lds_weight_gradient_tiles(hip, oracle, dtype, variant, tile):
     """The reduction-strided (weight-gradient) form of every tile that has one: dW += dY^T X with a
     ragged reduction length (not a multiple of any stage depth) and ragged M and N, fp32 accumulate
@@ -194,7 +196,7 @@ def test_gemm_direct_to_lds_weight_gradient_tiles(hip, oracle, dtype, variant, t
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("variant,bm", [(1, 256), (2, 256), (3, 128), (4, 192), (5, 128), (6, 256)])
+@pytest.mark.parametrize("variant,bm", [(1, 256), (2, 256), (3, 128), (4, 192), (5, 128), (6, 256), (7, 256), (8, 128), (9, 256)])
 def test_gemm_gelu_grad_epilogue_leaves_column_sums(hip, dtype, variant, bm):
     """The GELU' epilogue of the direct-to-LDS kernel can also leave the column sums of the values it
     stores (the bias gradient of the layer whose pre-activation gradient it writes) as one partial row

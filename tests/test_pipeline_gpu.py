@@ -156,10 +156,10 @@ def test_vit_l_width_fp16_headline_geometry():
     m, r, l, rl, runner = _run_vit(cfg, 64, 4, "blocks.2", "fp16", oracle_device="cuda")
     _check(m, r, l, rl, "fp16")
     names = _gemm_variants(runner)
-    want = ["gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 2>",    # fc1: GELU epilogue
-            "gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 5>",    # dX of fc2: GELU' epilogue
-            "gemm16x_kernel<1, 128, 128, 64, 2, 2, 3, false, false, 3>",    # proj / fc2: fp32 residual epilogue
-            "gemm16x_kernel<1, 128, 128, 64, 2, 2, 3, true, true, 4>"]      # weight gradients, accumulated
+    want = ["gemm16x_kernel<1, 256, 256, 32, 2, 4, 5, false, false, 2>",    # fc1: GELU epilogue
+            "gemm16x_kernel<1, 256, 256, 32, 2, 4, 5, false, false, 5>",    # dX of fc2: GELU' epilogue
+            "gemm16x_kernel<1, 128, 128, 64, 2, 4, 3, false, false, 3>",    # proj / fc2: fp32 residual epilogue
+            "gemm16x_kernel<1, 128, 128, 64, 2, 4, 3, true, true, 4>"]      # weight gradients, accumulated
     for w in want:
         assert w in names, (w, sorted(names))
 
@@ -1311,15 +1311,17 @@ def test_dynamic_loss_scale_with_an_optimizer_that_keeps_pytorchs_step():
     assert float(runner.worker.scaler_state[3]) == 4.0        # four completed steps, one skipped
 
 
-def test_fp16_defaults_to_dynamic_loss_scaling():
-    """mixed_precision="fp16" without an explicit loss_scale runs the device-side scaler (the
-    reference wraps fp16 training in a GradScaler, pfeife/mp/worker.py:133-145)."""
+@pytest.mark.parametrize("mixed", ["fp16", "bf16"])
+def test_mixed_precision_defaults_to_dynamic_loss_scaling(mixed):
+    """mixed_precision without an explicit loss_scale runs the device-side scaler, for fp16 and
+    bf16 alike (the reference wraps every mixed-precision run in a GradScaler,
+    pfeife/mp/worker.py:133-145)."""
     from pfeife_amd.bench_models.vit import ViTConfig
 
     cfg = ViTConfig(image_size=32, patch_size=16, dim=64, depth=2, heads=4, mlp_dim=128, num_classes=16)
-    m, r, l, rl, runner = _run_vit(cfg, 8, 2, "blocks.1", "fp16")
+    m, r, l, rl, runner = _run_vit(cfg, 8, 2, "blocks.1", mixed)
     assert runner.worker.dyn_scale and runner.worker.scaler_state is not None
-    _check(m, r, l, rl, "fp16")     # gradients leave the step unscaled
+    _check(m, r, l, rl, mixed)     # gradients leave the step unscaled
 
 
 def test_split_then_merge_round_trip_on_device():
