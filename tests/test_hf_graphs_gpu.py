@@ -4,6 +4,7 @@
 one optimisation step under mixed precision against plain PyTorch autocast on the same GPU
 (losses within 2e-2 relative, every parameter's gradient within 2.5e-2 relative L2)."""
 import copy
+import gc
 
 import pytest
 import torch
@@ -16,7 +17,18 @@ def _fresh_runner(option):
     from pfeife_amd.mp import PartialRunner, initialize_pfeife
     from pfeife_amd.mp import net_states
 
+    from pfeife_amd.mp.partial.module import PartialModule
+
+    # the previous test's programs (tens of GB of preallocated buffers at the full-size
+    # configurations) stay reachable through the compiled modules until they are released
+    old = PartialModule._runner
+    if old is not None and getattr(old, "worker", None) is not None:
+        old.worker.release()
+        old.exec_fn = None
+    PartialModule._runner = None
     torch._dynamo.reset()
+    gc.collect()
+    torch.cuda.empty_cache()
     net_states._reset_state_for_tests()
     initialize_pfeife()
     return PartialRunner(option)

@@ -7,6 +7,7 @@ Tolerances (from the task's north star): micro-batch split bit-exact; loss withi
 max|d| <= 1e-4 * max|g| per tensor, 16-bit relative L2 <= 2e-2 per tensor
 (fp32 accumulation of 16-bit products on both sides)."""
 import copy
+import gc
 
 import pytest
 import torch
@@ -19,7 +20,18 @@ def _fresh_runner(option):
     from pfeife_amd.mp import PartialRunner, initialize_pfeife
     from pfeife_amd.mp import net_states
 
+    from pfeife_amd.mp.partial.module import PartialModule
+
+    # the previous test's programs (tens of GB of preallocated buffers at the full-size
+    # configurations) stay reachable through the compiled modules until they are released
+    old = PartialModule._runner
+    if old is not None and getattr(old, "worker", None) is not None:
+        old.worker.release()
+        old.exec_fn = None
+    PartialModule._runner = None
     torch._dynamo.reset()
+    gc.collect()
+    torch.cuda.empty_cache()
     net_states._reset_state_for_tests()
     initialize_pfeife()
     return PartialRunner(option)
