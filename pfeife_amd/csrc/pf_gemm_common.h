@@ -209,14 +209,7 @@ enum {
   EC_DACT16 = 5,   // C 16-bit, multiplied by GELU'(aux_in)
   EC_ACC16 = 6,    // C 16-bit accumulated in place (beta = 1)
   EC_RES16 = 7,    // C 16-bit, residual of the same 16-bit dtype added (a 16-bit residual stream)
-  EC_ATOM32 = 8,   // C fp32 accumulated in place by no-return atomic adds (weight gradients; see acc_atomic())
 };
-// PF_GEMM_ACC_ATOMIC=1: weight-gradient products add their tile to C with buffer_atomic_add_f32
-// instead of load + add + store (measurement aid, read once)
-inline bool acc_atomic() {
-  static const bool on = [] { const char* e = getenv("PF_GEMM_ACC_ATOMIC"); return e && e[0] == '1'; }();
-  return on;
-}
 // Epilogue class of a problem (see the EC_* list): the straight-line classes need 16-byte
 // vector access to every epilogue operand, whole 8-column groups, and 32-bit byte offsets.
 inline int epi_class(const pf_gemm_desc& d, int vec_ok) {

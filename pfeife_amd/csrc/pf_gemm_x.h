@@ -366,14 +366,14 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
     // rows are issued before the stores of the current ones, and since the counter retires in
     // order, "those loads have landed" is "at most <the operations issued after them>
     // outstanding", a compile-time number because nothing here is predicated.
-    constexpr bool C32 = EC == EC_STORE32 || EC == EC_RES32 || EC == EC_ACC32 || EC == EC_ATOM32;
+    constexpr bool C32 = EC == EC_STORE32 || EC == EC_RES32 || EC == EC_ACC32;
     constexpr bool LOADS = EC == EC_RES32 || EC == EC_ACC32 || EC == EC_DACT16 || EC == EC_ACC16 || EC == EC_RES16;
     constexpr bool LOAD32 = EC == EC_RES32 || EC == EC_ACC32;
     constexpr int HB = 16;                 // rows per step
     constexpr int NHB = TM * 2;            // steps
     constexpr int NP = HB / RPP;           // passes per step (a pass: every lane 8 columns of one row)
     constexpr int LPP = LOADS ? (LOAD32 ? 2 : 1) : 0;               // load instructions per pass
-    constexpr int SPP = (EC == EC_ATOM32 ? 8 : (C32 ? 2 : 1)) + (EC == EC_ACT16 ? 1 : 0);   // store instructions per pass
+    constexpr int SPP = (C32 ? 2 : 1) + (EC == EC_ACT16 ? 1 : 0);   // store instructions per pass
     constexpr int ESC = C32 ? 4 : 2;
     constexpr int WAVE_LDS = HB * SLD * 4 + 2 * NP * 2 * 1024;      // stage + two operand buffers
     static_assert(NW * WAVE_LDS <= 160 * 1024, "epilogue patches exceed LDS");
@@ -490,15 +490,8 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
             lo[k] = __float_as_int(v[k]);
             hi[k] = __float_as_int(v[4 + k]);
           }
-          if constexpr (EC == EC_ATOM32) {
-            // every element of C is touched by exactly one lane of one workgroup per launch, and launches
-            // into one C are ordered by their stream: the sum is the same as with load + add + store
-#pragma unroll
-            for (int k = 0; k < 8; ++k) __builtin_amdgcn_raw_ptr_buffer_atomic_fadd_f32(v[k], rs_c, (int)(oc + 4 * k), 0, 0);
-          } else {
-            __builtin_amdgcn_raw_buffer_store_b128(lo, rs_c, (int)oc, 0, 0);
-            __builtin_amdgcn_raw_buffer_store_b128(hi, rs_c, (int)(oc + 16), 0, 0);
-          }
+          __builtin_amdgcn_raw_buffer_store_b128(lo, rs_c, (int)oc, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(hi, rs_c, (int)(oc + 16), 0, 0);
         } else {
           const v4i_t packed = pack16<DT>(v);
           if constexpr (EC == EC_DACT16) {   // sums run over the ROUNDED values, rows past M excluded
@@ -670,7 +663,7 @@ int launch16x(const pf_gemm_desc& d, hipStream_t st) {
   // transposed (reduction-strided) tiles exist for 128 and 256 rows only
   if constexpr ((BM == 128 || BM == 256) && (BN == 128 || BN == 256)) {
     if (d.a_trans && d.b_trans) {   // weight-gradient products
-      if (ec == EC_ACC32) return acc_atomic() ? PF_X(true, true, EC_ATOM32) : PF_X(true, true, EC_ACC32);
+      if (ec == EC_ACC32) return PF_X(true, true, EC_ACC32);
       if (ec == EC_STORE32) return PF_X(true, true, EC_STORE32);
       return PF_X(true, true, EC_GENERIC);
     }
@@ -706,8 +699,7 @@ int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
       ga.start[i] = blocks;
     }
     ga.n = n;
-    auto kern = acc_atomic() ? gemm16x_group_kernel<DT, BM, BN, BK, WGM, WGN, ST, true, true, EC_ATOM32>
-                             : gemm16x_group_kernel<DT, BM, BN, BK, WGM, WGN, ST, true, true, EC_ACC32>;
+    auto kern = gemm16x_group_kernel<DT, BM, BN, BK, WGM, WGN, ST, true, true, EC_ACC32>;
     if (lds > 64 * 1024) {
       static std::mutex mu;
       static bool raised[64] = {};
