@@ -272,7 +272,11 @@ def gemm_ceiling(kernels, mixed, reps=20):
     replays, HIP events) the 256x256-tile direct-to-LDS kernel on 8192^3, one of the step's own
     products ([3152 x 1024] . [1024 x 4096], the MLP's first layer, plain 16-bit store) and the same
     product with a four times longer reduction, plus the 128x128 tile on the step's dominant
-    shape ([3152 x 4096] . [4096 x 1024]) and on that shape with 16 times the rows."""
+    shape ([3152 x 4096] . [4096 x 1024]) and on that shape with 16 times the rows.  The first entry
+    is no product at all: the tile's matrix-instruction stream alone on register-resident fragments
+    of the same random data (`pf_mfma_rate`, no loads, LDS or barriers), on every CU for about as
+    long as the 8192^3 product runs: what the MFMA pipes sustain under the board's power limit, the
+    attainable ceiling the published peak (full boost clock) overstates."""
     import torch
 
     dt = {"fp16": torch.float16, "bf16": torch.bfloat16}.get(mixed)
@@ -281,20 +285,37 @@ def gemm_ceiling(kernels, mixed, reps=20):
     st = torch.cuda.Stream()
     s = st.cuda_stream
     out = []
-    for label, M, N, K, variant in (("8192^3, 256x256 tile", 8192, 8192, 8192, 1),
-                                    ("step shape 3152x4096x1024, 256x256 tile", 3152, 4096, 1024, 1),
-                                    ("same with K x4 (3152x4096x4096), 256x256 tile", 3152, 4096, 4096, 1),
-                                    ("step shape 3152x1024x4096, 128x128 tile", 3152, 1024, 4096, 3),
-                                    ("same with M x16 (50432x1024x4096), 128x128 tile", 50432, 1024, 4096, 3),
-                                    ("same with M x16 (50432x1024x4096), 256x256 tile", 50432, 1024, 4096, 1)):
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    frags = torch.cat([torch.randn(2048, device="cuda"), torch.randn(2048, device="cuda") * 0.03]).to(dt)
+    wgs, iters = 1024, 512          # 4 workgroups per CU in turn, 8192 MFMAs per wavefront: the 8192^3 product's count
+    sink = torch.empty(256 * wgs, device="cuda", dtype=torch.float32)
+    rate = kernels.mfma_rate(frags, iters, wgs, sink)
+    torch.cuda.synchronize()        # operands were made on the current stream, the launches go to `st`
+    rate(s)
+    ev0.record(st)
+    for _ in range(reps):
+        rate(s)
+    ev1.record(st)
+    ev1.synchronize()
+    us = 1e3 * ev0.elapsed_time(ev1) / reps
+    tf = wgs * 4 * iters * 16 * 2.0 * 32 * 32 * 16 / us / 1e6
+    out.append(dict(shape="MFMA instruction stream only (no operand traffic), %d workgroups x 4 wavefronts x %d MFMAs" % (wgs, iters * 16),
+                    kernel="mfma_rate_kernel<%d>" % {"fp16": 1, "bf16": 2}[mixed], avg_launch_us=round(us, 2),
+                    tflops=round(tf, 1), frac=round(tf / PEAK_TFLOPS[mixed], 4)))
+    for label, M, N, K, variant in (("8192^3, 256x256 tile", 8192, 8192, 8192, 7),
+                                    ("step shape 3152x4096x1024, 256x256 tile", 3152, 4096, 1024, 7),
+                                    ("same with K x4 (3152x4096x4096), 256x256 tile", 3152, 4096, 4096, 7),
+                                    ("step shape 3152x1024x4096, 128x128 tile", 3152, 1024, 4096, 8),
+                                    ("same with M x16 (50432x1024x4096), 128x128 tile", 50432, 1024, 4096, 8),
+                                    ("same with M x16 (50432x1024x4096), 256x256 tile", 50432, 1024, 4096, 7)):
         x = torch.randn(M, K, device="cuda", dtype=dt)
         w = torch.randn(N, K, device="cuda", dtype=dt) * 0.03
         c = torch.empty(M, N, device="cuda", dtype=dt)
         n = 4 if M * N * K > 1e11 else 16
+        torch.cuda.synchronize()
         chain = [kernels.gemm(x, w, c, M=M, N=N, K=K, lda=K, ldb=K, ldc=N, variant=variant) for _ in range(n)]
         graph = kernels.capture(chain, s)
         graph(s)
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ev0.record(st)
         for _ in range(reps):
             graph(s)

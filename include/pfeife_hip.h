@@ -128,9 +128,11 @@ typedef struct pf_gemm_desc {
   int64_t ld_res;
   int32_t res_dtype;
   int32_t variant; /* 0: automatic tile choice; otherwise one kernel variant by id (tuning
-                      harnesses): 1..6 direct-to-LDS kernel with 256x256 / 256x128 / 128x128 /
-                      192x256 tiles and the two-workgroups-per-CU 128x128 / 256x128 tiles
-                      (32-deep stages), 11..14 register-staged kernel with 128x128 (8 wavefronts),
+                      harnesses): 1..4 direct-to-LDS kernel with 256x256 / 256x128 / 128x128 /
+                      192x256 tiles shared by four wavefronts, 5 / 6 its 128x128 / 256x128 tiles
+                      with eight wavefronts as two grids that split each tile step's reduction
+                      depth, 7 / 8 / 9 its 256x256 / 128x128 / 256x128 tiles with eight
+                      wavefronts side by side, 11..14 register-staged kernel with 128x128 (8 wavefronts),
                       128x128, 128x64, 64x64 tiles; PF_ERR_INVALID if it cannot run the problem */
   float* colsum_ws; /* optional, with dact on the direct-to-LDS kernel (pf_gemm_variant ends in ", 5>"): the
                        launch also leaves the column sums of the 16-bit values it stores in C as partial
@@ -150,10 +152,16 @@ int pf_gemm(const pf_gemm_desc* desc, void* stream);
  * as by pf_gemm, in order.  The products of one call must not depend on each other's results.
  * torch.autograd issues the same products one by one (pfeife/mp/worker.py:1585-1587). */
 int pf_gemm_grouped(const pf_gemm_desc* descs, int n, void* stream);
+/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of 4 wavefronts each issue
+ * iters * 16 v_mfma_f32_32x32x16 instructions (2 * 32 * 32 * 16 FLOP each) on register-resident
+ * fragments taken from `operands` (8 KiB of 16-bit values: 4 A fragments of 64 lanes x 8 values, then
+ * 4 B fragments), with no loads, LDS traffic or barriers in the loop: the rate the matrix pipes
+ * sustain under the board's power limit, the ceiling of any GEMM K loop.  sink: 256 * workgroups floats (per-lane checksums). */
+int pf_mfma_rate(int dtype, const void* operands, int64_t iters, int workgroups, float* sink, void* stream);
 /* Name of the kernel instantiation pf_gemm would launch for `desc`, spelled the
- * way a profiler prints it, e.g. "gemm16x_kernel<1, 256, 256, 32, 2, 2, 5, false, false, 0>"
- * (dtype, tile M, tile N, stage depth, wavefront grid, stages, a_trans, b_trans, epilogue
- * class) or "gemm16_kernel<1, 128, 64, 64, 2, 2, false, true>".  Lets a harness attribute
+ * way a profiler prints it, e.g. "gemm16x_kernel<1, 256, 256, 32, 2, 4, 1, 5, false, false, 0>"
+ * (dtype, tile M, tile N, stage depth, wavefront rows, columns, reduction split, stages, a_trans,
+ * b_trans, epilogue class) or "gemm16_kernel<1, 128, 64, 64, 2, 2, false, true>".  Lets a harness attribute
  * measured kernel time to problem shapes.  No counterpart in the reference. */
 int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap);
 

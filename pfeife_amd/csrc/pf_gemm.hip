@@ -616,9 +616,10 @@ int launch16(const pf_gemm_desc& d, hipStream_t st) {
 }
 
 // Variant ids (pf_gemm_desc.variant; 0 = automatic):
-//   1..7   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128 / 192x256 / 128x128d / 256x128d / 256x256w8
+//   1..9   direct-to-LDS kernel, tiles PF_XT_256x256 / 256x128 / 128x128 / 192x256 / 128x128k2 / 256x128k2 /
+//          256x256w8 / 128x128w8 / 256x128w8
 //   11..14 register-staged kernel: 128x128 by 8 wavefronts, 128x128, 128x64, 64x64 by 4
-enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_X192x256 = 4, V_X128D = 5, V_X256x128D = 6, V_X256W8 = 7, V_X128W8 = 8, V_X256x128W8 = 9,
+enum { V_AUTO = 0, V_X256 = 1, V_X256x128 = 2, V_X128 = 3, V_X192x256 = 4, V_X128K2 = 5, V_X256x128K2 = 6, V_X256W8 = 7, V_X128W8 = 8, V_X256x128W8 = 9,
        V_R128W8 = 11, V_R128 = 12, V_R128x64 = 13, V_R64 = 14 };
 inline bool is_x_variant(int v) { return v >= V_X256 && v <= V_X256x128W8; }
 
@@ -655,23 +656,27 @@ bool x_supports(const pf_gemm_desc& d, int xt) {
 // are the eight-wavefront tiles (two wavefronts per SIMD: one's LDS reads, waits and barrier
 // arrivals run under the other's MFMAs; 4-13 % faster than the same tiles shared by four
 // wavefronts on every shape of the five workloads) and the 192x256 tile for outputs that 256-wide
-// row blocks cover badly.  On a sweep of 21 forward / input-gradient shapes of the workloads the
-// choice is the fastest variant or within 3 % of it.
+// row blocks cover badly; for long reductions (from about 4300 deep on a single round of tiles) the
+// 256x128 tile whose eight wavefronts split every tile step's depth between two 2 x 2 grids: its
+// K loop is 4-8 % faster (each wavefront reads half the fragment bytes from LDS per MFMA), the
+// exchange of partial sums before the epilogue costs about 3 us.  On a sweep of 21 forward /
+// input-gradient shapes of the workloads the choice is the fastest variant or within 3 % of it.
 int choose_variant(const pf_gemm_desc& d) {
   const int64_t nb = d.batch1 * d.batch2;
   if (d.M < 128 || d.N < 128 || d.M * d.N < 128 * 128 * 16) return choose_staged(d);
-  struct Cand { int v, xt, bm, bn; double t64, t64_busy; };
-  static const Cand cands[4] = {{V_X256W8, PF_XT_256x256w8, 256, 256, 1.20, 1.20},
-                                {V_X192x256, PF_XT_192x256, 192, 256, 1.05, 1.05},
-                                {V_X256x128W8, PF_XT_256x128w8, 256, 128, 0.70, 0.70},
-                                {V_X128W8, PF_XT_128x128w8, 128, 128, 0.45, 0.55}};
+  struct Cand { int v, xt, bm, bn; double t64, t64_busy, fixed; };
+  static const Cand cands[5] = {{V_X256W8, PF_XT_256x256w8, 256, 256, 1.20, 1.20, 8.0},
+                                {V_X192x256, PF_XT_192x256, 192, 256, 1.05, 1.05, 8.0},
+                                {V_X256x128W8, PF_XT_256x128w8, 256, 128, 0.70, 0.70, 8.0},
+                                {V_X256x128K2, PF_XT_256x128k2, 256, 128, 0.655, 0.655, 11.0},
+                                {V_X128W8, PF_XT_128x128w8, 128, 128, 0.45, 0.55, 8.0}};
   int best = -1;
   double best_t = 0;
   for (const Cand& c : cands) {
     if (!x_supports(d, c.xt)) continue;
     const int64_t tiles = ((d.M + c.bm - 1) / c.bm) * ((d.N + c.bn - 1) / c.bn) * nb;
     const int64_t rounds = (tiles + 255) / 256;
-    const double t = 8.0 + (double)rounds * ((double)d.K / 64.0) * (tiles > 256 ? c.t64_busy : c.t64);
+    const double t = c.fixed + (double)rounds * ((double)d.K / 64.0) * (tiles > 256 ? c.t64_busy : c.t64);
     if (best < 0 || t < best_t) { best = c.v; best_t = t; }
   }
   return best < 0 ? choose_staged(d) : best;
@@ -710,7 +715,7 @@ int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
     }
   }
   switch (v) {
-    case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128D: case V_X256x128D: case V_X256W8: case V_X128W8: case V_X256x128W8: {
+    case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128K2: case V_X256x128K2: case V_X256W8: case V_X128W8: case V_X256x128W8: {
       const int xt = v;   // variant ids 1..7 are the PF_XT_* tile ids
       if (!x_supports(d, xt)) {
         pf_set_error("pf_gemm: variant %d needs both operands stored alike and (unless transposed) K a multiple of the stage depth", v);
@@ -886,10 +891,11 @@ extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
   const char* bt = d.b_trans ? "true" : "false";
   const int v = resolve_variant(d);
   switch (v) {
-    case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128D: case V_X256x128D: case V_X256W8: case V_X128W8: case V_X256x128W8: {
-      static const char* shapes[PF_XT_COUNT] = {"", "256, 256, 32, 2, 2, 5", "256, 128, 64, 2, 2, 3", "128, 128, 64, 2, 2, 3",
-                                                "192, 256, 32, 2, 2, 5", "128, 128, 32, 2, 2, 4", "256, 128, 32, 2, 2, 3",
-                                                "256, 256, 32, 2, 4, 5", "128, 128, 64, 2, 4, 3", "256, 128, 64, 2, 4, 3"};
+    case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128K2: case V_X256x128K2: case V_X256W8: case V_X128W8: case V_X256x128W8: {
+      // BM, BN, BK, wavefront rows, columns, reduction split, stages: as rocprofv3 prints the instantiation
+      static const char* shapes[PF_XT_COUNT] = {"", "256, 256, 32, 2, 2, 1, 5", "256, 128, 64, 2, 2, 1, 3", "128, 128, 64, 2, 2, 1, 3",
+                                                "192, 256, 32, 2, 2, 1, 5", "128, 128, 64, 2, 2, 2, 3", "256, 128, 64, 2, 2, 2, 3",
+                                                "256, 256, 32, 2, 4, 1, 5", "128, 128, 64, 2, 4, 1, 3", "256, 128, 64, 2, 4, 1, 3"};
       if (!x_supports(d, v)) {   // a pinned tile that cannot run this product: say so here, not at launch time
         pf_set_error("pf_gemm_variant: variant %d needs both operands stored alike, K >= %d and (unless both are "
                      "reduction-strided) K a multiple of %d", v, x_tile_bk(v), x_tile_bk(v));

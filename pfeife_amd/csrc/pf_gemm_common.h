@@ -173,29 +173,27 @@ __device__ __forceinline__ uint4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t b
   return make_uint4((uint32_t)x.x, (uint32_t)x.y, (uint32_t)x.z, (uint32_t)x.w);
 }
 
-// Tile shapes of the direct-to-LDS kernel (BM x BN; reduction depth per stage, stages):
+// Tile shapes of the direct-to-LDS kernel (BM x BN; reduction depth per stage, stages; wavefronts):
 //   256x256 (32 deep, 5 stages): one 128x128 block per wavefront, the least operand traffic per FLOP
 //   256x128 (64 deep, 3 stages), 128x128 (64 deep, 3 stages): more workgroups for smaller outputs
-//   128x128 (32 deep, 4 stages; 64 KB) and 256x128 (32 deep, 3 stages; 72 KB): "d" tiles, small enough
-//   in LDS and registers for TWO workgroups per CU, so that workgroups of kernels launched on
-//   different streams share a CU and one's prologue and epilogue run under the other's reduction loop
-//   256x256w8: the 256x256 tile shared by EIGHT wavefronts (2 x 4, 128x64 each, two per SIMD)
-enum { PF_XT_256x256 = 1, PF_XT_256x128 = 2, PF_XT_128x128 = 3, PF_XT_192x256 = 4, PF_XT_128x128d = 5,
-       PF_XT_256x128d = 6, PF_XT_256x256w8 = 7, PF_XT_128x128w8 = 8, PF_XT_256x128w8 = 9, PF_XT_COUNT = 10 };
-// BM, BN, reduction depth per stage, stages, wavefront grid of each tile id
+//   192x256 (32 deep, 5 stages): for outputs that 256-row blocks cover badly
+//   ids 1-4: four wavefronts (2 x 2); ids 7-9: the same tiles shared by EIGHT wavefronts (2 x 4,
+//   two per SIMD); ids 5, 6: 128x128 and 256x128 with eight wavefronts as TWO 2 x 2 grids that
+//   split every tile's reduction depth between them ("k2")
+enum { PF_XT_256x256 = 1, PF_XT_256x128 = 2, PF_XT_128x128 = 3, PF_XT_192x256 = 4, PF_XT_128x128k2 = 5,
+       PF_XT_256x128k2 = 6, PF_XT_256x256w8 = 7, PF_XT_128x128w8 = 8, PF_XT_256x128w8 = 9, PF_XT_COUNT = 10 };
+// BM, BN, reduction depth per stage, stages, wavefront grid (rows x columns x reduction split) of each tile id
 template <int XT> struct XTile;
-template <> struct XTile<PF_XT_256x256> { static constexpr int BM = 256, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 2; };
-template <> struct XTile<PF_XT_256x128> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2; };
-template <> struct XTile<PF_XT_128x128> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2; };
-template <> struct XTile<PF_XT_192x256> { static constexpr int BM = 192, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 2; };
-template <> struct XTile<PF_XT_128x128d> { static constexpr int BM = 128, BN = 128, BK = 32, ST = 4, WGM = 2, WGN = 2; };
-template <> struct XTile<PF_XT_256x128d> { static constexpr int BM = 256, BN = 128, BK = 32, ST = 3, WGM = 2, WGN = 2; };
-template <> struct XTile<PF_XT_256x256w8> { static constexpr int BM = 256, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 4; };
-template <> struct XTile<PF_XT_128x128w8> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 4; };
-template <> struct XTile<PF_XT_256x128w8> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 4; };
-inline int x_tile_bk(int xt) {
-  return (xt == PF_XT_256x128 || xt == PF_XT_128x128 || xt == PF_XT_128x128w8 || xt == PF_XT_256x128w8) ? 64 : 32;
-}
+template <> struct XTile<PF_XT_256x256> { static constexpr int BM = 256, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 2, KS = 1; };
+template <> struct XTile<PF_XT_256x128> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2, KS = 1; };
+template <> struct XTile<PF_XT_128x128> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2, KS = 1; };
+template <> struct XTile<PF_XT_192x256> { static constexpr int BM = 192, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 2, KS = 1; };
+template <> struct XTile<PF_XT_128x128k2> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2, KS = 2; };
+template <> struct XTile<PF_XT_256x128k2> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2, KS = 2; };
+template <> struct XTile<PF_XT_256x256w8> { static constexpr int BM = 256, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 4, KS = 1; };
+template <> struct XTile<PF_XT_128x128w8> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 4, KS = 1; };
+template <> struct XTile<PF_XT_256x128w8> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 4, KS = 1; };
+inline int x_tile_bk(int xt) { return (xt == PF_XT_256x256 || xt == PF_XT_192x256 || xt == PF_XT_256x256w8) ? 32 : 64; }
 
 // Epilogue classes with straight-line code (which operands exist, and their dtypes, fixed at
 // compile time).  Everything else takes EC_GENERIC: one rolled loop with runtime switches.

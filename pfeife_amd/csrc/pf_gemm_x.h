@@ -98,19 +98,21 @@ template <int R, int BK, int NW, bool TRANS> struct DTile {
   //   [row][k]: foff[kk] = byte offset of (row w0 + lane%32, chunk 2*kk + lane/32); + i*32*ROWB per MFMA tile
   //   [k][row]: foff[i]  = byte offset for MFMA tile i at kk = 0, first half; + (16*kk + 4*h)*ROWB
   static constexpr int NOFF_T = 4;
+  // kk0: first 16-deep MFMA group of a tile that this wavefront multiplies (wavefronts that split
+  // a tile's reduction depth between them start at different groups)
   template <int NF>
-  static __device__ __forceinline__ void frag_init(uint32_t (&foff)[NF], int w0, int lane) {
+  static __device__ __forceinline__ void frag_init(uint32_t (&foff)[NF], int w0, int lane, int kk0) {
     if constexpr (!TRANS) {
       const int row = w0 + (lane & 31), half = lane >> 5;
 #pragma unroll
-      for (int kk = 0; kk < NF; ++kk) foff[kk] = (uint32_t)(row * ROWB + (((kk * 2 + half) ^ swz_row(row)) * 16));
+      for (int kk = 0; kk < NF; ++kk) foff[kk] = (uint32_t)(row * ROWB + ((((kk0 + kk) * 2 + half) ^ swz_row(row)) * 16));
     } else {
       const int g = lane >> 4, j = lane & 15;
       const int k = (g >> 1) * 8 + (j >> 2);
 #pragma unroll
       for (int i = 0; i < NF; ++i) {
         const int m = w0 + i * 32 + (g & 1) * 16 + 4 * (j & 3);
-        foff[i] = (uint32_t)(k * ROWB + (((m >> 3) ^ swz_k(k)) * 16) + (m & 7) * 2);
+        foff[i] = (uint32_t)((k + kk0 * 16) * ROWB + (((m >> 3) ^ swz_k(k)) * 16) + (m & 7) * 2);
       }
     }
   }
@@ -170,12 +172,21 @@ template <int DT> __device__ __forceinline__ v4i_t pack16(const float8_t& v) {
 
 // `pid`: index of this workgroup among the workgroups of its problem (the launch may hold several
 // problems, see gemm16x_group_kernel)
-template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int KS, int ST, bool AT, bool BT, int EC>
 __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGrid& g, const int pid) {
-  constexpr int NW = WGM * WGN;
+  // KS = 2: the wavefronts form two WGM x WGN grids; grid h multiplies the h-th half of every
+  // tile's 16-deep MFMA groups, and the two partial accumulator blocks are added through LDS
+  // before the epilogue.  Eight wavefronts (two per SIMD, so that one's LDS reads and waits run
+  // under the other's MFMAs) then read no more fragment bytes from LDS than four do, and the
+  // LDS port (128 B/clk per CU for fragment reads and arriving tiles together) is what bounds
+  // these tiles.
+  constexpr int NWMN = WGM * WGN;
+  constexpr int NW = NWMN * KS;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int TM = WM / 32, TN = WN / 32;
-  constexpr int KK = BK / 16;
+  constexpr int KK = BK / 16 / KS;     // MFMA groups per tile and wavefront
+  static_assert(KS == 1 || KS == 2, "the reduction depth of a tile is split over one or two wavefront grids");
+  static_assert((BK / 16) % KS == 0, "MFMA groups do not divide over the wavefront grids");
   using TA = DTile<BM, BK, NW, AT>;
   using TB = DTile<BN, BK, NW, BT>;
   constexpr int STAGE = TA::BYTES + TB::BYTES;
@@ -200,7 +211,8 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / WGN) * WM, wn0 = (wave % WGN) * WN;
+  const int wave_k = wave / NWMN, wave_mn = wave % NWMN;
+  const int wm0 = (wave_mn / WGN) * WM, wn0 = (wave_mn % WGN) * WN;
   const uint32_t lds0 = (uint32_t)(uintptr_t)smem;
 
   float16_t acc[TM][TN];
@@ -218,8 +230,8 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
   TB::init(offb, ldb, n0, wave, lane);
   const uint32_t step_a = TA::tile_step(lda), step_b = TB::tile_step(ldb);
   uint32_t foa[NFA], fob[NFB];
-  TA::template frag_init<NFA>(foa, wm0, lane);
-  TB::template frag_init<NFB>(fob, wn0, lane);
+  TA::template frag_init<NFA>(foa, wm0, lane, wave_k * KK);
+  TB::template frag_init<NFB>(fob, wn0, lane, wave_k * KK);
 
   const int nk = (int)((K + BK - 1) / BK);
 
@@ -349,8 +361,34 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
   // of a few tens of microseconds cannot afford to stream 100 KB of unrolled epilogue code
   // through the instruction cache, which starts cold at every launch.
   lds_barrier();  // every wavefront is done with the operand tiles
+  if constexpr (KS == 2) {
+    // the second grid hands its partial sums over (16 bytes per lane, lanes side by side: no bank
+    // conflicts) and leaves; a barrier only counts the wavefronts that are still running
+    float4* xch = (float4*)smem + wave_mn * (TM * TN * 4 * 64) + lane;
+    if (wave_k == 1) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            xch[((i * TN + j) * 4 + q) * 64] = make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+    }
+    lds_barrier();
+    if (wave_k == 1) return;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float4 t = xch[((i * TN + j) * 4 + q) * 64];
+          acc[i][j][4 * q] += t.x; acc[i][j][4 * q + 1] += t.y; acc[i][j][4 * q + 2] += t.z; acc[i][j][4 * q + 3] += t.w;
+        }
+    lds_barrier();  // all partial sums are read before the epilogue patches overwrite them
+  }
   constexpr int SLD = WN + 8;        // floats per staged row: lanes 32..63 (4 rows down) land 32 banks away
-  constexpr int RB = epi_row_blocks(NW, WN, TM);   // 32-row blocks staged together
+  constexpr int RB = epi_row_blocks(NWMN, WN, TM);   // 32-row blocks staged together
   float* stage = (float*)smem + wave * (RB * 32 * SLD);
   const int wr_off = ((lane >> 5) * 4) * SLD + (lane & 31);
 
@@ -376,7 +414,7 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
     constexpr int SPP = (C32 ? 2 : 1) + (EC == EC_ACT16 ? 1 : 0);   // store instructions per pass
     constexpr int ESC = C32 ? 4 : 2;
     constexpr int WAVE_LDS = HB * SLD * 4 + 2 * NP * 2 * 1024;      // stage + two operand buffers
-    static_assert(NW * WAVE_LDS <= 160 * 1024, "epilogue patches exceed LDS");
+    static_assert(NWMN * WAVE_LDS <= 160 * 1024, "epilogue patches exceed LDS");
     static_assert(NP * (SPP + LPP) <= 63, "too many operations in flight for the 6-bit counter");
     float* stg = (float*)((char*)smem + wave * WAVE_LDS);
     const uint32_t raw0 = lds0 + (uint32_t)(wave * WAVE_LDS + HB * SLD * 4);
@@ -513,7 +551,7 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
         // is done with its own epilogue patch at the barrier; the patch of partial sums lies below
         // the first wavefront's operand buffers, which the last, unused prefetch may still be filling)
         float* red = (float*)smem;
-        static_assert(NW * WN * 4 <= HB * SLD * 4, "partial column sums overlap the operand buffers");
+        static_assert(NWMN * WN * 4 <= HB * SLD * 4, "partial column sums overlap the operand buffers");
         lds_barrier();
         if (lane < LPR) {
 #pragma unroll
@@ -573,10 +611,10 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
   __builtin_amdgcn_s_waitcnt(0x0F70);
 }
 
-#define PF_X_BOUNDS __launch_bounds__(64 * WGM * WGN, (ST * (BM + BN) * BK * 2 <= 80 * 1024 && 64 * WGM * WGN <= 256) ? 2 : 1)
-template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
+#define PF_X_BOUNDS __launch_bounds__(64 * WGM * WGN * KS, (ST * (BM + BN) * BK * 2 <= 80 * 1024 && 64 * WGM * WGN * KS <= 256) ? 2 : 1)
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int KS, int ST, bool AT, bool BT, int EC>
 __global__ PF_X_BOUNDS void gemm16x_kernel(const pf_gemm_desc p, const GemmGrid g) {
-  gemm16x_body<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>(p, g, (int)blockIdx.x);
+  gemm16x_body<DT, BM, BN, BK, WGM, WGN, KS, ST, AT, BT, EC>(p, g, (int)blockIdx.x);
 }
 
 // Several independent problems of the same kind in one launch: problem i owns the workgroups
@@ -590,26 +628,27 @@ struct GemmGroup {
   int start[GEMM_GROUP_MAX];
   int n;
 };
-template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int KS, int ST, bool AT, bool BT, int EC>
 __global__ PF_X_BOUNDS void gemm16x_group_kernel(const GemmGroup ga) {
   int i = 0;
 #pragma unroll
   for (int k = 1; k < GEMM_GROUP_MAX; ++k)
     if (k < ga.n && (int)blockIdx.x >= ga.start[k]) i = k;
   i = __builtin_amdgcn_readfirstlane(i);
-  gemm16x_body<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>(ga.p[i], ga.g[i], (int)blockIdx.x - ga.start[i]);
+  gemm16x_body<DT, BM, BN, BK, WGM, WGN, KS, ST, AT, BT, EC>(ga.p[i], ga.g[i], (int)blockIdx.x - ga.start[i]);
 }
 
-template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST, bool AT, bool BT, int EC>
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int KS, int ST, bool AT, bool BT, int EC>
 int launch16x_t(const pf_gemm_desc& d, const GemmGrid& g, hipStream_t st) {
-  constexpr int NT = 64 * WGM * WGN;
-  constexpr size_t lds_main = (size_t)ST * (BM + BN) * BK * 2;
+  constexpr int NT = 64 * WGM * WGN * KS;
+  constexpr size_t lds_xch = KS == 2 ? (size_t)BM * BN * 4 : 0;   // one grid's partial sums on their way to the other
+  constexpr size_t lds_main = ((size_t)ST * (BM + BN) * BK * 2 > lds_xch) ? (size_t)ST * (BM + BN) * BK * 2 : lds_xch;
   constexpr size_t lds_gen = (size_t)(WGM * WGN) * epi_row_blocks(WGM * WGN, BN / WGN, BM / WGM / 32) * 32 * (BN / WGN + 8) * sizeof(float);
   constexpr size_t lds_fast = (size_t)(WGM * WGN) * (16 * (BN / WGN + 8) * 4 + 2 * (16 / (64 / (BN / WGN / 8))) * 2 * 1024);
   constexpr size_t lds_epi = EC == EC_GENERIC ? lds_gen : lds_fast;
   constexpr size_t lds = lds_main > lds_epi ? lds_main : lds_epi;
   static_assert(lds <= 160 * 1024, "tile pipeline exceeds the 160 KB of LDS");
-  auto kern = gemm16x_kernel<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>;
+  auto kern = gemm16x_kernel<DT, BM, BN, BK, WGM, WGN, KS, ST, AT, BT, EC>;
   if (lds > 64 * 1024) {  // opt in to the large LDS carve-out once per instantiation and device
     static std::mutex mu;
     static bool raised[64] = {};
@@ -631,7 +670,7 @@ int launch16x_t(const pf_gemm_desc& d, const GemmGrid& g, hipStream_t st) {
   return PF_OK;
 }
 
-template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST>
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int KS, int ST>
 int launch16x(const pf_gemm_desc& d, hipStream_t st) {
   GemmGrid g;
   g.tiles_m = (int)((d.M + BM - 1) / BM);
@@ -646,7 +685,7 @@ int launch16x(const pf_gemm_desc& d, hipStream_t st) {
     return PF_ERR_INVALID;
   }
   const int ec = epi_class(d, g.vec_epi);
-#define PF_X(AT, BT, EC) launch16x_t<DT, BM, BN, BK, WGM, WGN, ST, AT, BT, EC>(d, g, st)
+#define PF_X(AT, BT, EC) launch16x_t<DT, BM, BN, BK, WGM, WGN, KS, ST, AT, BT, EC>(d, g, st)
   if (!d.a_trans && !d.b_trans) {   // forward and input-gradient products
     switch (ec) {
       case EC_STORE16: return PF_X(false, false, EC_STORE16);
@@ -675,11 +714,12 @@ int launch16x(const pf_gemm_desc& d, hipStream_t st) {
 
 // Several weight-gradient products (both operands reduction-strided, fp32 C accumulated) in one
 // launch; the caller has checked that they all take tile BMxBN and the EC_ACC32 epilogue.
-template <int DT, int BM, int BN, int BK, int WGM, int WGN, int ST>
+template <int DT, int BM, int BN, int BK, int WGM, int WGN, int KS, int ST>
 int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
   if constexpr ((BM == 128 || BM == 256) && (BN == 128 || BN == 256)) {
-    constexpr int NT = 64 * WGM * WGN;
-    constexpr size_t lds_main = (size_t)ST * (BM + BN) * BK * 2;
+    constexpr int NT = 64 * WGM * WGN * KS;
+    constexpr size_t lds_xch = KS == 2 ? (size_t)BM * BN * 4 : 0;
+    constexpr size_t lds_main = ((size_t)ST * (BM + BN) * BK * 2 > lds_xch) ? (size_t)ST * (BM + BN) * BK * 2 : lds_xch;
     constexpr size_t lds_fast = (size_t)(WGM * WGN) * (16 * (BN / WGN + 8) * 4 + 2 * (16 / (64 / (BN / WGN / 8))) * 2 * 1024);
     constexpr size_t lds = lds_main > lds_fast ? lds_main : lds_fast;
     GemmGroup ga;
@@ -699,7 +739,7 @@ int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
       ga.start[i] = blocks;
     }
     ga.n = n;
-    auto kern = gemm16x_group_kernel<DT, BM, BN, BK, WGM, WGN, ST, true, true, EC_ACC32>;
+    auto kern = gemm16x_group_kernel<DT, BM, BN, BK, WGM, WGN, KS, ST, true, true, EC_ACC32>;
     if (lds > 64 * 1024) {
       static std::mutex mu;
       static bool raised[64] = {};
@@ -727,12 +767,12 @@ int launch16x_group(const pf_gemm_desc* d, int n, hipStream_t st) {
 template <int DT, int XT>
 int gemm_x_group_launch(const pf_gemm_desc* d, int n, hipStream_t st) {
   using T = XTile<XT>;
-  return launch16x_group<DT, T::BM, T::BN, T::BK, T::WGM, T::WGN, T::ST>(d, n, st);
+  return launch16x_group<DT, T::BM, T::BN, T::BK, T::WGM, T::WGN, T::KS, T::ST>(d, n, st);
 }
 template <int DT, int XT>
 int gemm_x_launch(const pf_gemm_desc& d, hipStream_t st) {
   using T = XTile<XT>;
-  return launch16x<DT, T::BM, T::BN, T::BK, T::WGM, T::WGN, T::ST>(d, st);
+  return launch16x<DT, T::BM, T::BN, T::BK, T::WGM, T::WGN, T::KS, T::ST>(d, st);
 }
 
 }  // namespace

@@ -139,6 +139,7 @@ _SIGNATURES = {
     "pf_merge_scatter": [_P, _P, _L, _L, _L, _P, _P],
     "pf_embedding_fwd": [_P, _I, _P, _P, _I, _L, _L, _L, _P],
     "pf_embedding_bwd": [_P, _I, _P, _P, _L, _L, _L, _L, _P],
+    "pf_mfma_rate": [_I, _P, _L, _I, _P, _P],
 }
 _RET_I64 = {"pf_colreduce_workspace": [_L, _L], "pf_reduce_workspace": [_L], "pf_groupnorm_workspace": [_L, _L, _I],
             "pf_colsum_static_capacity": []}
@@ -598,6 +599,11 @@ class HipKernels:
 
     def fill(self, dst, value, n):
         return self._prep("pf_fill", (_ptr(dst), _dt(dst), float(value), n), (dst,))
+
+    def mfma_rate(self, operands, iters, workgroups, sink):
+        """Measurement aid: the GEMM tile's matrix-instruction stream alone (see pf_mfma_rate)."""
+        assert operands.numel() >= 4096 and sink.numel() >= 256 * workgroups and sink.dtype == torch.float32
+        return self._prep("pf_mfma_rate", (_dt(operands), _ptr(operands), int(iters), int(workgroups), _ptr(sink)), (operands, sink))
 
     def copy_strided(self, src, src_strides, dst, dst_strides, sizes, accumulate=0):
         nd = len(sizes)

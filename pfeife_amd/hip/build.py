@@ -24,10 +24,11 @@ SOURCES = [
     "pf_elementwise.hip",
     "pf_softmax_loss.hip",
     "pf_batch.hip",
+    "pf_mfma_rate.hip",
 ]
 
 # the direct-to-LDS MFMA kernel: one object per (operand dtype id, tile id), all from one source
-# (ids as in csrc/pf_gemm_common.h: dtypes PF_F16 = 1, PF_BF16 = 2; tiles PF_XT_* = 1..7)
+# (ids as in csrc/pf_gemm_common.h: dtypes PF_F16 = 1, PF_BF16 = 2; tiles PF_XT_* = 1..9)
 GEMM_X_SOURCE = "pf_gemm_x_inst.hip"
 GEMM_X_PAIRS = [(dt, xt) for xt in (1, 2, 3, 4, 5, 6, 7, 8, 9) for dt in (1, 2)]
 

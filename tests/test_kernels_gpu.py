@@ -123,9 +123,9 @@ def test_gemm_epilogues(hip, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 5"), (2, "256, 128, 64, 2, 2, 3"), (3, "128, 128, 64, 2, 2, 3"),
-                                          (4, "192, 256, 32, 2, 2, 5"), (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3"),
-                                          (7, "256, 256, 32, 2, 4, 5"), (8, "128, 128, 64, 2, 4, 3"), (9, "256, 128, 64, 2, 4, 3")])
+@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 1, 5"), (2, "256, 128, 64, 2, 2, 1, 3"), (3, "128, 128, 64, 2, 2, 1, 3"),
+                                          (4, "192, 256, 32, 2, 2, 1, 5"), (5, "128, 128, 64, 2, 2, 2, 3"), (6, "256, 128, 64, 2, 2, 2, 3"),
+                                          (7, "256, 256, 32, 2, 4, 1, 5"), (8, "128, 128, 64, 2, 4, 1, 3"), (9, "256, 128, 64, 2, 4, 1, 3")])
 def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
     """Every straight-line epilogue class of the direct-to-LDS kernel on every tile shape, ragged in M
     (and in N against the 256- and 192-wide tiles), against the oracle; the launch names the class."""
@@ -171,9 +171,9 @@ def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 5"), (2, "256, 128, 64, 2, 2, 3"), (3, "128, 128, 64, 2, 2, 3"),
-                                          (5, "128, 128, 32, 2, 2, 4"), (6, "256, 128, 32, 2, 2, 3"), (7, "256, 256, 32, 2, 4, 5"),
-                                          (8, "128, 128, 64, 2, 4, 3"), (9, "256, 128, 64, 2, 4, 3")])
+@pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 1, 5"), (2, "256, 128, 64, 2, 2, 1, 3"), (3, "128, 128, 64, 2, 2, 1, 3"),
+                                          (5, "128, 128, 64, 2, 2, 2, 3"), (6, "256, 128, 64, 2, 2, 2, 3"), (7, "256, 256, 32, 2, 4, 1, 5"),
+                                          (8, "128, 128, 64, 2, 4, 1, 3"), (9, "256, 128, 64, 2, 4, 1, 3")])
 def test_gemm_direct_to_lds_weight_gradient_tiles(hip, oracle, dtype, variant, tile):
     """The reduction-strided (weight-gradient) form of every tile that has one: dW += dY^T X with a
     ragged reduction length (not a multiple of any stage depth) and ragged M and N, fp32 accumulate
@@ -963,3 +963,21 @@ def test_weight_gradients_that_fill_the_device_together_share_a_launch_on_large_
             assert torch.equal(c_three[i], c_four[i])
     torch.testing.assert_close(c_one[0].double(), probs[0][2].double() + probs[0][0].double().t() @ probs[0][1].double(),
                                rtol=2e-3, atol=5e-2)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_mfma_rate_probe_multiplies_what_it_is_given(hip, dtype):
+    """The matrix-instruction rate probe (bench.py's attainable-ceiling record) really issues
+    iters * 16 MFMAs per wavefront on the fragments it is handed: every wavefront's 64 per-lane
+    checksums add up to iters * sum_{i,j} sum(A_i . B_j), computed here from the fragment layout of
+    v_mfma_f32_32x32x16 (lane l holds row or column l % 32 and reduction indices 8 * (l / 32) + 0..7).
+    Small integers keep every fp32 sum exact."""
+    g = torch.Generator().manual_seed(5)
+    frags = torch.randint(-2, 3, (8, 64, 8), generator=g).to(dtype)
+    iters, wgs = 7, 3
+    sink = torch.full((256 * wgs,), float("nan"), device="cuda")
+    hip.mfma_rate(frags.cuda(), iters, wgs, sink)(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    per_k = frags.double().reshape(8, 2, 32, 8).sum(2).reshape(8, 16)     # [fragment][k]: sum over its 32 rows / columns
+    want = iters * float((per_k[:4].sum(0) * per_k[4:].sum(0)).sum())
+    assert sink.cpu().double().reshape(4 * wgs, 64).sum(1).tolist() == [want] * (4 * wgs)
