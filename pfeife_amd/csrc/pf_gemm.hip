@@ -656,19 +656,21 @@ bool x_supports(const pf_gemm_desc& d, int xt) {
 // are the eight-wavefront tiles (two wavefronts per SIMD: one's LDS reads, waits and barrier
 // arrivals run under the other's MFMAs; 4-13 % faster than the same tiles shared by four
 // wavefronts on every shape of the five workloads) and the 192x256 tile for outputs that 256-wide
-// row blocks cover badly; for long reductions (from about 4300 deep on a single round of tiles) the
-// 256x128 tile whose eight wavefronts split every tile step's depth between two 2 x 2 grids: its
-// K loop is 4-8 % faster (each wavefront reads half the fragment bytes from LDS per MFMA), the
-// exchange of partial sums before the epilogue costs about 3 us.  On a sweep of 21 forward /
-// input-gradient shapes of the workloads the choice is the fastest variant or within 3 % of it.
+// row blocks cover badly.  On a sweep of 21 forward / input-gradient shapes of the workloads the
+// choice is the fastest variant or within 3 % of it, but for long reductions: from about 4300
+// deep on, the 256x128 tile whose eight wavefronts split every tile step's depth between two
+// 2 x 2 grids (variant 6) is 4-8 % faster when launches of one shape run back to back (each
+// wavefront reads half the fragment bytes from LDS per MFMA; the exchange of partial sums costs
+// about 3 us).  It is NOT a candidate: inside the pipeline step, with other streams' kernels
+// around it, the Llama and UNet-stage steps that would use it ran 0.7 % slower with it in two
+// A/B runs each, so it stays a variant that can be pinned.
 int choose_variant(const pf_gemm_desc& d) {
   const int64_t nb = d.batch1 * d.batch2;
   if (d.M < 128 || d.N < 128 || d.M * d.N < 128 * 128 * 16) return choose_staged(d);
   struct Cand { int v, xt, bm, bn; double t64, t64_busy, fixed; };
-  static const Cand cands[5] = {{V_X256W8, PF_XT_256x256w8, 256, 256, 1.20, 1.20, 8.0},
+  static const Cand cands[4] = {{V_X256W8, PF_XT_256x256w8, 256, 256, 1.20, 1.20, 8.0},
                                 {V_X192x256, PF_XT_192x256, 192, 256, 1.05, 1.05, 8.0},
                                 {V_X256x128W8, PF_XT_256x128w8, 256, 128, 0.70, 0.70, 8.0},
-                                {V_X256x128K2, PF_XT_256x128k2, 256, 128, 0.655, 0.655, 11.0},
                                 {V_X128W8, PF_XT_128x128w8, 128, 128, 0.45, 0.55, 8.0}};
   int best = -1;
   double best_t = 0;
