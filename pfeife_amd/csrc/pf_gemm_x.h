@@ -472,21 +472,27 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
       }
       const uint32_t rawb = raw0 + (uint32_t)((hb & 1) * NP * LPP) * 1024u + (uint32_t)lane * 16u;
       const uint32_t stg_addr = lds0 + (uint32_t)(wave * WAVE_LDS + (rd_row * SLD + rd_col) * 4);
-#pragma nounroll
+      // LDS reads by inline assembly: the compiler cannot tell these addresses from the
+      // destinations of the direct-to-LDS loads in flight and would wait for all of them (and,
+      // the counter being shared, for every store issued so far) before each ordinary read.
+      // The reads of all passes of a step are issued together and waited for once: a rolled
+      // pass loop exposed one LDS round trip per pass.
+      v4i_t sxs[NP], sys[NP], ras[NP], rbs[NP];
+#pragma unroll
       for (int pp = 0; pp < NP; ++pp) {
-        // LDS reads by inline assembly: the compiler cannot tell these addresses from the
-        // destinations of the direct-to-LDS loads in flight and would wait for all of them (and,
-        // the counter being shared, for every store issued so far) before each ordinary read
-        v4i_t sx, sy, ra, rb;
         const uint32_t sa = stg_addr + (uint32_t)((pp * RPP) * SLD * 4);
-        asm volatile("ds_read_b128 %0, %1" : "=v"(sx) : "v"(sa) : "memory");
-        asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(sy) : "v"(sa) : "memory");
+        asm volatile("ds_read_b128 %0, %1" : "=v"(sxs[pp]) : "v"(sa) : "memory");
+        asm volatile("ds_read_b128 %0, %1 offset:16" : "=v"(sys[pp]) : "v"(sa) : "memory");
         if constexpr (LOADS) {
           const uint32_t rp = rawb + (uint32_t)(pp * LPP) * 1024u;
-          asm volatile("ds_read_b128 %0, %1" : "=v"(ra) : "v"(rp) : "memory");
-          if constexpr (LOAD32) asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rb) : "v"(rp) : "memory");
+          asm volatile("ds_read_b128 %0, %1" : "=v"(ras[pp]) : "v"(rp) : "memory");
+          if constexpr (LOAD32) asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rbs[pp]) : "v"(rp) : "memory");
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+      for (int pp = 0; pp < NP; ++pp) {
+        const v4i_t sx = sxs[pp], sy = sys[pp], ra = ras[pp], rb = rbs[pp];
         float8_t v;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
@@ -494,9 +500,13 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
           v[4 + k] = __int_as_float(sy[k]);
         }
         v = v * alpha + bias8;
-        if (round_mid) {
+        // (the plain 16-bit store rounds once, when it packs: rounding to the same format before
+        // that changes nothing and cost 16 of the pass's 30 vector instructions)
+        if constexpr (EC != EC_STORE16) {
+          if (round_mid) {
 #pragma unroll
-          for (int k = 0; k < 8; ++k) v[k] = Codec<DT>::round(v[k]);
+            for (int k = 0; k < 8; ++k) v[k] = Codec<DT>::round(v[k]);
+          }
         }
         const uint32_t rowk = (uint32_t)(hb * HB + pp * RPP);
         if constexpr (EC == EC_ACT16) {   // GELU only (other activations take the generic class)
