@@ -135,6 +135,9 @@ def _step_launches(runner):
         for prog in slot.stage_programs.values():
             for launch in list(prog.fwd) + list(prog.bwd):
                 yield launch
+    for launches, _ in runner.worker.dw_jobs.values():   # the once-per-step weight-gradient job of each stage
+        for launch in launches:
+            yield launch
 
 
 def _time_launches(launches, reps):

@@ -235,6 +235,7 @@ class BufferPool:
         self.device = device
         self._scratch = {}
         self._bwd = {}
+        self._stacked = {}
         self.bytes = 0
         # Jobs of different pipeline ranks may run at the same time on streams of their own;
         # the worker sets `lane` to the rank whose stage is being lowered, and every shared
@@ -267,6 +268,26 @@ class BufferPool:
         self.bytes += t.numel() * t.element_size()
         return t
 
+    def stacked(self, key, shape, dtype, mb, count):
+        """Buffer `key` of micro-batch `mb`, one of `count` equal buffers laid end to end in one
+        allocation: what the micro-batches of a step write at the same place of the same stage
+        (an activation, the gradient of a layer's output) then forms ONE matrix with `count` times
+        the rows, which the weight-gradient product of the whole step reads in a single launch."""
+        shape = tuple(int(x) for x in shape)
+        if mb is None or not 0 <= mb < count:
+            return torch.empty(shape, dtype=dtype, device=self.device)
+        key = (key, shape, dtype, count)
+        slab = self._stacked.get(key)
+        if slab is None:
+            slab = self._stacked[key] = torch.empty((count,) + shape, dtype=dtype, device=self.device)
+            self.bytes += slab.numel() * slab.element_size()
+        return slab[mb]
+
+    def drop_stacked(self):
+        """Later requests get new allocations (a micro-batch slot is being rebuilt for other shapes);
+        buffers handed out so far live on with the programs that hold them."""
+        self._stacked = {}
+
 
 class StageProgram:
     def __init__(self, stage, mb):
@@ -287,6 +308,11 @@ class StageProgram:
         self.fwd_ranges = []
         self.bwd_ranges = []
         self.backward_nodes = []  # node name per entry of backward_fns
+        self.alloc_seq = 0        # forward buffers handed out so far (the same sequence for every micro-batch)
+        # weight-gradient products left to the stage's once-per-step job: (numel, dtype) of the layer
+        # output gradients they read, and per product (dy, x, accumulator, gemm arguments)
+        self.dw_sigs = set()
+        self.dw_deferred = []
 
     def run_forward(self, stream):
         if self.fwd_graph is not None:
@@ -325,9 +351,25 @@ class BwdCtx:
         # 16-bit copies of fp32 gradients that a producing kernel wrote on the side, and column
         # sums of such copies left as partial rows: {data_ptr: (storage_ptr, copy, colsum or None)}
         self._lp = {}
+        self._kept = {}     # (numel, dtype) -> buffers of that kind handed out so far in this job
 
     def emit(self, launch):
         self.out.append(launch)
+
+    def _kept_for_dw(self, shape, dtype):
+        """Gradients that a deferred weight-gradient product may read must outlive the job and lie
+        end to end across micro-batches: buffers of those sizes come from stacked allocations
+        (per stage and position in the job), not from the set every job of a lane shares."""
+        sigs = self.program.dw_sigs
+        if not sigs or self.L.stack_mbs <= 1:
+            return None
+        n = 1
+        for d in shape:
+            n *= int(d)
+        if (n, dtype) not in sigs:
+            return None
+        i = self._kept[(n, dtype)] = self._kept.get((n, dtype), 0) + 1
+        return self.L.pool.stacked(("g", self.program.stage, i, n), shape, dtype, self.program.mb, self.L.stack_mbs)
 
     # -- weight-gradient products that share a launch ---------------------------------------------
     FULL_GRID = 256     # workgroups that fill the device (one tile per CU)
@@ -465,6 +507,10 @@ class BwdCtx:
         self.reduces.append((ws, 0, self.k.colsum_partials(rows), cols, cols, acc))
 
     def new_like(self, like, private=False):
+        if like.is_contiguous():
+            kept = self._kept_for_dw(like.shape, like.dtype)
+            if kept is not None:
+                return kept
         if private:
             # gradients that outlive this job (they cross a stage boundary) get their own storage
             return self.L.pool.fresh_like(like)
@@ -472,6 +518,9 @@ class BwdCtx:
         return self.L.pool.bwd_like(self._seq, like)
 
     def temp(self, shape, dtype):
+        kept = self._kept_for_dw(shape, dtype)
+        if kept is not None:
+            return kept
         self._seq += 1
         return self.L.pool.bwd_like(self._seq, torch.empty(tuple(shape), dtype=dtype, device="meta"))
 
@@ -637,10 +686,18 @@ class Lowerer:
         self.params = params or ParamStore(kernels, self.device)
         self.pool = pool or BufferPool(self.device)
         self._ws = None
+        # > 1: weight-gradient products of linear layers are left out of the backward jobs and run once
+        # per step over all `stack_mbs` micro-batches (the worker builds that job); forward buffers and
+        # the gradients those products read are then laid end to end across micro-batches
+        self.stack_mbs = 1
 
     # -- buffers -------------------------------------------------------------
     def alloc(self, shape, dtype):
-        t = torch.empty(tuple(int(s) for s in shape), dtype=dtype, device=self.device)
+        if self.stack_mbs > 1:
+            self.cur.alloc_seq += 1
+            t = self.pool.stacked(("f", self.cur.stage, self.cur.alloc_seq), shape, dtype, self.cur.mb, self.stack_mbs)
+        else:
+            t = torch.empty(tuple(int(s) for s in shape), dtype=dtype, device=self.device)
         self.cur.fwd_bytes += t.numel() * t.element_size()
         return t
 
@@ -730,6 +787,51 @@ class Lowerer:
                                    "the unwritten region would hold garbage" % prog.stage)
         prog.backward_fns = []  # closures keep build-time state alive; not needed any more
         return prog
+
+    def lower_deferred_dw(self, progs):
+        """The once-per-step weight-gradient job of one stage.  `progs`: the stage's programs, one
+        per micro-batch, in micro-batch order.  Product i of every program reads that micro-batch's
+        layer-output gradient and layer input; where those lie end to end in memory (equal
+        micro-batches, stacked buffers) the micro-batches are ONE product over all their rows:
+        one launch and one read-modify-write of the fp32 accumulator instead of one per micro-batch
+        (ViT-L: a quarter of a weight-gradient launch was that pass).  Otherwise (ragged batch, an
+        operand in a buffer of its own) one product per micro-batch, in micro-batch order.
+        Returns the launch list."""
+        job = StageProgram(progs[0].stage, None)
+        B = BwdCtx(self, job)
+        for recs in zip(*[p.dw_deferred for p in progs]):
+            r0 = recs[0]
+            es = r0["dy"].element_size()
+            same = all(r["name"] == r0["name"] and r["wg"] is r0["wg"] and
+                       (r["rows"], r["n_out"], r["n_in"], r["ld_dy"], r["ld_x"]) ==
+                       (r0["rows"], r0["n_out"], r0["n_in"], r0["ld_dy"], r0["ld_x"]) and
+                       r["dy"].dtype == r0["dy"].dtype and r["x"].dtype == r0["x"].dtype for r in recs)
+            if not all(r["name"] == r0["name"] for r in recs):
+                raise RuntimeError("stage %d: the micro-batches' backward jobs list different weight-gradient "
+                                   "products" % job.stage)
+            stacked = same and len(recs) > 1 and r0["rows"] > 0 and all(
+                r["dy"].untyped_storage().data_ptr() == r0["dy"].untyped_storage().data_ptr() and
+                r["x"].untyped_storage().data_ptr() == r0["x"].untyped_storage().data_ptr() and
+                r["dy"].data_ptr() == r0["dy"].data_ptr() + j * r0["rows"] * r0["ld_dy"] * es and
+                r["x"].data_ptr() == r0["x"].data_ptr() + j * r0["rows"] * r0["ld_x"] * es
+                for j, r in enumerate(recs))
+            if stacked:
+                n = len(recs)
+                dy = torch.as_strided(r0["dy"], (n * r0["rows"], r0["n_out"]), (r0["ld_dy"], 1))
+                x = torch.as_strided(r0["x"], (n * r0["rows"], r0["n_in"]), (r0["ld_x"], 1))
+                B.emit_dw(self.kernels.gemm(dy, x, r0["wg"], M=r0["n_out"], N=r0["n_in"], K=n * r0["rows"],
+                                            lda=r0["ld_dy"], ldb=r0["ld_x"], ldc=r0["n_in"], a_trans=1, b_trans=1,
+                                            beta=1), r0["wg"])
+            else:
+                for r in recs:
+                    if r["rows"] == 0:
+                        continue
+                    B.emit_dw(self.kernels.gemm(r["dy"], r["x"], r["wg"], M=r["n_out"], N=r["n_in"], K=r["rows"],
+                                                lda=r["ld_dy"], ldb=r["ld_x"], ldc=r["n_in"], a_trans=1, b_trans=1,
+                                                beta=1), r["wg"])
+        B.close_dw()
+        B.compact([])
+        return job.bwd
 
     # -- helpers for handlers ----------------------------------------------------
     def arg(self, a):
@@ -869,6 +971,9 @@ def lower_linear(L, node):
     if res is not None:
         kw.update(residual=res.buf, ld_res=as_matrix(res.buf)[2])
     L.emit(L.kernels.gemm(xm, w_cd, out, **kw))
+    defer_dw = L.stack_mbs > 1 and w.req_grad and w.param is not None
+    if defer_dw:
+        L.cur.dw_sigs.add((M * N, cd))
     req = x.req_grad or w.req_grad or (b is not None and b.req_grad) or (res is not None and res.req_grad)
     outv = Val(out, req_grad=req, name=out_node.name)
     if L.mixed and out_dtype == torch.float32 and act == ACT_NONE:
@@ -900,7 +1005,13 @@ def lower_linear(L, node):
             # dW = dY^T X reduces over the token rows, the strided dimension of both operands: the
             # GEMM reads them with transposing LDS reads (no transposed copies in memory)
             wg = L.params.grad(w.param)
-            B.emit_dw(B.k.gemm(dy, xm, wg, M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1, b_trans=1, beta=1), wg)
+            if defer_dw:
+                # left to the stage's once-per-step job: over all micro-batches the operands form one
+                # product with that many times the reduction length, and one pass over the accumulator
+                B.program.dw_deferred.append(dict(name=node.name, dy=dy, x=xm, wg=wg, rows=M, n_out=N, n_in=K,
+                                                  ld_dy=ld_dy, ld_x=lda))
+            else:
+                B.emit_dw(B.k.gemm(dy, xm, wg, M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1, b_trans=1, beta=1), wg)
         if b is not None and b.req_grad and b.param is not None:
             B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
         if x.req_grad:

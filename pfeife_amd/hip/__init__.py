@@ -363,6 +363,7 @@ class HipKernels:
         launch = self._prep("pf_gemm_grouped", (arr, n), (arr, launches))
         launch.variant = launches[0].variant.replace("gemm16x_kernel<", "gemm16x_group_kernel<")
         launch.flops = sum(l.flops for l in launches)
+        launch.members = list(launches)
         return launch
 
     # -- fused attention -----------------------------------------------------------

@@ -50,7 +50,8 @@ class StageWorker:
         self.log = get_logger()
         self.params = ParamStore(kernels, self.device)
         self.pool = BufferPool(self.device)
-        self.lowerer = Lowerer(kernels, self.device, option.mixed_precision, self.params, self.pool)
+        self.lowerer = self._new_lowerer()
+        self.dw_jobs = {}          # stage -> [launch list, captured graph or None]: the once-per-step weight-gradient job
         self.part_graph = None
         self.static_inputs = {}
         self.mbs = {}
@@ -84,6 +85,14 @@ class StageWorker:
             self.scaler_state = torch.tensor([option.init_scale] + [0.0] * 7, dtype=torch.float32,
                                              device=self.device)
             self._one = torch.ones((), dtype=torch.float32, device=self.device)
+
+    def _new_lowerer(self):
+        L = Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
+        # Weight gradients of the linear layers once per step instead of once per micro-batch
+        # (PFEIFE_DW_STACK=0: inside every backward job, as torch.autograd issues them)
+        if self.option.batch_cnt > 1 and os.environ.get("PFEIFE_DW_STACK", "1") != "0":
+            L.stack_mbs = self.option.batch_cnt
+        return L
 
     # -- graph ---------------------------------------------------------------------
     def set_partition_graph(self, part_graph, example_inputs):
@@ -131,6 +140,11 @@ class StageWorker:
             if is_fwd:
                 last[mb] = i
         self.last_forward = {i: mb for mb, i in last.items()}
+        # the job after which a stage's once-per-step weight-gradient job runs: its last backward
+        self.last_backward = {}
+        for stage, mb, is_fwd in self.order:
+            if not is_fwd:
+                self.last_backward[stage] = mb
 
     def _lane_key(self, stage, is_fwd):
         rank = self.part_graph.nodes[stage].rank
@@ -260,7 +274,11 @@ class StageWorker:
                 v = stage_out[ref[0]][ref[1]]
                 slot.outputs.append(v)
                 if isinstance(v, Val) and v.req_grad:
-                    slot.loss_grads[oi] = torch.zeros_like(v.buf)
+                    if L.stack_mbs > 1 and v.buf.is_contiguous():
+                        # (the last layer's weight gradient reads these across micro-batches as one matrix)
+                        slot.loss_grads[oi] = self.pool.stacked(("loss", oi), v.buf.shape, v.buf.dtype, mb, L.stack_mbs).zero_()
+                    else:
+                        slot.loss_grads[oi] = torch.zeros_like(v.buf)
         # backward, last stage first: a stage's output gradients are its consumers' input gradients
         for sid in sorted(pg.nodes, reverse=True):
             st = pg.nodes[sid]
@@ -280,7 +298,10 @@ class StageWorker:
             self.pool.lane = self._lane_key(sid, False) if self.lanes is not None else 0
             L.lower_backward(prog, out_grads)
         self.pool.lane = 0
-        self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
+        if mb in self.mbs:                    # a slot rebuilt for another micro-batch shape
+            self.pool.drop_stacked()
+        self._drop_graphs(self.mbs.get(mb))
+        self._drop_dw_jobs()
         self.mbs[mb] = slot
         self.graphs_ready = False   # new programs (and possibly new parameters): capture again
         self._drop_begin_graph()
@@ -297,6 +318,12 @@ class StageWorker:
                     self.kernels.destroy_graph(g)
                     setattr(prog, attr, None)
 
+    def _drop_dw_jobs(self):
+        for job in self.dw_jobs.values():
+            if job[1] is not None and hasattr(self.kernels, "destroy_graph"):
+                self.kernels.destroy_graph(job[1])
+        self.dw_jobs = {}
+
     def _drop_begin_graph(self):
         if self.begin_graph is not None and hasattr(self.kernels, "destroy_graph"):
             self.kernels.destroy_graph(self.begin_graph)
@@ -310,6 +337,7 @@ class StageWorker:
         for slot in self.mbs.values():
             self._drop_graphs(slot)
         self._drop_begin_graph()
+        self._drop_dw_jobs()
         self.mbs = {}
         self.graphs_ready = False
         self.static_inputs = {}
@@ -323,7 +351,7 @@ class StageWorker:
         self._host_steps_stale = False
         self.params = ParamStore(self.kernels, self.device)
         self.pool = BufferPool(self.device)
-        self.lowerer = Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
+        self.lowerer = self._new_lowerer()
         self.__dict__.pop("_adam_tables", None)
 
     # -- per step --------------------------------------------------------------------
@@ -341,6 +369,9 @@ class StageWorker:
                     prog.fwd_graph = self.kernels.capture(prog.fwd, s)
                 if prog.bwd_graph is None and prog.bwd:
                     prog.bwd_graph = self.kernels.capture(prog.bwd, s)
+        for job in self.dw_jobs.values():
+            if job[1] is None and job[0]:
+                job[1] = self.kernels.capture(job[0], s)
         pre = self.params.zero_launches() + self.params.refresh_launches()
         self._drop_begin_graph()
         self.begin_graph = self.kernels.capture(pre, s) if pre else None
@@ -454,6 +485,20 @@ class StageWorker:
                     continue
                 self.kernels.fill(buf, self.option.loss_scale if buf.dim() == 0 else 0.0, buf.numel())(self.stream())
 
+    def _run_dw_job(self, stage, stream):
+        """The stage's weight-gradient products over all micro-batches of the step, after its last
+        backward job and on that job's stream (built when every micro-batch slot exists)."""
+        job = self.dw_jobs.get(stage)
+        if job is None:
+            progs = [self.mbs[m].stage_programs[stage] for m in sorted(self.mbs)]
+            launches = self.lowerer.lower_deferred_dw(progs) if any(p.dw_deferred for p in progs) else []
+            job = self.dw_jobs[stage] = [launches, None]
+        if job[1] is not None:
+            job[1](stream)
+        else:
+            for launch in job[0]:
+                launch(stream)
+
     def run_job(self, stage, mb, is_fwd):
         prog = self.mbs[mb].stage_programs[stage]
         if self.lanes is None:
@@ -461,6 +506,8 @@ class StageWorker:
                 prog.run_forward(self.stream())
             else:
                 prog.run_backward(self.stream())
+                if self.last_backward.get(stage) == mb and self.lowerer.stack_mbs > 1:
+                    self._run_dw_job(stage, self.stream())
             return
         # the job goes to its rank's stream, after the jobs of other ranks whose results it reads:
         # forward after the producers of its inputs, backward after the consumers of its outputs
@@ -488,7 +535,9 @@ class StageWorker:
             prog.run_forward(lane.cuda_stream)
         else:
             prog.run_backward(lane.cuda_stream)
-        self._event(self._job_events, (stage, mb, is_fwd)).record(lane)
+        self._event(self._job_events, (stage, mb, is_fwd)).record(lane)   # (the weight-gradient job feeds no other job)
+        if not is_fwd and self.last_backward.get(stage) == mb and self.lowerer.stack_mbs > 1:
+            self._run_dw_job(stage, lane.cuda_stream)
 
     def init_optimizer(self, optimizer):
         if optimizer is not None:

@@ -424,3 +424,37 @@ def test_weights_tied_across_two_stages_accumulate_both_contributions():
         assert abs(float(got) - float(want.detach())) <= 1e-5 * abs(float(want.detach()))
     for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
         assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+
+
+def test_weight_gradients_run_once_per_step_over_all_micro_batches(monkeypatch):
+    """Equal micro-batches: every linear layer's weight gradient is ONE product whose reduction runs
+    over the rows of all micro-batches (their activations and output gradients lie end to end in
+    stacked buffers), issued after the stage's last backward job.  A ragged batch keeps one product
+    per micro-batch in that job; PFEIFE_DW_STACK=0 keeps them inside the backward jobs.  All three
+    give the gradients of plain accumulation (checked by the callers' own comparisons above)."""
+    model, ref, out, (x, y), runner, crit = run_case(None)            # 8 samples in 4 micro-batches, 2 stages
+    w = runner.worker
+    assert sorted(w.dw_jobs) == [0, 1] and w.last_backward == {0: 3, 1: 3}
+    tokens = (CFG.image_size // CFG.patch_size) ** 2 + 1
+    per_stage = {sid: len(w.mbs[0].stage_programs[sid].dw_deferred) for sid in (0, 1)}
+    assert per_stage[0] >= 8 and per_stage[1] >= 8                    # four linear layers per block, two blocks each
+    for sid, (launches, _) in w.dw_jobs.items():
+        assert len(launches) == per_stage[sid]                        # one launch per layer, not per micro-batch
+    # the block layers reduce over 4 micro-batches x 2 samples x tokens rows
+    ks = sorted({int(r["rows"]) for r in w.mbs[0].stage_programs[0].dw_deferred})
+    assert 2 * tokens in ks
+    run_pipeline_step(split_stages(ref, 2), crit, x, y, 4, device_cnt=2)
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+    # ragged: 7 samples over 3 micro-batches: one product per micro-batch and layer
+    model, ref, out, (x, y), runner, crit = run_case(None, batch=7, batch_cnt=3, device_cnt=1, split=None)
+    w = runner.worker
+    n_layers = len(w.mbs[0].stage_programs[0].dw_deferred)
+    assert len(w.dw_jobs[0][0]) == 3 * n_layers
+    # switched off: nothing is deferred
+    monkeypatch.setenv("PFEIFE_DW_STACK", "0")
+    model, ref, out, (x, y), runner, crit = run_case(None)
+    assert runner.worker.dw_jobs == {} and not runner.worker.mbs[0].stage_programs[0].dw_deferred
+    run_unpipelined(ref, crit, x, y, 4)
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n

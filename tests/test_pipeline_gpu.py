@@ -174,6 +174,14 @@ def test_vit_l_width_fp16_headline_geometry():
             "gemm16x_kernel<1, 128, 128, 64, 2, 4, 1, 3, true, true, 4>"]      # weight gradients, accumulated
     for w in want:
         assert w in names, (w, sorted(names))
+    # the blocks' weight gradients: once per step, one product per layer over the 4 x 3152 token rows of
+    # all micro-batches, several layers sharing a launch on 256x256 tiles
+    for sid, (launches, graph) in runner.worker.dw_jobs.items():
+        members = [m for l in launches for m in getattr(l, "members", [l])]
+        assert len(members) == 2 * 4 + (sid == 1), (sid, len(members))         # 2 blocks x 4 layers (+ the head)
+        assert sum(m.desc.K == 4 * 3152 for m in members) == 2 * 4
+        assert any(l.variant == "gemm16x_group_kernel<1, 256, 256, 32, 2, 4, 1, 5, true, true, 4>" for l in launches), \
+            [l.variant for l in launches]
 
 
 def test_vit_l16_headline_config_trains_like_pytorch():
