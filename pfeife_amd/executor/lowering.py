@@ -283,10 +283,10 @@ class BufferPool:
             self.bytes += slab.numel() * slab.element_size()
         return slab[mb]
 
-    def drop_stacked(self):
-        """Later requests get new allocations (a micro-batch slot is being rebuilt for other shapes);
-        buffers handed out so far live on with the programs that hold them."""
-        self._stacked = {}
+    def prune_stacked(self, live_tags):
+        """Forget the stacked allocations made under tags no micro-batch slot uses any more (their
+        memory goes when the programs that hold slices of them do)."""
+        self._stacked = {k: v for k, v in self._stacked.items() if k[0][0] in live_tags}
 
 
 class StageProgram:
@@ -369,7 +369,8 @@ class BwdCtx:
         if (n, dtype) not in sigs:
             return None
         i = self._kept[(n, dtype)] = self._kept.get((n, dtype), 0) + 1
-        return self.L.pool.stacked(("g", self.program.stage, i, n), shape, dtype, self.program.mb, self.L.stack_mbs)
+        return self.L.pool.stacked((self.L.stack_tag, "g", self.program.stage, i, n), shape, dtype, self.program.mb,
+                                   self.L.stack_mbs)
 
     # -- weight-gradient products that share a launch ---------------------------------------------
     FULL_GRID = 256     # workgroups that fill the device (one tile per CU)
@@ -690,12 +691,14 @@ class Lowerer:
         # per step over all `stack_mbs` micro-batches (the worker builds that job); forward buffers and
         # the gradients those products read are then laid end to end across micro-batches
         self.stack_mbs = 1
+        self.stack_tag = None   # micro-batch slots lowered under the same tag (input shapes) share stacked allocations
 
     # -- buffers -------------------------------------------------------------
     def alloc(self, shape, dtype):
         if self.stack_mbs > 1:
             self.cur.alloc_seq += 1
-            t = self.pool.stacked(("f", self.cur.stage, self.cur.alloc_seq), shape, dtype, self.cur.mb, self.stack_mbs)
+            t = self.pool.stacked((self.stack_tag, "f", self.cur.stage, self.cur.alloc_seq), shape, dtype, self.cur.mb,
+                                  self.stack_mbs)
         else:
             t = torch.empty(tuple(int(s) for s in shape), dtype=dtype, device=self.device)
         self.cur.fwd_bytes += t.numel() * t.element_size()
@@ -799,16 +802,20 @@ class Lowerer:
         Returns the launch list."""
         job = StageProgram(progs[0].stage, None)
         B = BwdCtx(self, job)
-        for recs in zip(*[p.dw_deferred for p in progs]):
+        lists = [p.dw_deferred for p in progs]
+        if len({tuple(r["name"] for r in recs) for recs in lists}) == 1:
+            groups = list(zip(*lists))              # product i of every micro-batch
+        else:
+            # programs lowered at different times (a slot rebuilt for another shape without the
+            # deferral): every program's products on their own
+            groups = [(r,) for recs in lists for r in recs]
+        for recs in groups:
             r0 = recs[0]
             es = r0["dy"].element_size()
             same = all(r["name"] == r0["name"] and r["wg"] is r0["wg"] and
                        (r["rows"], r["n_out"], r["n_in"], r["ld_dy"], r["ld_x"]) ==
                        (r0["rows"], r0["n_out"], r0["n_in"], r0["ld_dy"], r0["ld_x"]) and
                        r["dy"].dtype == r0["dy"].dtype and r["x"].dtype == r0["x"].dtype for r in recs)
-            if not all(r["name"] == r0["name"] for r in recs):
-                raise RuntimeError("stage %d: the micro-batches' backward jobs list different weight-gradient "
-                                   "products" % job.stage)
             stacked = same and len(recs) > 1 and r0["rows"] > 0 and all(
                 r["dy"].untyped_storage().data_ptr() == r0["dy"].untyped_storage().data_ptr() and
                 r["x"].untyped_storage().data_ptr() == r0["x"].untyped_storage().data_ptr() and

@@ -40,6 +40,18 @@ from ..worker import StageWorker
 STEP_TOKEN = "###<<STEP_TOKEN>>###"
 
 
+def _same_shapes(args, kwargs):
+    """Do the micro-batches of a step agree in the shapes and dtypes of all their tensors?  (A batch
+    that does not divide evenly gives the first micro-batches one row more, pfeife/batch.py:45.)"""
+    from torch.utils._pytree import tree_flatten
+
+    sigs = set()
+    for a, k in zip(args, kwargs):
+        leaves, _ = tree_flatten((a, k))
+        sigs.add(tuple((tuple(t.shape), t.dtype) for t in leaves if torch.is_tensor(t)))
+    return len(sigs) <= 1
+
+
 class _ExecError:
     def __init__(self, exc):
         self.exc = exc
@@ -98,6 +110,7 @@ class PartialRunner:
             raise RuntimeError("call set_exec_fn() before step()")
         option = self.option
         args, kwargs = split_args_kwargs(args, kwargs, option.batch_cnt)
+        self.worker.uniform_mbs = _same_shapes(args, kwargs)
 
         if not self._compiled:
             self._probe_forward(args[0], kwargs[0])

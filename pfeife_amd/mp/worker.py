@@ -87,12 +87,13 @@ class StageWorker:
             self._one = torch.ones((), dtype=torch.float32, device=self.device)
 
     def _new_lowerer(self):
-        L = Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
         # Weight gradients of the linear layers once per step instead of once per micro-batch
-        # (PFEIFE_DW_STACK=0: inside every backward job, as torch.autograd issues them)
-        if self.option.batch_cnt > 1 and os.environ.get("PFEIFE_DW_STACK", "1") != "0":
-            L.stack_mbs = self.option.batch_cnt
-        return L
+        # (PFEIFE_DW_STACK=0: inside every backward job, as torch.autograd issues them); decided per
+        # micro-batch slot when it is lowered: only steps whose micro-batches all have the same
+        # shapes stack their buffers (`uniform_mbs`, set by the runner before the step's first job)
+        self.stack_dw = self.option.batch_cnt > 1 and os.environ.get("PFEIFE_DW_STACK", "1") != "0"
+        self.uniform_mbs = getattr(self, "uniform_mbs", True)
+        return Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
 
     # -- graph ---------------------------------------------------------------------
     def set_partition_graph(self, part_graph, example_inputs):
@@ -237,6 +238,8 @@ class StageWorker:
         for i, v in pg.static_vals.items():
             graph_vals[i] = v
         L = self.lowerer
+        L.stack_mbs = self.option.batch_cnt if (self.stack_dw and self.uniform_mbs) else 1
+        L.stack_tag = slot.input_sig
         stage_out = {}
         for sid in sorted(pg.nodes):
             st = pg.nodes[sid]
@@ -276,7 +279,8 @@ class StageWorker:
                 if isinstance(v, Val) and v.req_grad:
                     if L.stack_mbs > 1 and v.buf.is_contiguous():
                         # (the last layer's weight gradient reads these across micro-batches as one matrix)
-                        slot.loss_grads[oi] = self.pool.stacked(("loss", oi), v.buf.shape, v.buf.dtype, mb, L.stack_mbs).zero_()
+                        slot.loss_grads[oi] = self.pool.stacked((L.stack_tag, "loss", oi), v.buf.shape, v.buf.dtype, mb,
+                                                                L.stack_mbs).zero_()
                     else:
                         slot.loss_grads[oi] = torch.zeros_like(v.buf)
         # backward, last stage first: a stage's output gradients are its consumers' input gradients
@@ -298,11 +302,10 @@ class StageWorker:
             self.pool.lane = self._lane_key(sid, False) if self.lanes is not None else 0
             L.lower_backward(prog, out_grads)
         self.pool.lane = 0
-        if mb in self.mbs:                    # a slot rebuilt for another micro-batch shape
-            self.pool.drop_stacked()
-        self._drop_graphs(self.mbs.get(mb))
+        self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
         self._drop_dw_jobs()
         self.mbs[mb] = slot
+        self.pool.prune_stacked({s.input_sig for s in self.mbs.values()})
         self.graphs_ready = False   # new programs (and possibly new parameters): capture again
         self._drop_begin_graph()
         return slot
@@ -506,7 +509,7 @@ class StageWorker:
                 prog.run_forward(self.stream())
             else:
                 prog.run_backward(self.stream())
-                if self.last_backward.get(stage) == mb and self.lowerer.stack_mbs > 1:
+                if self.last_backward.get(stage) == mb and self.stack_dw:
                     self._run_dw_job(stage, self.stream())
             return
         # the job goes to its rank's stream, after the jobs of other ranks whose results it reads:
@@ -536,7 +539,7 @@ class StageWorker:
         else:
             prog.run_backward(lane.cuda_stream)
         self._event(self._job_events, (stage, mb, is_fwd)).record(lane)   # (the weight-gradient job feeds no other job)
-        if not is_fwd and self.last_backward.get(stage) == mb and self.lowerer.stack_mbs > 1:
+        if not is_fwd and self.last_backward.get(stage) == mb and self.stack_dw:
             self._run_dw_job(stage, lane.cuda_stream)
 
     def init_optimizer(self, optimizer):
