@@ -1359,3 +1359,61 @@ def test_split_then_merge_round_trip_on_device():
         args, _ = split_args_kwargs((x,), {}, n)
         merged = merge_chunks([a[0] for a in args])
         assert torch.equal(merged, x)
+
+
+def test_weight_gradients_once_per_step_equal_the_per_micro_batch_sums(monkeypatch):
+    """Linear layers' weight gradients run once per step over the rows of all micro-batches
+    (stacked activations and output gradients, one product per layer after the stage's last
+    backward job) instead of once per micro-batch.  Both ways sum the same products in fp32 in
+    another order: over three Adam steps (eager build step, then hipGraph replays) on a two-stage
+    ViT, fp32 and bf16, losses and every gradient must agree to rounding, and the deferred job must
+    really hold one product per layer with four times the rows."""
+    from pfeife_amd.bench_models.vit import ViTConfig, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    def run(stack, mixed):
+        monkeypatch.setenv("PFEIFE_DW_STACK", stack)
+        cfg = ViTConfig(image_size=64, patch_size=16, dim=128, depth=4, heads=4, mlp_dim=256, num_classes=16)
+        torch.manual_seed(0)
+        model = VisionTransformer(cfg)
+        g = torch.Generator().manual_seed(42)
+        x = torch.randn(12, 3, 64, 64, generator=g).cuda()
+        y = torch.randint(0, 16, (12,), generator=g).cuda()
+        option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=3, split_points=["blocks.2"],
+                            mixed_precision=mixed, optimizer=dict(type="adam", lr=1e-3))
+        runner = _fresh_runner(option)
+        model.cuda()
+        cmodel = torch.compile(model, backend=partial_compiler)
+        crit = nn.CrossEntropyLoss()
+
+        def fn(px, labels):
+            loss = crit(cmodel(px).float(), labels)
+            loss.backward()
+            return loss.detach()
+
+        runner.set_exec_fn(fn)
+        hist = []
+        for _ in range(3):
+            losses = runner.step(x, y)
+            torch.cuda.synchronize()
+            hist.append(([float(l) for l in losses], {n: p.grad.detach().clone() for n, p in model.named_parameters()}))
+        return hist, runner
+
+    for mixed, tol in ((None, 2e-5), ("bf16", 2e-2)):
+        per_mb, r0 = run("0", mixed)
+        assert r0.worker.dw_jobs == {} or all(not launches for launches, _ in r0.worker.dw_jobs.values())
+        once, r1 = run("1", mixed)
+        w = r1.worker
+        assert sorted(w.dw_jobs) == [0, 1] and all(graph is not None for _, graph in w.dw_jobs.values())
+        rows = 3 * (1 + (64 // 16) ** 2)                               # micro-batch 3 x 17 tokens
+        for sid, (launches, _) in w.dw_jobs.items():
+            members = [m for l in launches for m in getattr(l, "members", [l])]
+            assert len(members) == len(w.mbs[0].stage_programs[sid].dw_deferred)    # one product per layer
+            assert sum(m.desc.K == 4 * rows for m in members) >= 8                  # 2 blocks x 4 layers over all rows
+        for (la, ga), (lb, gb) in zip(per_mb, once):
+            for a, b in zip(la, lb):
+                assert abs(a - b) <= tol * abs(a), (mixed, a, b)
+            for n in ga:
+                d = (ga[n].double() - gb[n].double()).norm() / (ga[n].double().norm() + 1e-12)
+                assert d <= tol, (mixed, n, float(d))
