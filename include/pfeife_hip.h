@@ -140,12 +140,19 @@ typedef struct pf_gemm_desc {
                        tile dimension): the bias gradient of the layer whose pre-activation gradient C is
                        (aten.sum of the reference's autograd, pfeife/mp/worker.py:1585-1587), finished by
                        pf_colreduce_finalize(_batch).  PF_ERR_UNSUPPORTED on any other kernel path. */
+  const float* unscale_by; /* optional: device pointer to a loss scale s > 0, read when the kernel runs: the
+                       product is multiplied by alpha / s[0] instead of alpha, so a gradient computed from a scaled
+                       loss leaves the product unscaled (GradScaler.unscale_ of pfeife/mp/worker.py:1432-1436 without
+                       a pass of its own) */
+  float* nonfinite_flag; /* optional: set to 1.0f when a value written to C is not finite (the overflow check of
+                       the same unscale_); only on the fp32-store / fp32-accumulate classes of the direct-to-LDS
+                       kernel (pf_gemm_variant ends in ", 1>" or ", 4>"), PF_ERR_UNSUPPORTED elsewhere */
 } pf_gemm_desc;
 
 int pf_gemm(const pf_gemm_desc* desc, void* stream);
 #define PF_GEMM_GROUP_MAX 8
 /* n products in as few launches as possible.  Runs of consecutive descriptors that are weight
- * gradients (a_trans = b_trans = 1, 16-bit operands, fp32 C with beta = 1, no epilogue operands,
+ * gradients (a_trans = b_trans = 1, 16-bit operands, fp32 C stored or accumulated, no epilogue operands,
  * no batch) and resolve to the same kernel instantiation share ONE launch (up to PF_GEMM_GROUP_MAX
  * per launch):
  * dW of a 1024x1024 weight covers only 64 of the 256 CUs on its own.  Everything else is issued

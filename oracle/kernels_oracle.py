@@ -99,7 +99,7 @@ class OracleKernels:
 
     def gemm(self, a, b, c, M, N, K, lda, ldb, ldc, a_trans=0, b_trans=0, batch=(1, 1), sa=(0, 0), sb=(0, 0),
              sc=(0, 0), alpha=1.0, beta=0, bias=None, round_mid=0, aux_out=None, ld_aux_out=0, act=0, dact=0,
-             aux_in=None, ld_aux_in=0, residual=None, ld_res=0):
+             aux_in=None, ld_aux_in=0, residual=None, ld_res=0, unscale_by=None, nonfinite_flag=None):
         b1, b2 = batch
         in_dtype = a.dtype
 
@@ -108,7 +108,9 @@ class OracleKernels:
             # op(B) is K x N
             Bm = _strided(b, (b1, b2, K, N), (sb[0], sb[1], ldb, 1) if b_trans else (sb[0], sb[1], 1, ldb))
             C = _strided(c, (b1, b2, M, N), (sc[0], sc[1], ldc, 1))
-            v = alpha * torch.matmul(A.float(), Bm.float())
+            # unscale_by: a loss scale read when the product runs (GradScaler.unscale_ folded in)
+            a_eff = alpha if unscale_by is None else alpha / float(unscale_by.reshape(-1)[0])
+            v = a_eff * torch.matmul(A.float(), Bm.float())
             if bias is not None:
                 v = v + _flat(bias, N).float()
             if round_mid:
@@ -124,8 +126,14 @@ class OracleKernels:
             if beta:
                 v = v + C.float()
             C.copy_(v.to(c.dtype))
+            if nonfinite_flag is not None and not bool(torch.isfinite(v).all()):
+                nonfinite_flag.fill_(1.0)     # the overflow check of the same unscale_
 
         return launch
+
+    @staticmethod
+    def gemm_stores_checked(launch):
+        return True       # every product of the oracle honours unscale_by / nonfinite_flag
 
     # -- fused attention -----------------------------------------------------------
     MAX_FUSED_HEAD_DIM = 96

@@ -716,9 +716,17 @@ int dispatch16(const pf_gemm_desc& d, hipStream_t st) {
       return PF_ERR_UNSUPPORTED;
     }
   }
+  if (d.nonfinite_flag != nullptr) {   // only the fp32 classes of the direct-to-LDS kernel check what they write
+    const int ec = epi_class(d, epi_vec_ok(d));
+    if (!is_x_variant(v) || !x_supports(d, v) || (ec != EC_STORE32 && ec != EC_ACC32) ||
+        (d.a_trans != d.b_trans)) {
+      pf_set_error("pf_gemm: nonfinite_flag needs a 16-bit product with fp32 C (stored or accumulated) on the direct-to-LDS kernel");
+      return PF_ERR_UNSUPPORTED;
+    }
+  }
   switch (v) {
     case V_X256: case V_X256x128: case V_X128: case V_X192x256: case V_X128K2: case V_X256x128K2: case V_X256W8: case V_X128W8: case V_X256x128W8: {
-      const int xt = v;   // variant ids 1..7 are the PF_XT_* tile ids
+      const int xt = v;   // variant ids 1..9 are the PF_XT_* tile ids
       if (!x_supports(d, xt)) {
         pf_set_error("pf_gemm: variant %d needs both operands stored alike and (unless transposed) K a multiple of the stage depth", v);
         return PF_ERR_INVALID;
@@ -765,6 +773,10 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
   if (d.in_dtype == PF_F32) {
     if (d.colsum_ws != nullptr) {
       pf_set_error("pf_gemm: colsum_ws needs a 16-bit product with the GELU' epilogue on the direct-to-LDS kernel");
+      return PF_ERR_UNSUPPORTED;
+    }
+    if (d.nonfinite_flag != nullptr || d.unscale_by != nullptr) {
+      pf_set_error("pf_gemm: unscale_by / nonfinite_flag need a 16-bit product");
       return PF_ERR_UNSUPPORTED;
     }
     GemmGrid g;
@@ -832,7 +844,7 @@ extern "C" int pf_gemm(const pf_gemm_desc* desc, void* stream) {
 namespace {
 bool groupable(const pf_gemm_desc& d, int& variant) {
   if (d.in_dtype != PF_F16 && d.in_dtype != PF_BF16) return false;
-  if (!(d.a_trans && d.b_trans) || d.c_dtype != PF_F32 || d.beta != 1 || d.alpha != 1.f) return false;
+  if (!(d.a_trans && d.b_trans) || d.c_dtype != PF_F32 || (d.beta != 0 && d.beta != 1)) return false;
   if (d.batch1 > 1 || d.batch2 > 1 || d.bias || d.residual || d.aux_in || d.aux_out || d.act || d.dact) return false;
   if (d.M <= 0 || d.N <= 0 || d.K <= 0 || !d.A || !d.B || !d.C) return false;
   if (!pf_aligned(d.A, 16) || !pf_aligned(d.B, 16) || d.lda % 8 || d.ldb % 8 || d.lda < d.M || d.ldb < d.N ||
@@ -843,7 +855,9 @@ bool groupable(const pf_gemm_desc& d, int& variant) {
   variant = resolve_variant(d);
   if (!is_x_variant(variant) || variant == V_X192x256) return false;
   if (!x_supports(d, variant)) return false;
-  return epi_class(d, epi_vec_ok(d)) == EC_ACC32;
+  // (a product that stores rides in the accumulate launch: its old C reads as zeros)
+  const int ec = epi_class(d, epi_vec_ok(d));
+  return ec == EC_ACC32 || ec == EC_STORE32;
 }
 }  // namespace
 

@@ -26,15 +26,19 @@ struct Epi {
   void* C;
   int64_t ldc, ld_aux_out, ld_aux_in, ld_res;
   float* colsum_ws;
+  float* nonfinite;
 };
 
 __device__ __forceinline__ Epi make_epi(const pf_gemm_desc& p) {
   Epi e;
-  e.alpha = p.alpha; e.beta = p.beta; e.round_mid = p.round_mid; e.act = p.act; e.dact = p.dact;
+  // (a loss scale kept on the device divides the product: read here, once per workgroup)
+  e.alpha = p.unscale_by != nullptr ? p.alpha / p.unscale_by[0] : p.alpha;
+  e.beta = p.beta; e.round_mid = p.round_mid; e.act = p.act; e.dact = p.dact;
   e.in_dtype = p.in_dtype; e.c_dtype = p.c_dtype; e.bias_dtype = p.bias_dtype; e.res_dtype = p.res_dtype;
   e.bias = p.bias; e.aux_out = p.aux_out; e.aux_in = p.aux_in; e.residual = p.residual; e.C = p.C;
   e.ldc = p.ldc; e.ld_aux_out = p.ld_aux_out; e.ld_aux_in = p.ld_aux_in; e.ld_res = p.ld_res;
   e.colsum_ws = p.colsum_ws;
+  e.nonfinite = p.nonfinite_flag;
   return e;
 }
 

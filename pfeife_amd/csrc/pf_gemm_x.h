@@ -428,7 +428,10 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
                                                             : (EC == EC_DACT16 ? epi.aux_in : (const void*)((const char*)epi.C + c_base * ESC));
     const int64_t ld_l = (EC == EC_RES32 || EC == EC_RES16) ? epi.ld_res : (EC == EC_DACT16 ? epi.ld_aux_in : epi.ldc);
     constexpr int ESL = LOAD32 ? 4 : 2;
-    const __amdgpu_buffer_rsrc_t rs_l = make_rsrc(LOADS ? lp : epi.C, LOADS ? (uint32_t)(((M - 1) * ld_l + N) * ESL) : 0u);
+    // (a product that stores, beta = 0, inside a launch of the accumulate class, i.e. one member of a
+    // grouped weight-gradient launch, reads its old C through a descriptor of extent 0: all zeros)
+    const bool loads_on = LOADS && !(EC == EC_ACC32 && epi.beta == 0);
+    const __amdgpu_buffer_rsrc_t rs_l = make_rsrc(LOADS ? lp : epi.C, loads_on ? (uint32_t)(((M - 1) * ld_l + N) * ESL) : 0u);
     const uint32_t off_l = col_ok ? (uint32_t)((row0 * ld_l + c8) * ESL) : OOB;
     const uint32_t step_l = (uint32_t)(ld_l * ESL);
     const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(EC == EC_ACT16 ? epi.aux_out : epi.C,
@@ -452,6 +455,7 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
       }
     };
     float8_t csum = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // EC_DACT16: column sums of the stored values
+    float worst = 0.f;   // fp32 classes: sum of v - v over the values written: 0 if all are finite, NaN otherwise
     fetch(0);
 #pragma nounroll
     for (int hb = 0; hb < NHB; ++hb) {
@@ -532,6 +536,10 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
         }
         const uint32_t oc = off_c + rowk * step_c;
         if constexpr (C32) {
+          if constexpr (EC == EC_STORE32 || EC == EC_ACC32) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) worst += (row0 + (int64_t)rowk < M) ? (v[k] - v[k]) : 0.f;
+          }
           v4i_t lo, hi;
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
@@ -549,6 +557,10 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
           __builtin_amdgcn_raw_buffer_store_b128(packed, rs_c, (int)oc, 0, 0);
         }
       }
+    }
+    if constexpr (EC == EC_STORE32 || EC == EC_ACC32) {
+      // every writer writes the same value: no atomic needed
+      if (epi.nonfinite != nullptr && worst != 0.f) *epi.nonfinite = 1.f;
     }
     if constexpr (EC == EC_DACT16) {
       if (epi.colsum_ws != nullptr) {   // uniform over the grid

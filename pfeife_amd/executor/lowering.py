@@ -58,6 +58,14 @@ class ParamStore:
         self._arena = None     # current block of the gradient arena
         self._arena_used = 0
         self.arena_block = 64 * 1024 * 1024   # fp32 elements per arena block (256 MiB)
+        # Gradients that ONE once-per-step weight-gradient product writes whole (stored, already
+        # unscaled and checked for overflow by that product's epilogue) need no zero fill and no
+        # unscale pass: they live in blocks of their own, outside the arena those passes sweep.
+        self._lazy = {}            # id(param) -> True while that holds, False once another writer appeared
+        self._lazy_block = None
+        self._lazy_used = 0
+        self.deferred_sites = {}   # id(param) -> {(stage, node name)} of the deferred products that write it
+        self.demoted = []          # gradients in such blocks that need the fill and the unscale after all
 
     def shadow(self, tensor, dtype):
         if tensor.dtype == dtype:
@@ -154,7 +162,7 @@ class ParamStore:
         for p in self.params:
             g = self._grads[id(p)]
             base = g._base if g._base is not None else g
-            if base.data_ptr() not in done:
+            if base.data_ptr() not in done and not self._lazy.get(id(p)):
                 out.append((g, g.numel()))
         return out
 
@@ -172,7 +180,7 @@ class ParamStore:
         for p in self.params:
             g = self._grads[id(p)]
             base = g._base if g._base is not None else g
-            if base.data_ptr() not in done:
+            if base.data_ptr() not in done and not self._lazy.get(id(p)):
                 out.append(self.kernels.axpby(g, factor, None, 0.0, g, g.numel()))
         return out
 
@@ -205,10 +213,43 @@ class ParamStore:
             self._keep.append(tensor)
         return sh
 
-    def grad(self, param):
+    def _lazy_alloc(self, shape, device):
+        n = 1
+        for d in shape:
+            n *= int(d)
+        pad = (n + 63) // 64 * 64
+        if n >= self.arena_block // 4:
+            return torch.zeros(shape, dtype=torch.float32, device=device)
+        if self._lazy_block is None or self._lazy_used + pad > self._lazy_block.numel():
+            self._lazy_block = torch.zeros(self.arena_block, dtype=torch.float32, device=device)
+            self._lazy_used = 0
+        t = self._lazy_block[self._lazy_used:self._lazy_used + n].view(shape)
+        self._lazy_used += pad
+        return t
+
+    def demote(self, param):
+        """The gradient of `param` has (or may have) a writer besides its one storing product: from now
+        on it is zeroed at the start of a step and swept by the unscale pass like any other."""
+        if self._lazy.get(id(param)):
+            self._lazy[id(param)] = False
+            g = self._grads[id(param)]
+            self.zero.append(self.kernels.fill(g, 0.0, g.numel()))
+            self.demoted.append(g)
+
+    def stored_whole(self, param):
+        return bool(self._lazy.get(id(param))) and len(self.deferred_sites.get(id(param), ())) == 1
+
+    def grad(self, param, deferred_site=None):
+        """fp32 gradient accumulator of `param` (== param.grad).  deferred_site: (stage, node name) of
+        a once-per-step weight-gradient product that asks for it; any other caller accumulates."""
         g = self._grads.get(id(param))
+        if deferred_site is not None:
+            self.deferred_sites.setdefault(id(param), set()).add(deferred_site)
         if g is None:
-            if param.grad is None or param.grad.dtype != torch.float32 or not param.grad.is_contiguous():
+            if deferred_site is not None and param.grad is None and param.dim() == 2:
+                param.grad = g = self._lazy_alloc(param.shape, param.device)
+                self._lazy[id(param)] = True
+            elif param.grad is None or param.grad.dtype != torch.float32 or not param.grad.is_contiguous():
                 param.grad = self._arena_alloc(param.shape, param.device)
                 g = param.grad
             else:
@@ -216,9 +257,12 @@ class ParamStore:
                 self.zero.append(self.kernels.fill(g, 0.0, g.numel()))
             self._grads[id(param)] = g
             self.params.append(param)
-        elif param.grad is not g:
-            # user code replaced .grad (e.g. zero_grad(set_to_none=True)); programs hold raw pointers
-            param.grad = g
+        else:
+            if deferred_site is None:
+                self.demote(param)
+            if param.grad is not g:
+                # user code replaced .grad (e.g. zero_grad(set_to_none=True)); programs hold raw pointers
+                param.grad = g
         return g
 
     def rebind_grads(self):
@@ -401,7 +445,7 @@ class BwdCtx:
             self._offer_big(launch, [(launch, grad)])
             return
         held = sum(t for _, _, t in self._dw)
-        if self._dw and (self._dw[0][0].variant != launch.variant or held + tiles > self.FULL_GRID
+        if self._dw and (self._dw[0][0].group_key != launch.group_key or held + tiles > self.FULL_GRID
                          or len(self._dw) == self.k.GEMM_GROUP_MAX):
             self.flush_dw()
             held = 0
@@ -436,7 +480,7 @@ class BwdCtx:
         mine = None
         for entries in self._dw_big:
             held = sum(t for _, _, _, t in entries)
-            if entries[0][1][0].variant == bigs[0].variant and held + t256 <= self.FULL_GRID \
+            if entries[0][1][0].group_key == bigs[0].group_key and held + t256 <= self.FULL_GRID \
                     and sum(len(b) for _, b, _, _ in entries) + len(bigs) <= self.k.GEMM_GROUP_MAX \
                     and (mine is None or held > sum(t for _, _, _, t in mine)):
                 mine = entries
@@ -692,6 +736,9 @@ class Lowerer:
         # the gradients those products read are then laid end to end across micro-batches
         self.stack_mbs = 1
         self.stack_tag = None   # micro-batch slots lowered under the same tag (input shapes) share stacked allocations
+        # loss scaling as the once-per-step weight-gradient products see it: (device scale or None,
+        # device overflow flag or None, constant factor); set by the worker
+        self.dw_unscale = (None, None, 1.0)
 
     # -- buffers -------------------------------------------------------------
     def alloc(self, shape, dtype):
@@ -826,16 +873,38 @@ class Lowerer:
                 n = len(recs)
                 dy = torch.as_strided(r0["dy"], (n * r0["rows"], r0["n_out"]), (r0["ld_dy"], 1))
                 x = torch.as_strided(r0["x"], (n * r0["rows"], r0["n_in"]), (r0["ld_x"], 1))
-                B.emit_dw(self.kernels.gemm(dy, x, r0["wg"], M=r0["n_out"], N=r0["n_in"], K=n * r0["rows"],
-                                            lda=r0["ld_dy"], ldb=r0["ld_x"], ldc=r0["n_in"], a_trans=1, b_trans=1,
-                                            beta=1), r0["wg"])
+                products = [(dy, x, n * r0["rows"])]
             else:
-                for r in recs:
-                    if r["rows"] == 0:
-                        continue
-                    B.emit_dw(self.kernels.gemm(r["dy"], r["x"], r["wg"], M=r["n_out"], N=r["n_in"], K=r["rows"],
-                                                lda=r["ld_dy"], ldb=r["ld_x"], ldc=r["n_in"], a_trans=1, b_trans=1,
-                                                beta=1), r["wg"])
+                products = [(r["dy"], r["x"], r["rows"]) for r in recs if r["rows"] > 0]
+            # A gradient that nothing else writes is STORED by its (first) product, unscaled and
+            # checked for overflow in that product's epilogue: no zero fill, no read of the old
+            # value, no unscale pass over it.  Anything else accumulates as every gradient does.
+            direct = getattr(self.kernels, "gemm_stores_checked", None)
+            whole = direct is not None and len(groups) > 0 and self.params.stored_whole(r0["param"])
+            scale, flag, factor = self.dw_unscale
+            launches = []
+            for i, (dy, x, rows) in enumerate(products):
+                kw = dict(M=r0["n_out"], N=r0["n_in"], K=rows, lda=r0["ld_dy"], ldb=r0["ld_x"], ldc=r0["n_in"],
+                          a_trans=1, b_trans=1)
+                if whole:
+                    launch = self.kernels.gemm(dy, x, r0["wg"], beta=int(i > 0), alpha=factor, unscale_by=scale,
+                                               nonfinite_flag=flag, **kw)
+                    if not direct(launch):     # this product runs on a kernel without that epilogue
+                        whole = False
+                        launches = []
+                        break
+                else:
+                    launch = self.kernels.gemm(dy, x, r0["wg"], beta=1, **kw)
+                launches.append(launch)
+            if not launches:
+                self.params.demote(r0["param"])
+                launches = [self.kernels.gemm(dy, x, r0["wg"], beta=1, M=r0["n_out"], N=r0["n_in"], K=rows,
+                                              lda=r0["ld_dy"], ldb=r0["ld_x"], ldc=r0["n_in"], a_trans=1, b_trans=1)
+                            for dy, x, rows in products]
+            elif not whole:
+                self.params.demote(r0["param"])
+            for launch in launches:
+                B.emit_dw(launch, r0["wg"])
         B.close_dw()
         B.compact([])
         return job.bwd
@@ -1011,12 +1080,12 @@ def lower_linear(L, node):
         if w.req_grad and w.param is not None:
             # dW = dY^T X reduces over the token rows, the strided dimension of both operands: the
             # GEMM reads them with transposing LDS reads (no transposed copies in memory)
-            wg = L.params.grad(w.param)
+            wg = L.params.grad(w.param, (B.program.stage, node.name) if defer_dw else None)
             if defer_dw:
                 # left to the stage's once-per-step job: over all micro-batches the operands form one
                 # product with that many times the reduction length, and one pass over the accumulator
-                B.program.dw_deferred.append(dict(name=node.name, dy=dy, x=xm, wg=wg, rows=M, n_out=N, n_in=K,
-                                                  ld_dy=ld_dy, ld_x=lda))
+                B.program.dw_deferred.append(dict(name=node.name, dy=dy, x=xm, wg=wg, param=w.param, rows=M, n_out=N,
+                                                  n_in=K, ld_dy=ld_dy, ld_x=lda))
             else:
                 B.emit_dw(B.k.gemm(dy, xm, wg, M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1, b_trans=1, beta=1), wg)
         if b is not None and b.req_grad and b.param is not None:

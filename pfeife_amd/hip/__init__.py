@@ -58,7 +58,7 @@ class GemmDesc(Structure):
         ("aux_in", c_void_p), ("ld_aux_in", c_int64),
         ("residual", c_void_p), ("ld_res", c_int64),
         ("res_dtype", c_int32), ("variant", c_int32),
-        ("colsum_ws", c_void_p),
+        ("colsum_ws", c_void_p), ("unscale_by", c_void_p), ("nonfinite_flag", c_void_p),
     ]
 
 
@@ -278,7 +278,7 @@ class HipKernels:
     # -- dense contractions ----------------------------------------------------
     def gemm(self, a, b, c, M, N, K, lda, ldb, ldc, a_trans=0, b_trans=0, batch=(1, 1), sa=(0, 0), sb=(0, 0),
              sc=(0, 0), alpha=1.0, beta=0, bias=None, round_mid=0, aux_out=None, ld_aux_out=0, act=0, dact=0,
-             aux_in=None, ld_aux_in=0, residual=None, ld_res=0, variant=0):
+             aux_in=None, ld_aux_in=0, residual=None, ld_res=0, variant=0, unscale_by=None, nonfinite_flag=None):
         if a.dtype != b.dtype:
             raise RuntimeError("gemm: operand dtypes differ (%s, %s)" % (a.dtype, b.dtype))
         d = GemmDesc()
@@ -297,13 +297,18 @@ class HipKernels:
         d.aux_in, d.ld_aux_in = _ptr(aux_in), ld_aux_in
         d.residual, d.ld_res, d.res_dtype = _ptr(residual), ld_res, _dt(residual)
         d.variant = int(variant)
+        d.unscale_by, d.nonfinite_flag = _ptr(unscale_by), _ptr(nonfinite_flag)
+        for t in (unscale_by, nonfinite_flag):
+            if t is not None and t.dtype != torch.float32:
+                raise RuntimeError("gemm: unscale_by / nonfinite_flag are fp32 device scalars")
         for t in (aux_out, aux_in):
             if t is not None and t.dtype != a.dtype:
                 raise RuntimeError("gemm: aux tensors must have the operand dtype")
-        launch = self._prep("pf_gemm", (byref(d),), (d, a, b, c, bias, aux_out, aux_in, residual))
+        launch = self._prep("pf_gemm", (byref(d),), (d, a, b, c, bias, aux_out, aux_in, residual, unscale_by, nonfinite_flag))
         name = ctypes.create_string_buffer(128)
         self.lib.pf_gemm_variant(byref(d), name, 128)
         launch.variant = name.value.decode()
+        launch.group_key = self._group_key(launch.variant)
         launch.flops = 2.0 * M * N * K * batch[0] * batch[1]
         launch.desc = d
         return launch
@@ -338,6 +343,7 @@ class HipKernels:
             return None
         new = self._prep("pf_gemm", (byref(d),), (d, launch))
         new.variant = name.value.decode()
+        new.group_key = self._group_key(new.variant)
         new.flops = launch.flops
         new.desc = d
         return new
@@ -345,23 +351,38 @@ class HipKernels:
     GEMM_GROUP_MAX = 8      # PF_GEMM_GROUP_MAX
 
     @staticmethod
+    def _group_key(variant):
+        """Weight-gradient products that store (class 1) and that accumulate (class 4) share the
+        accumulate launch of their tile: one key for both."""
+        if variant.startswith("gemm16x_kernel<") and variant.endswith("true, true, 1>"):
+            return variant[:-3] + " 4>"
+        return variant
+
+    @staticmethod
     def gemm_groupable(launch):
-        """A weight-gradient product on the direct-to-LDS kernel (fp32 C accumulated): launches of
-        this kind with the same `variant` may share one launch (pf_gemm_grouped)."""
-        v = getattr(launch, "variant", "")
+        """A weight-gradient product on the direct-to-LDS kernel (fp32 C stored or accumulated):
+        launches of this kind with the same `group_key` may share one launch (pf_gemm_grouped)."""
+        v = getattr(launch, "group_key", "")
         return v.startswith("gemm16x_kernel<") and v.endswith("true, true, 4>")
+
+    @staticmethod
+    def gemm_stores_checked(launch):
+        """Does this product run on a kernel whose epilogue honours `nonfinite_flag` (the fp32 classes
+        of the direct-to-LDS kernel)?"""
+        return HipKernels.gemm_groupable(launch)
 
     def gemm_group(self, launches):
         """One launch for 2..GEMM_GROUP_MAX independent `gemm_groupable` products of the same variant."""
         n = len(launches)
-        if not (2 <= n <= self.GEMM_GROUP_MAX) or len({l.variant for l in launches}) != 1 \
+        if not (2 <= n <= self.GEMM_GROUP_MAX) or len({l.group_key for l in launches}) != 1 \
                 or not all(self.gemm_groupable(l) for l in launches):
             raise RuntimeError("gemm_group: needs 2..%d groupable launches of one variant" % self.GEMM_GROUP_MAX)
         arr = (GemmDesc * n)()
         for i, l in enumerate(launches):
             ctypes.memmove(ctypes.byref(arr[i]), ctypes.byref(l.desc), ctypes.sizeof(GemmDesc))
         launch = self._prep("pf_gemm_grouped", (arr, n), (arr, launches))
-        launch.variant = launches[0].variant.replace("gemm16x_kernel<", "gemm16x_group_kernel<")
+        launch.variant = launches[0].group_key.replace("gemm16x_kernel<", "gemm16x_group_kernel<")
+        launch.group_key = launch.variant
         launch.flops = sum(l.flops for l in launches)
         launch.members = list(launches)
         return launch

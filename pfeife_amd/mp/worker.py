@@ -239,6 +239,10 @@ class StageWorker:
             graph_vals[i] = v
         L = self.lowerer
         L.stack_mbs = self.option.batch_cnt if (self.stack_dw and self.uniform_mbs) else 1
+        if self.dyn_scale:     # gradients stored whole by a once-per-step product leave it unscaled and checked
+            L.dw_unscale = (self.scaler_state[0:1], self.scaler_state[2:3], 1.0)
+        else:
+            L.dw_unscale = (None, None, 1.0 / float(self.option.loss_scale))
         L.stack_tag = slot.input_sig
         stage_out = {}
         for sid in sorted(pg.nodes):

@@ -432,9 +432,16 @@ def test_weight_gradients_run_once_per_step_over_all_micro_batches(monkeypatch):
     stacked buffers), issued after the stage's last backward job.  A ragged batch and PFEIFE_DW_STACK=0
     keep one product per micro-batch inside the backward jobs.  All three
     give the gradients of plain accumulation (checked by the callers' own comparisons above)."""
-    model, ref, out, (x, y), runner, crit = run_case(None)            # 8 samples in 4 micro-batches, 2 stages
+    model, ref, out, (x, y), runner, crit = run_case(None, steps=2)   # 8 samples in 4 micro-batches, 2 stages
     w = runner.worker
     assert sorted(w.dw_jobs) == [0, 1] and w.last_backward == {0: 3, 1: 3}
+    # the linear layers' weight gradients are STORED by their one product (no zero fill, no unscale pass
+    # over them: the second step above must not add to the first), every other gradient accumulates
+    whole = [n for n, p in model.named_parameters() if w.params.stored_whole(p)]
+    assert len(whole) == 8 + 9 and all(n.endswith("weight") for n in whole), whole
+    swept = sum(n for _, n in w.params.grad_buffers())               # what the unscale pass walks (padded to 64)
+    rest = sum(p.numel() for n, p in model.named_parameters() if n not in whole)
+    assert rest <= swept < rest + 64 * len(list(model.parameters()))
     tokens = (CFG.image_size // CFG.patch_size) ** 2 + 1
     per_stage = {sid: len(w.mbs[0].stage_programs[sid].dw_deferred) for sid in (0, 1)}
     assert per_stage[0] >= 8 and per_stage[1] >= 8                    # four linear layers per block, two blocks each

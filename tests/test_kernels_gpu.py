@@ -981,3 +981,57 @@ def test_mfma_rate_probe_multiplies_what_it_is_given(hip, dtype):
     per_k = frags.double().reshape(8, 2, 32, 8).sum(2).reshape(8, 16)     # [fragment][k]: sum over its 32 rows / columns
     want = iters * float((per_k[:4].sum(0) * per_k[4:].sum(0)).sum())
     assert sink.cpu().double().reshape(4 * wgs, 64).sum(1).tolist() == [want] * (4 * wgs)
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+def test_weight_gradient_product_unscales_checks_and_stores_inside_a_group(hip, oracle, dtype):
+    """A weight-gradient product can divide by a loss scale kept on the device (`unscale_by`), raise
+    an overflow flag when it writes a non-finite value (`nonfinite_flag`), and STORE its result
+    (beta = 0) as a member of a grouped launch whose other members accumulate.  Against the oracle:
+    three products of ragged sizes in one launch (store, accumulate, store), then the same launch
+    replayed with an inf planted in one operand: the flag goes up, and stays down without it."""
+    rows = 520
+    shapes = [(264, 392), (520, 136), (136, 264)]
+    scale = torch.tensor([1024.0], device="cuda")
+    flag = torch.zeros(1, device="cuda")
+    devs, cpus, launches = [], [], []
+    for i, (m, n) in enumerate(shapes):
+        dy, x = rnd((rows, m), dtype, 10 + i), rnd((rows, n), dtype, 20 + i, 0.1)
+        c0 = rnd((m, n), F32, 30 + i)
+        beta = int(i == 1)
+        dev = dict(a=dy.cuda(), b=x.cuda(), c=c0.clone().cuda())
+        kw = dict(M=m, N=n, K=rows, lda=m, ldb=n, ldc=n, a_trans=1, b_trans=1, beta=beta, variant=8)
+        launch = hip.gemm(**dev, unscale_by=scale, nonfinite_flag=flag, **kw)
+        assert launch.variant.endswith("true, true, %d>" % (4 if beta else 1)) and hip.gemm_stores_checked(launch)
+        kw.pop("variant")
+        cpu = dict(a=dy, b=x, c=c0.clone())
+        oracle.gemm(**cpu, unscale_by=scale.cpu(), **kw)()
+        devs.append(dev)
+        cpus.append(cpu)
+        launches.append(launch)
+    group = hip.gemm_group(launches)
+    assert group.variant.startswith("gemm16x_group_kernel<") and group.variant.endswith("true, true, 4>")
+    group(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for dev, cpu in zip(devs, cpus):
+        close((dev["c"].cpu(), cpu["c"]), 1e-3, 1e-4)
+    assert float(flag) == 0.0
+    # each on its own as well (the store class and the accumulate class of the plain kernel)
+    for dev, cpu, launch in zip(devs, cpus, launches):
+        if launch.desc.beta:
+            continue
+        dev["c"].fill_(7.0)
+        launch(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        close((dev["c"].cpu(), cpu["c"]), 1e-3, 1e-4)
+    assert float(flag) == 0.0
+    devs[2]["a"][3, 5] = float("inf")
+    group(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert float(flag) == 1.0 and not bool(torch.isfinite(devs[2]["c"]).all())
+    # kernels without that epilogue refuse the flag loudly (here: operands stored differently)
+    a, b = rnd((64, 96), dtype, 1).cuda(), rnd((96, 80), dtype, 2).cuda()
+    bad = hip.gemm(a, b, torch.zeros(64, 80, device="cuda"), M=64, N=80, K=96, lda=96, ldb=80, ldc=80, b_trans=1,
+                   nonfinite_flag=flag)
+    with pytest.raises(RuntimeError, match="nonfinite_flag"):
+        bad(torch.cuda.current_stream().cuda_stream)
