@@ -546,7 +546,7 @@ def model_flops_per_step(info):
     return 3.0 * samples * T * per_tok
 
 
-def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
+def run_workload(name, steps, warmup, device, roofline=True, hbm=True, ceiling=True):
     """Builds the workload, runs warm-up + `steps` timed steps, then the per-kernel replays."""
     import torch
 
@@ -607,7 +607,7 @@ def run_workload(name, steps, warmup, device, roofline=True, hbm=True):
                100 * r["frac"], PEAK_HBM_GBS, "" if r["on_path"] else "  [off-path micro-benchmark]",
                "" if "frac_of_copy" not in r else "  copy of the same bytes: %.1f us (kernel at %.0f%% of it)"
                % (r["copy_same_bytes_us"], 100 * r["frac_of_copy"])))
-    ceiling = gemm_ceiling(w.kernels, info["mixed"]) if (roofline and hbm) else None
+    ceiling = gemm_ceiling(w.kernels, info["mixed"]) if (roofline and hbm and ceiling) else None
     for r in ceiling or []:
         log("[bench] gemm ceiling [off-path] %-52s %8.1f us/launch %7.1f TFLOP/s (%.0f%% of peak)  %s"
             % (r["shape"], r["avg_launch_us"], r["tflops"], 100 * r["frac"], r["kernel"]))
@@ -650,6 +650,8 @@ def main():
     ap.add_argument("--workload", default="vit_l16_fp16", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-roofline", action="store_true")
+    ap.add_argument("--no-gemm-ceiling", action="store_true",
+                    help="skip the off-path gemm_ceiling record (profiles of the step's own kernels)")
     ap.add_argument("--no-eager-baseline", action="store_true",
                     help="skip timing the same step in plain PyTorch eager on this GPU")
     ap.add_argument("--no-others", action="store_true",
@@ -681,7 +683,7 @@ def main():
         os.environ["PFEIFE_NO_GRAPH"] = "1"
     t_start = time.perf_counter()
     runner, head = run_workload(args.workload, args.steps, args.warmup, device, roofline=not args.no_roofline,
-                                hbm=not args.no_roofline)
+                                hbm=not args.no_roofline, ceiling=not args.no_gemm_ceiling)
     if args.calibrate_copy:
         n = 64 * 1024 * 1024
         src = torch.ones(n, device=device)
