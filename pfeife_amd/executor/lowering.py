@@ -405,7 +405,7 @@ class BwdCtx:
         end to end across micro-batches: buffers of those sizes come from stacked allocations
         (per stage and position in the job), not from the set every job of a lane shares."""
         sigs = self.program.dw_sigs
-        if not sigs or self.L.stack_mbs <= 1:
+        if not sigs or not self.L.defer_dw:
             return None
         n = 1
         for d in shape:
@@ -731,9 +731,10 @@ class Lowerer:
         self.params = params or ParamStore(kernels, self.device)
         self.pool = pool or BufferPool(self.device)
         self._ws = None
-        # > 1: weight-gradient products of linear layers are left out of the backward jobs and run once
-        # per step over all `stack_mbs` micro-batches (the worker builds that job); forward buffers and
-        # the gradients those products read are then laid end to end across micro-batches
+        # defer_dw: weight-gradient products of linear layers are left out of the backward jobs and run
+        # once per step over all `stack_mbs` micro-batches (the worker builds that job); forward buffers
+        # and the gradients those products read are then laid end to end across micro-batches
+        self.defer_dw = False
         self.stack_mbs = 1
         self.stack_tag = None   # micro-batch slots lowered under the same tag (input shapes) share stacked allocations
         # loss scaling as the once-per-step weight-gradient products see it: (device scale or None,
@@ -742,7 +743,7 @@ class Lowerer:
 
     # -- buffers -------------------------------------------------------------
     def alloc(self, shape, dtype):
-        if self.stack_mbs > 1:
+        if self.defer_dw:
             self.cur.alloc_seq += 1
             t = self.pool.stacked((self.stack_tag, "f", self.cur.stage, self.cur.alloc_seq), shape, dtype, self.cur.mb,
                                   self.stack_mbs)
@@ -1047,7 +1048,7 @@ def lower_linear(L, node):
     if res is not None:
         kw.update(residual=res.buf, ld_res=as_matrix(res.buf)[2])
     L.emit(L.kernels.gemm(xm, w_cd, out, **kw))
-    defer_dw = L.stack_mbs > 1 and w.req_grad and w.param is not None
+    defer_dw = L.defer_dw and w.req_grad and w.param is not None
     if defer_dw:
         L.cur.dw_sigs.add((M * N, cd))
     req = x.req_grad or w.req_grad or (b is not None and b.req_grad) or (res is not None and res.req_grad)

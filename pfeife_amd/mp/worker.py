@@ -91,7 +91,7 @@ class StageWorker:
         # (PFEIFE_DW_STACK=0: inside every backward job, as torch.autograd issues them); decided per
         # micro-batch slot when it is lowered: only steps whose micro-batches all have the same
         # shapes stack their buffers (`uniform_mbs`, set by the runner before the step's first job)
-        self.stack_dw = self.option.batch_cnt > 1 and os.environ.get("PFEIFE_DW_STACK", "1") != "0"
+        self.stack_dw = os.environ.get("PFEIFE_DW_STACK", "1") != "0"
         self.uniform_mbs = getattr(self, "uniform_mbs", True)
         return Lowerer(self.kernels, self.device, self.option.mixed_precision, self.params, self.pool)
 
@@ -238,7 +238,8 @@ class StageWorker:
         for i, v in pg.static_vals.items():
             graph_vals[i] = v
         L = self.lowerer
-        L.stack_mbs = self.option.batch_cnt if (self.stack_dw and self.uniform_mbs) else 1
+        L.defer_dw = self.stack_dw and self.uniform_mbs
+        L.stack_mbs = self.option.batch_cnt
         if self.dyn_scale:     # gradients stored whole by a once-per-step product leave it unscaled and checked
             L.dw_unscale = (self.scaler_state[0:1], self.scaler_state[2:3], 1.0)
         else:
@@ -281,7 +282,7 @@ class StageWorker:
                 v = stage_out[ref[0]][ref[1]]
                 slot.outputs.append(v)
                 if isinstance(v, Val) and v.req_grad:
-                    if L.stack_mbs > 1 and v.buf.is_contiguous():
+                    if L.defer_dw and v.buf.is_contiguous():
                         # (the last layer's weight gradient reads these across micro-batches as one matrix)
                         slot.loss_grads[oi] = self.pool.stacked((L.stack_tag, "loss", oi), v.buf.shape, v.buf.dtype, mb,
                                                                 L.stack_mbs).zero_()
