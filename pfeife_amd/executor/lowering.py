@@ -540,14 +540,26 @@ class BwdCtx:
             for key in [k for k, v in self._lp.items() if v[0] == st]:
                 del self._lp[key]
 
-    def colsum_into(self, x, rows, cols, ld, acc):
-        """acc[c] += sum_r x[r, c] (bias gradient), reduction finished at the end of the job."""
+    def colsum_from_producer(self, x, rows, cols, ld, acc):
+        """The kernel that produced x may already have summed its columns (partial rows on the side):
+        then acc[c] += those, finished with the job's other reductions.  -> whether that was so."""
         for _, copy, cs in self._lp.values():
             if cs is not None and copy.data_ptr() == x.data_ptr() and copy.numel() == rows * cols and ld == cols:
-                ws, off, nb, stride = cs     # the kernel that produced x already summed its columns
+                ws, off, nb, stride = cs
                 self.reduces.append((ws, off, nb, stride, cols, acc))
-                return
+                return True
+        return False
+
+    def colsum_into(self, x, rows, cols, ld, acc, at_once=False):
+        """acc[c] += sum_r x[r, c] (bias gradient), reduction finished at the end of the job (the
+        batched finish adds every accumulator from one workgroup column: an accumulator may appear
+        in it ONCE; at_once: finish here instead, for a second sum into the same accumulator)."""
+        if self.colsum_from_producer(x, rows, cols, ld, acc):
+            return
         ws = self.temp((self.k.colreduce_workspace(rows, cols),), torch.float32)
+        if at_once:
+            self.emit(self.k.colsum_accumulate(x, rows, cols, ld, acc, ws, defer=0))
+            return
         self.emit(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
         self.reduces.append((ws, 0, self.k.colsum_partials(rows), cols, cols, acc))
 
@@ -906,7 +918,17 @@ class Lowerer:
                 self.params.demote(r0["param"])
             for launch in launches:
                 B.emit_dw(launch, r0["wg"])
+            # the layer's bias gradient: one column sum over all micro-batches' rows where they are
+            # stacked, else one per micro-batch (each finished on the spot: same accumulator)
+            if len(products) == 1 and all(r.get("bias_grad") is not None for r in recs):
+                B.colsum_into(products[0][0], products[0][2], r0["n_out"], r0["ld_dy"], r0["bias_grad"])
+            else:
+                for r in recs:
+                    if r.get("bias_grad") is not None and r["rows"] > 0:
+                        B.colsum_into(r["dy"], r["rows"], r["n_out"], r["ld_dy"], r["bias_grad"], at_once=True)
         B.close_dw()
+        if B.reduces:
+            job.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
         B.compact([])
         return job.bwd
 
@@ -1090,7 +1112,13 @@ def lower_linear(L, node):
             else:
                 B.emit_dw(B.k.gemm(dy, xm, wg, M=N, N=K, K=M, lda=ld_dy, ldb=lda, ldc=K, a_trans=1, b_trans=1, beta=1), wg)
         if b is not None and b.req_grad and b.param is not None:
-            B.colsum_into(dy, M, N, ld_dy, L.params.grad(b.param))
+            bg = L.params.grad(b.param)
+            if defer_dw and w.req_grad and w.param is not None:
+                # the bias gradient is the column sum of the same dy: with the weight gradient, once per step
+                if not B.colsum_from_producer(dy, M, N, ld_dy, bg):
+                    B.program.dw_deferred[-1]["bias_grad"] = bg
+            else:
+                B.colsum_into(dy, M, N, ld_dy, bg)
         if x.req_grad:
             dst, prev = B.grad_target(x)
             dm = as_matrix(dst)

@@ -228,23 +228,26 @@ class StageWorker:
         slot = MicroBatchPrograms()
         slot.input_sig = self._signature([dynamic_inputs[i] for i in sorted(dynamic_inputs)])
         graph_vals = {}
+        L = self.lowerer
+        L.defer_dw = self.stack_dw and self.uniform_mbs
+        L.stack_mbs = self.option.batch_cnt
+        L.stack_tag = slot.input_sig
         for i, v in dynamic_inputs.items():
             if torch.is_tensor(v):
-                buf = torch.empty(v.shape, dtype=v.dtype, device=self.device)
+                if L.defer_dw:   # (a layer that reads a graph input directly: its rows of all micro-batches in one matrix)
+                    buf = self.pool.stacked((L.stack_tag, "in", i), v.shape, v.dtype, mb, L.stack_mbs)
+                else:
+                    buf = torch.empty(v.shape, dtype=v.dtype, device=self.device)
                 slot.input_buffers[i] = buf
                 graph_vals[i] = Val(buf, req_grad=False, name=pg.placeholder_names[i])
             else:
                 graph_vals[i] = v
         for i, v in pg.static_vals.items():
             graph_vals[i] = v
-        L = self.lowerer
-        L.defer_dw = self.stack_dw and self.uniform_mbs
-        L.stack_mbs = self.option.batch_cnt
         if self.dyn_scale:     # gradients stored whole by a once-per-step product leave it unscaled and checked
             L.dw_unscale = (self.scaler_state[0:1], self.scaler_state[2:3], 1.0)
         else:
             L.dw_unscale = (None, None, 1.0 / float(self.option.loss_scale))
-        L.stack_tag = slot.input_sig
         stage_out = {}
         for sid in sorted(pg.nodes):
             st = pg.nodes[sid]
@@ -499,7 +502,13 @@ class StageWorker:
         job = self.dw_jobs.get(stage)
         if job is None:
             progs = [self.mbs[m].stage_programs[stage] for m in sorted(self.mbs)]
+            self.pool.lane = ("dw", stage)    # this job's temporaries are its own: jobs of two stages may overlap
             launches = self.lowerer.lower_deferred_dw(progs) if any(p.dw_deferred for p in progs) else []
+            self.pool.lane = 0
+            if self.stream_obj is not None:
+                # the job is about to run on its lane; what its lowering put on the device through
+                # torch's current stream (the table of the batched reduction) has to be there first
+                torch.cuda.current_stream(self.device).synchronize()
             job = self.dw_jobs[stage] = [launches, None]
         if job[1] is not None:
             job[1](stream)

@@ -446,7 +446,10 @@ def test_weight_gradients_run_once_per_step_over_all_micro_batches(monkeypatch):
     per_stage = {sid: len(w.mbs[0].stage_programs[sid].dw_deferred) for sid in (0, 1)}
     assert per_stage[0] >= 8 and per_stage[1] >= 8                    # four linear layers per block, two blocks each
     for sid, (launches, _) in w.dw_jobs.items():
-        assert len(launches) == per_stage[sid]                        # one launch per layer, not per micro-batch
+        kinds = [l.__qualname__.split(".")[1] for l in launches]
+        assert kinds.count("gemm") == per_stage[sid]                     # one product per layer, not per micro-batch
+        # ... and one column sum per layer for its bias, over the same stacked rows, finished together
+        assert kinds.count("colsum_accumulate") == per_stage[sid] and kinds.count("colreduce_finalize_batch") == 1
     # the block layers reduce over 4 micro-batches x 2 samples x tokens rows
     ks = sorted({int(r["rows"]) for r in w.mbs[0].stage_programs[0].dw_deferred})
     assert 2 * tokens in ks

@@ -177,11 +177,15 @@ def test_vit_l_width_fp16_headline_geometry():
     # the blocks' weight gradients: once per step, one product per layer over the 4 x 3152 token rows of
     # all micro-batches, several layers sharing a launch on 256x256 tiles
     for sid, (launches, graph) in runner.worker.dw_jobs.items():
-        members = [m for l in launches for m in getattr(l, "members", [l])]
+        gemms = [l for l in launches if getattr(l, "kernel", "") in ("pf_gemm", "pf_gemm_grouped")]
+        members = [m for l in gemms for m in getattr(l, "members", [l])]
         assert len(members) == 2 * 4 + (sid == 1), (sid, len(members))         # 2 blocks x 4 layers (+ the head)
         assert sum(m.desc.K == 4 * 3152 for m in members) == 2 * 4
-        assert any(l.variant == "gemm16x_group_kernel<1, 256, 256, 32, 2, 4, 1, 5, true, true, 4>" for l in launches), \
-            [l.variant for l in launches]
+        assert any(l.variant == "gemm16x_group_kernel<1, 256, 256, 32, 2, 4, 1, 5, true, true, 4>" for l in gemms), \
+            [l.variant for l in gemms]
+        # the layers' bias gradients not already summed by a producing kernel: one column sum each over the
+        # same stacked rows, finished by one launch
+        assert sum(getattr(l, "kernel", "") == "pf_colreduce_finalize_batch" for l in launches) == 1
 
 
 def test_vit_l16_headline_config_trains_like_pytorch():
@@ -1408,7 +1412,8 @@ def test_weight_gradients_once_per_step_equal_the_per_micro_batch_sums(monkeypat
         assert sorted(w.dw_jobs) == [0, 1] and all(graph is not None for _, graph in w.dw_jobs.values())
         rows = 3 * (1 + (64 // 16) ** 2)                               # micro-batch 3 x 17 tokens
         for sid, (launches, _) in w.dw_jobs.items():
-            members = [m for l in launches for m in getattr(l, "members", [l])]
+            members = [m for l in launches if getattr(l, "kernel", "") in ("pf_gemm", "pf_gemm_grouped")
+                       for m in getattr(l, "members", [l])]
             assert len(members) == len(w.mbs[0].stage_programs[sid].dw_deferred)    # one product per layer
             assert sum(m.desc.K == 4 * rows for m in members) >= 8                  # 2 blocks x 4 layers over all rows
         for (la, ga), (lb, gb) in zip(per_mb, once):
