@@ -563,6 +563,21 @@ class BwdCtx:
         self.emit(self.k.colsum_accumulate(x, rows, cols, ld, None, ws, defer=1))
         self.reduces.append((ws, 0, self.k.colsum_partials(rows), cols, cols, acc))
 
+    def finish_reduces(self):
+        """Launches that finish the deferred column reductions.  One batched launch adds every listed
+        accumulator from its own workgroups, without atomics: an accumulator that was reduced into
+        twice (a parameter used by two layers of the job) goes into a later launch."""
+        out, rest = [], list(self.reduces)
+        while rest:
+            seen, now, later = set(), [], []
+            for item in rest:
+                key = item[5].data_ptr()
+                (later if key in seen else now).append(item)
+                seen.add(key)
+            out.append(self.k.colreduce_finalize_batch(now))
+            rest = later
+        return out
+
     def new_like(self, like, private=False):
         if like.is_contiguous():
             kept = self._kept_for_dw(like.shape, like.dtype)
@@ -832,8 +847,7 @@ class Lowerer:
             prog.bwd_ranges.append((name, first, len(prog.bwd)))
         first = len(prog.bwd)
         B.close_dw()
-        if B.reduces:
-            prog.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
+        prog.bwd.extend(B.finish_reduces())
         if prog.bwd_ranges and len(prog.bwd) > first:   # held-back tail: charged to the job's last node
             prog.bwd_ranges.append((prog.bwd_ranges[-1][0], first, len(prog.bwd)))
         B.compact(prog.bwd_ranges)
@@ -927,8 +941,7 @@ class Lowerer:
                     if r.get("bias_grad") is not None and r["rows"] > 0:
                         B.colsum_into(r["dy"], r["rows"], r["n_out"], r["ld_dy"], r["bias_grad"], at_once=True)
         B.close_dw()
-        if B.reduces:
-            job.bwd.append(self.kernels.colreduce_finalize_batch(B.reduces))
+        job.bwd.extend(B.finish_reduces())
         B.compact([])
         return job.bwd
 

@@ -310,6 +310,10 @@ class StageWorker:
             self.pool.lane = self._lane_key(sid, False) if self.lanes is not None else 0
             L.lower_backward(prog, out_grads)
         self.pool.lane = 0
+        if self.stream_obj is not None:
+            # tables the lowering copied to the device went through torch's current stream; the jobs
+            # that read them run on the lanes
+            torch.cuda.current_stream(self.device).synchronize()
         self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
         self._drop_dw_jobs()
         self.mbs[mb] = slot
