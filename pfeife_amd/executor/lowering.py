@@ -66,6 +66,7 @@ class ParamStore:
         self._lazy_used = 0
         self.deferred_sites = {}   # id(param) -> {(stage, node name)} of the deferred products that write it
         self.demoted = []          # gradients in such blocks that need the fill and the unscale after all
+        self.pending_fills = []    # zero fills of gradients demoted since the step's zero fill ran
 
     def shadow(self, tensor, dtype):
         if tensor.dtype == dtype:
@@ -233,7 +234,11 @@ class ParamStore:
         if self._lazy.get(id(param)):
             self._lazy[id(param)] = False
             g = self._grads[id(param)]
-            self.zero.append(self.kernels.fill(g, 0.0, g.numel()))
+            fill = self.kernels.fill(g, 0.0, g.numel())
+            self.zero.append(fill)
+            # this step's zero fill has already run without it, and the buffer may still hold the
+            # previous step's stored gradient: the worker runs these before anything accumulates
+            self.pending_fills.append(fill)
             self.demoted.append(g)
 
     def stored_whole(self, param):

@@ -310,9 +310,13 @@ class StageWorker:
             self.pool.lane = self._lane_key(sid, False) if self.lanes is not None else 0
             L.lower_backward(prog, out_grads)
         self.pool.lane = 0
+        # gradients that lost their single storing writer in this lowering: zero them now (their backward
+        # jobs, which accumulate, come later in the step)
+        self._run_pending_fills(self.stream())
         if self.stream_obj is not None:
             # tables the lowering copied to the device went through torch's current stream; the jobs
             # that read them run on the lanes
+            self.stream_obj.synchronize()
             torch.cuda.current_stream(self.device).synchronize()
         self._drop_graphs(self.mbs.get(mb))   # a slot rebuilt for another micro-batch shape
         self._drop_dw_jobs()
@@ -500,6 +504,11 @@ class StageWorker:
                     continue
                 self.kernels.fill(buf, self.option.loss_scale if buf.dim() == 0 else 0.0, buf.numel())(self.stream())
 
+    def _run_pending_fills(self, stream):
+        fills, self.params.pending_fills = self.params.pending_fills, []
+        for launch in fills:
+            launch(stream)
+
     def _run_dw_job(self, stage, stream):
         """The stage's weight-gradient products over all micro-batches of the step, after its last
         backward job and on that job's stream (built when every micro-batch slot exists)."""
@@ -514,6 +523,7 @@ class StageWorker:
                 # torch's current stream (the table of the batched reduction) has to be there first
                 torch.cuda.current_stream(self.device).synchronize()
             job = self.dw_jobs[stage] = [launches, None]
+            self._run_pending_fills(stream)    # (demoted while the job was lowered: only this job writes them)
         if job[1] is not None:
             job[1](stream)
         else:

@@ -468,3 +468,45 @@ def test_weight_gradients_run_once_per_step_over_all_micro_batches(monkeypatch):
     run_unpipelined(ref, crit, x, y, 4)
     for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
         assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+
+
+def test_ragged_step_after_uniform_steps_starts_from_zeroed_gradients():
+    """Uniform steps store the linear weights' gradients from one product per step (no zero fill over
+    them).  A later step whose micro-batches differ (7 samples over 3: 3, 2, 2) rebuilds only the slot
+    whose shape changed, without the deferral: from then on those gradients are accumulated again, and
+    the very step in which that happens must already start from zero, not from the previous step's
+    stored values."""
+    from pfeife_amd.mp import partial_compiler
+
+    torch.manual_seed(0)
+    model = VisionTransformer(CFG)
+    ref = copy.deepcopy(model)
+    option = PipeOption(device_cnt=1, batch_cnt=3, batch_size=2, split_points=None, optimizer=dict(type="sgd", lr=0.0))
+    runner = make_runner(option)
+    cmodel = torch.compile(model, backend=partial_compiler, dynamic=False)
+    crit = nn.CrossEntropyLoss()
+
+    def fn(x, y):
+        loss = crit(cmodel(x).float(), y)
+        loss.backward()
+        return loss.detach()
+
+    runner.set_exec_fn(fn)
+    g = torch.Generator().manual_seed(42)
+    x6, y6 = torch.randn(6, 3, 32, 32, generator=g), torch.randint(0, 10, (6,), generator=g)
+    x7, y7 = torch.randn(7, 3, 32, 32, generator=g), torch.randint(0, 10, (7,), generator=g)
+    runner.step(x6, y6)
+    runner.step(x6, y6)
+    w = runner.worker
+    assert any(w.params.stored_whole(p) for p in model.parameters())
+    runner.step(x7, y7)
+    assert not any(w.params.stored_whole(p) for p in model.parameters())
+    run_unpipelined(ref, crit, x7, y7, 3)
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
+    runner.step(x6, y6)          # and back: every slot has its uniform shape again
+    for q in ref.parameters():
+        q.grad = None
+    run_unpipelined(ref, crit, x6, y6, 3)
+    for (n, p), (_, q) in zip(model.named_parameters(), ref.named_parameters()):
+        assert (p.grad - q.grad).abs().max() <= 1e-4 * q.grad.abs().max() + 1e-9, n
