@@ -65,7 +65,6 @@ class ParamStore:
         self._lazy_block = None
         self._lazy_used = 0
         self.deferred_sites = {}   # id(param) -> {(stage, node name)} of the deferred products that write it
-        self.demoted = []          # gradients in such blocks that need the fill and the unscale after all
         self.pending_fills = []    # zero fills of gradients demoted since the step's zero fill ran
 
     def shadow(self, tensor, dtype):
@@ -239,7 +238,6 @@ class ParamStore:
             # this step's zero fill has already run without it, and the buffer may still hold the
             # previous step's stored gradient: the worker runs these before anything accumulates
             self.pending_fills.append(fill)
-            self.demoted.append(g)
 
     def stored_whole(self, param):
         return bool(self._lazy.get(id(param))) and len(self.deferred_sites.get(id(param), ())) == 1
@@ -888,6 +886,7 @@ class Lowerer:
             # programs lowered at different times (a slot rebuilt for another shape without the
             # deferral): every program's products on their own
             groups = [(r,) for recs in lists for r in recs]
+        stored = set()      # gradients this job has written so far: only the first product into one stores
         for recs in groups:
             r0 = recs[0]
             es = r0["dy"].element_size()
@@ -919,8 +918,8 @@ class Lowerer:
                 kw = dict(M=r0["n_out"], N=r0["n_in"], K=rows, lda=r0["ld_dy"], ldb=r0["ld_x"], ldc=r0["n_in"],
                           a_trans=1, b_trans=1)
                 if whole:
-                    launch = self.kernels.gemm(dy, x, r0["wg"], beta=int(i > 0), alpha=factor, unscale_by=scale,
-                                               nonfinite_flag=flag, **kw)
+                    launch = self.kernels.gemm(dy, x, r0["wg"], beta=int(i > 0 or id(r0["param"]) in stored),
+                                               alpha=factor, unscale_by=scale, nonfinite_flag=flag, **kw)
                     if not direct(launch):     # this product runs on a kernel without that epilogue
                         whole = False
                         launches = []
@@ -935,6 +934,7 @@ class Lowerer:
                             for dy, x, rows in products]
             elif not whole:
                 self.params.demote(r0["param"])
+            stored.add(id(r0["param"]))
             for launch in launches:
                 B.emit_dw(launch, r0["wg"])
             # the layer's bias gradient: one column sum over all micro-batches' rows where they are
