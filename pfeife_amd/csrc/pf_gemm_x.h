@@ -43,6 +43,12 @@ template <> struct Frag<true> {
   short4_t lo, hi;
   __device__ __forceinline__ short8_t get() const { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
 };
+// Keeps the registers of a fragment that inline assembly reads into allocated to it up to this
+// point of the program: the compiler takes the output of such a read for complete where the read
+// is issued, and once the value is dead it is free to put something else into the register, which
+// the read, arriving later, would then overwrite.
+__device__ __forceinline__ void frag_hold(Frag<false>&) {}
+__device__ __forceinline__ void frag_hold(Frag<true>& f) { asm volatile("" : "+v"(f.lo), "+v"(f.hi)); }
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -351,6 +357,20 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
     sb_prev = sb;
     sb = sb_next;
   }
+  // The last tile's last phase has read fragments of a tile that does not exist, and nothing
+  // consumes them: the reads issued by inline assembly may still be in flight here, and the
+  // compiler, which knows nothing of that, would hand their registers to the epilogue's first
+  // values (seen: the lane's row inside the block, overwritten with a fragment of zeros whenever
+  // other kernels on the same compute unit delayed the LDS: every lane then took itself for a
+  // lane of row 0 and 15 rows in 16 of the wavefront's block were never written).
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int sl = 0; sl < 2; ++sl) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) frag_hold(fa[sl][i]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) frag_hold(fb[sl][j]);
+  }
   // (the dropped requests past K are counted too)  The builtin, not inline assembly: the compiler
   // tracks the LDS-writing loads itself and, unless it sees them retired here, makes every LDS
   // read of the epilogue wait for ALL vector memory operations, i.e. for the epilogue's own
@@ -499,6 +519,13 @@ __device__ __forceinline__ void gemm16x_body(const pf_gemm_desc& p, const GemmGr
         }
       }
       asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      // (the values are only complete from here on: nothing that uses them may move above the wait)
+#pragma unroll
+      for (int pp = 0; pp < NP; ++pp) {
+        asm volatile("" : "+v"(sxs[pp]), "+v"(sys[pp]));
+        if constexpr (LOADS) asm volatile("" : "+v"(ras[pp]));
+        if constexpr (LOAD32) asm volatile("" : "+v"(rbs[pp]));
+      }
 #pragma unroll
       for (int pp = 0; pp < NP; ++pp) {
         const v4i_t sx = sxs[pp], sy = sys[pp], ra = ras[pp], rb = rbs[pp];

@@ -945,6 +945,54 @@ def test_lanes_give_bit_identical_steps(monkeypatch):
                     assert torch.equal(a, b), mode
 
 
+def test_lanes_give_bit_identical_per_micro_batch_weight_gradients(monkeypatch):
+    """The same, for weight gradients added up micro-batch by micro-batch (PFEIFE_DW_STACK=0, the
+    form steps with ragged micro-batches take) at ViT-S/16 size: those products run on the tile
+    whose two operands both go through the transposing LDS reads, next to the kernels of the
+    other streams on the same compute units, where a fragment read still in flight at the end
+    of the reduction loop once overwrote the epilogue's row index."""
+    from pfeife_amd.bench_models.vit import VIT_S16, VisionTransformer
+    from pfeife_amd.mp import partial_compiler
+    from pfeife_amd.option import PipeOption
+
+    monkeypatch.setenv("PFEIFE_DW_STACK", "0")
+
+    def run(mode):
+        monkeypatch.setenv("PFEIFE_LANES", mode)
+        torch.manual_seed(0)
+        model = VisionTransformer(VIT_S16)
+        g = torch.Generator().manual_seed(42)
+        x = torch.randn(16, 3, 224, 224, generator=g).cuda()
+        y = torch.randint(0, VIT_S16.num_classes, (16,), generator=g).cuda()
+        option = PipeOption(device_cnt=2, batch_cnt=4, batch_size=4, split_points=["blocks.6"],
+                            mixed_precision="fp16", optimizer=dict(type="sgd", lr=0.0))
+        runner = _fresh_runner(option)
+        model.cuda()
+        cmodel = torch.compile(model, backend=partial_compiler)
+        crit = nn.CrossEntropyLoss()
+
+        def fn(px, labels):
+            loss = crit(cmodel(px).float(), labels)
+            loss.backward()
+            return loss.detach()
+
+        runner.set_exec_fn(fn)
+        out = []
+        for _ in range(4):
+            losses = runner.step(x, y)
+            torch.cuda.synchronize()
+            out.append(([float(l) for l in losses], {n: p.grad.clone() for n, p in model.named_parameters()}))
+        return out
+
+    base = run("0")
+    for rep in range(3):
+        got = run("rankdir")
+        for step, ((l0, g0), (l1, g1)) in enumerate(zip(base, got)):
+            assert l0 == l1, (rep, step, l0, l1)
+            for n in g0:
+                assert torch.equal(g0[n], g1[n]), (rep, step, n)
+
+
 @pytest.mark.parametrize("mixed", [None, "bf16"])
 def test_vit_g_block_share_head_dim_88(mixed):
     """The ViT-g/14 block-share configuration at reduced depth: blocks (dim 1408, 16 heads of 88,
