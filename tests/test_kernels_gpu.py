@@ -983,6 +983,39 @@ def test_mfma_rate_probe_multiplies_what_it_is_given(hip, dtype):
     assert sink.cpu().double().reshape(4 * wgs, 64).sum(1).tolist() == [want] * (4 * wgs)
 
 
+@pytest.mark.parametrize("variant", [0, 7, 8, 9])
+def test_accumulating_products_stay_exact_next_to_other_streams(hip, variant):
+    """Weight-gradient products (both operands reduction-strided, fp32 accumulate) on one stream while
+    two other streams keep the compute units busy with other products.  Small integers make every
+    sum exact in fp32: after n launches the accumulator is n times the product, bit for bit, or a
+    launch lost, repeated or mixed up rows."""
+    torch.manual_seed(0)
+    M, N, K, reps = 1536, 384, 788, 12
+    dy = torch.randint(-2, 3, (K, M), device="cuda").to(F16)
+    x = torch.randint(-2, 3, (K, N), device="cuda").to(F16)
+    want = dy.float().t() @ x.float()
+    accs = [torch.zeros(M, N, device="cuda") for _ in range(6)]
+    launches = [hip.gemm(dy, x, c, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1, variant=variant)
+                for c in accs]
+    a2 = torch.randn(K, N, device="cuda").to(F16)
+    w2 = torch.randn(M, N, device="cuda").to(F16)
+    o2 = torch.empty(K, M, device="cuda", dtype=F16)
+    side_a = hip.gemm(a2, w2, o2, M=K, N=M, K=N, lda=N, ldb=N, ldc=M)
+    o3 = torch.zeros(M, N, device="cuda")
+    side_b = hip.gemm(dy, x, o3, M=M, N=N, K=K, lda=M, ldb=N, ldc=N, a_trans=1, b_trans=1, beta=1)
+    main, s1, s2 = torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(reps):
+        for launch in launches:
+            launch(main.cuda_stream)
+            side_a(s1.cuda_stream)
+            side_b(s2.cuda_stream)
+    torch.cuda.synchronize()
+    for c in accs:
+        assert torch.equal(c, reps * want)
+    assert torch.equal(o3, reps * len(accs) * want)
+
+
 @pytest.mark.parametrize("dtype", [F16, BF16])
 def test_weight_gradient_product_unscales_checks_and_stores_inside_a_group(hip, oracle, dtype):
     """A weight-gradient product can divide by a loss scale kept on the device (`unscale_by`), raise
