@@ -911,7 +911,7 @@ extern "C" int pf_gemm_variant(const pf_gemm_desc* desc, char* out, int cap) {
       // BM, BN, BK, wavefront rows, columns, reduction split, stages: as rocprofv3 prints the instantiation
       static const char* shapes[PF_XT_COUNT] = {"", "256, 256, 32, 2, 2, 1, 5", "256, 128, 64, 2, 2, 1, 3", "128, 128, 64, 2, 2, 1, 3",
                                                 "192, 256, 32, 2, 2, 1, 5", "128, 128, 64, 2, 2, 2, 3", "256, 128, 64, 2, 2, 2, 3",
-                                                "256, 256, 32, 2, 4, 1, 5", "128, 128, 64, 4, 2, 1, 3", "256, 128, 64, 4, 2, 1, 3"};
+                                                "256, 256, 32, 2, 4, 1, 5", "128, 128, 64, 2, 4, 1, 3", "256, 128, 64, 4, 2, 1, 3"};
       if (!x_supports(d, v)) {   // a pinned tile that cannot run this product: say so here, not at launch time
         pf_set_error("pf_gemm_variant: variant %d needs both operands stored alike, K >= %d and (unless both are "
                      "reduction-strided) K a multiple of %d", v, x_tile_bk(v), x_tile_bk(v));

@@ -195,7 +195,7 @@ template <> struct XTile<PF_XT_192x256> { static constexpr int BM = 192, BN = 25
 template <> struct XTile<PF_XT_128x128k2> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2, KS = 2; };
 template <> struct XTile<PF_XT_256x128k2> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 2, KS = 2; };
 template <> struct XTile<PF_XT_256x256w8> { static constexpr int BM = 256, BN = 256, BK = 32, ST = 5, WGM = 2, WGN = 4, KS = 1; };
-template <> struct XTile<PF_XT_128x128w8> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 4, WGN = 2, KS = 1; };
+template <> struct XTile<PF_XT_128x128w8> { static constexpr int BM = 128, BN = 128, BK = 64, ST = 3, WGM = 2, WGN = 4, KS = 1; };
 template <> struct XTile<PF_XT_256x128w8> { static constexpr int BM = 256, BN = 128, BK = 64, ST = 3, WGM = 4, WGN = 2, KS = 1; };
 inline int x_tile_bk(int xt) { return (xt == PF_XT_256x256 || xt == PF_XT_192x256 || xt == PF_XT_256x256w8) ? 32 : 64; }
 
