@@ -125,7 +125,7 @@ def test_gemm_epilogues(hip, oracle, dtype):
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 1, 5"), (2, "256, 128, 64, 2, 2, 1, 3"), (3, "128, 128, 64, 2, 2, 1, 3"),
                                           (4, "192, 256, 32, 2, 2, 1, 5"), (5, "128, 128, 64, 2, 2, 2, 3"), (6, "256, 128, 64, 2, 2, 2, 3"),
-                                          (7, "256, 256, 32, 2, 4, 1, 5"), (8, "128, 128, 64, 4, 2, 1, 3"), (9, "256, 128, 64, 4, 2, 1, 3")])
+                                          (7, "256, 256, 32, 2, 4, 1, 5"), (8, "128, 128, 64, 2, 4, 1, 3"), (9, "256, 128, 64, 4, 2, 1, 3")])
 def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
     """Every straight-line epilogue class of the direct-to-LDS kernel on every tile shape, ragged in M
     (and in N against the 256- and 192-wide tiles), against the oracle; the launch names the class."""
@@ -173,7 +173,7 @@ def test_gemm_direct_to_lds_epilogue_classes(hip, oracle, dtype, variant, tile):
 @pytest.mark.parametrize("dtype", [F16, BF16])
 @pytest.mark.parametrize("variant,tile", [(1, "256, 256, 32, 2, 2, 1, 5"), (2, "256, 128, 64, 2, 2, 1, 3"), (3, "128, 128, 64, 2, 2, 1, 3"),
                                           (5, "128, 128, 64, 2, 2, 2, 3"), (6, "256, 128, 64, 2, 2, 2, 3"), (7, "256, 256, 32, 2, 4, 1, 5"),
-                                          (8, "128, 128, 64, 4, 2, 1, 3"), (9, "256, 128, 64, 4, 2, 1, 3")])
+                                          (8, "128, 128, 64, 2, 4, 1, 3"), (9, "256, 128, 64, 4, 2, 1, 3")])
 def test_gemm_direct_to_lds_weight_gradient_tiles(hip, oracle, dtype, variant, tile):
     """The reduction-strided (weight-gradient) form of every tile that has one: dW += dY^T X with a
     ragged reduction length (not a multiple of any stage depth) and ragged M and N, fp32 accumulate

@@ -170,8 +170,8 @@ def test_vit_l_width_fp16_headline_geometry():
     names = _gemm_variants(runner)
     want = ["gemm16x_kernel<1, 256, 256, 32, 2, 4, 1, 5, false, false, 2>",    # fc1: GELU epilogue
             "gemm16x_kernel<1, 256, 256, 32, 2, 4, 1, 5, false, false, 5>",    # dX of fc2: GELU' epilogue
-            "gemm16x_kernel<1, 128, 128, 64, 4, 2, 1, 3, false, false, 3>",    # proj / fc2: fp32 residual epilogue
-            "gemm16x_kernel<1, 128, 128, 64, 4, 2, 1, 3, true, true, 4>"]      # weight gradients, accumulated
+            "gemm16x_kernel<1, 128, 128, 64, 2, 4, 1, 3, false, false, 3>",    # proj / fc2: fp32 residual epilogue
+            "gemm16x_kernel<1, 128, 128, 64, 2, 4, 1, 3, true, true, 4>"]      # weight gradients, accumulated
     for w in want:
         assert w in names, (w, sorted(names))
     # the blocks' weight gradients: once per step, one product per layer over the 4 x 3152 token rows of
